@@ -1,0 +1,2 @@
+from .batch import StepBatch, StepEntry
+from .runner import ModelRunner, load_model, resolve_dtype

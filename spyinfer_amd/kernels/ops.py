@@ -1,0 +1,352 @@
+"""The engine's operations, as checked calls into the HIP kernel library.
+
+Every function checks on the host that shapes, dtypes, devices and contiguity
+are what its kernel and grid assume before anything is launched, and raises
+otherwise.  There is no CPU implementation here: on a machine without the
+library or without a GPU every call raises.  Kernels run on torch's current
+HIP stream, so they order with torch's own work and can be captured in graphs.
+
+dtype rules: activations are float32 or bfloat16; the residual stream and
+logits are always float32; a weight may be float32 or bfloat16 independently of
+the activations (a tensor stored in 32-bit stays so).
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build as _build
+
+F32, BF16, I32 = 0, 1, 2
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+_impl = None          # object with the same functions; installed by tests that emulate the kernels
+_hip = None
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def install_test_double(impl) -> None:
+    """Route all operations to ``impl`` (None restores the HIP library).  For tests of the
+    engine's logic on machines without a GPU; never used by the engine itself."""
+    global _impl
+    _impl = impl
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    if t.dtype not in _CODES:
+        raise KernelError("%s has dtype %s; float32 or bfloat16 expected" % (what, t.dtype))
+    return _CODES[t.dtype]
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*tensors) -> None:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        _check(t.is_cuda, "a kernel operand lies on %s; the kernels run on the GPU only" % t.device)
+        _check(t.is_contiguous(), "a kernel operand is not contiguous")
+        dev = dev or t.device
+        _check(t.device == dev, "kernel operands lie on different devices")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+class _Hip:
+    """ctypes view of the library; one instance per process."""
+
+    def __init__(self):
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: spyinfer_amd runs on an AMD GPU (gfx950) only")
+        self.lib = _build.load()
+        self.lib.spy_last_error.restype = ctypes.c_char_p
+        for name in ("spy_embedding", "spy_add_rmsnorm", "spy_rmsnorm", "spy_gemm", "spy_qknorm_rope_store",
+                     "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_swiglu",
+                     "spy_sample", "spy_gemm_skinny"):
+            getattr(self.lib, name).restype = ctypes.c_int64 if name.endswith("_workspace") else ctypes.c_int
+
+    def call(self, name, *args):
+        rc = getattr(self.lib, name)(*args)
+        if rc != 0:
+            raise KernelError("%s: %s" % (name, self.lib.spy_last_error().decode()))
+
+    @staticmethod
+    def stream():
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def hip() -> _Hip:
+    global _hip
+    if _hip is None:
+        _hip = _Hip()
+    return _hip
+
+
+def library_path() -> str:
+    return hip().lib._name
+
+
+# --------------------------------------------------------------------------
+def embedding(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """out[t, :] = table[ids[t], :] widened to float32 (the start of the residual stream)."""
+    if _impl is not None:
+        return _impl.embedding(ids, table)
+    _dev(ids, table)
+    _check(ids.dtype == torch.int32 and ids.dim() == 1, "embedding: ids must be int32 [T]")
+    _check(table.dim() == 2, "embedding: table must be [V, H]")
+    T, (V, H) = ids.shape[0], table.shape
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    if T:
+        hip().call("spy_embedding", _ptr(out), _ptr(table), _code(table, "embedding table"), _ptr(ids),
+                   ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(V), _Hip.stream())
+    return out
+
+
+def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """resid += delta (float32, in place; skipped if delta is None), then RMS-normalise.
+
+    Without ``rows``: every row is updated and normalised -> [T, H].  With ``rows``
+    (int32 [R]): only those rows are summed and normalised -> [R, H]; resid is left as it is."""
+    if _impl is not None:
+        return _impl.add_rms_norm(resid, delta, weight, eps, out_dtype, rows)
+    _dev(resid, delta, weight, rows)
+    _check(resid.dtype == torch.float32 and resid.dim() == 2, "add_rms_norm: the residual stream must be float32 [T, H]")
+    T, H = resid.shape
+    _check(weight.shape == (H,), "add_rms_norm: weight must be [H]")
+    if delta is not None:
+        _check(delta.shape == (T, H) and delta.dtype == out_dtype, "add_rms_norm: delta must be [T, H] of the activation dtype")
+    if rows is not None:
+        _check(rows.dtype == torch.int32 and rows.dim() == 1, "add_rms_norm: rows must be int32 [R]")
+    n_out = T if rows is None else rows.shape[0]
+    out = torch.empty((n_out, H), dtype=out_dtype, device=resid.device)
+    if n_out:
+        hip().call("spy_add_rmsnorm", _ptr(resid), _ptr(delta), _ptr(weight), _code(weight, "norm weight"),
+                   ctypes.c_float(eps), _ptr(out), _code(out, "norm output"), _ptr(rows), ctypes.c_int(n_out),
+                   ctypes.c_int(T), ctypes.c_int(H), _Hip.stream())
+    return out
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """RMS norm over the last dimension, same dtype out as in."""
+    if _impl is not None:
+        return _impl.rms_norm(x, weight, eps)
+    _dev(x, weight)
+    n = x.shape[-1]
+    _check(weight.shape == (n,), "rms_norm: weight must match the last dimension")
+    out = torch.empty_like(x)
+    rows = x.numel() // n if n else 0
+    if rows:
+        hip().call("spy_rmsnorm", _ptr(x), _code(x, "rms_norm input"), _ptr(weight), _code(weight, "norm weight"),
+                   ctypes.c_float(eps), _ptr(out), ctypes.c_int64(rows), ctypes.c_int(n), _Hip.stream())
+    return out
+
+
+#: at or above this many rows a bfloat16 product goes to the library (hipBLASLt via torch), as the
+#: reference sends m >= 8 to cuBLAS (src/backends/cuda/cuda_operator.cpp); below, to the hand-written
+#: streaming kernel.  Set by the engine after measuring; tests pin both paths.
+LIBRARY_GEMM_MIN_ROWS = 8
+SKINNY_MAX_ROWS = 64
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """y = x . w^T with w stored [N, K] (out_features, in_features), float32 accumulation.
+
+    float32 anywhere among x and w -> the hand-written true-fp32 kernel.  All bfloat16: the streaming
+    MFMA kernel for few rows, the library product for many."""
+    if _impl is not None:
+        return _impl.linear(x, w, out_dtype)
+    _dev(x, w)
+    _check(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "linear: x [M, K] and w [N, K] expected, got %s and %s"
+           % (tuple(x.shape), tuple(w.shape)))
+    M, K = x.shape
+    N = w.shape[0]
+    out_dtype = out_dtype or x.dtype
+    _check(out_dtype in _CODES, "linear: output dtype must be float32 or bfloat16")
+    if M == 0:
+        return torch.empty((0, N), dtype=out_dtype, device=x.device)
+    all_bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    if all_bf16 and M <= SKINNY_MAX_ROWS and (M < LIBRARY_GEMM_MIN_ROWS or out_dtype == torch.float32 or _skinny_preferred(M, N, K)) \
+            and K % 8 == 0:
+        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        hip().call("spy_gemm_skinny", _ptr(x), _ptr(w), _ptr(out), _code(out, "out"), ctypes.c_int(M), ctypes.c_int(N),
+                   ctypes.c_int(K), _Hip.stream())
+        return out
+    if all_bf16 and out_dtype == torch.bfloat16 and M >= LIBRARY_GEMM_MIN_ROWS:
+        return torch.matmul(x, w.t())
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    hip().call("spy_gemm", _ptr(x), _code(x, "x"), _ptr(w), _code(w, "w"), _ptr(out), _code(out, "out"),
+               ctypes.c_int(M), ctypes.c_int(N), ctypes.c_int(K), _Hip.stream())
+    return out
+
+
+def _skinny_preferred(M, N, K) -> bool:
+    return True
+
+
+def qk_norm_rope_store(qkv: torch.Tensor, n_q: int, n_kv: int, d: int, q_norm_w, k_norm_w, eps: float,
+                       cos, sin, rotary_dim: int, positions: torch.Tensor, k_cache, v_cache, page_size: int,
+                       slots: Optional[torch.Tensor]) -> torch.Tensor:
+    """From the fused projection ``qkv [T, (n_q + 2 n_kv) d]``: per-head RMS norm of q and k (if
+    weights are given), half-split rotation of the first ``rotary_dim`` dims by the tables
+    ``cos/sin [positions, rotary_dim/2]`` (if given), q written to the result ``[T, n_q d]``;
+    k and v written into the cache pages at ``slots[t] = page * page_size + offset``
+    (skipped for slot -1 or when ``slots`` is None)."""
+    if _impl is not None:
+        return _impl.qk_norm_rope_store(qkv, n_q, n_kv, d, q_norm_w, k_norm_w, eps, cos, sin, rotary_dim, positions,
+                                        k_cache, v_cache, page_size, slots)
+    _dev(qkv, q_norm_w, k_norm_w, cos, sin, positions, k_cache, v_cache, slots)
+    T = qkv.shape[0]
+    _check(qkv.dim() == 2 and qkv.shape[1] == (n_q + 2 * n_kv) * d, "qk_norm_rope_store: qkv must be [T, (n_q + 2 n_kv) d]")
+    _check(positions.dtype == torch.int32 and positions.shape == (T,), "qk_norm_rope_store: positions must be int32 [T]")
+    _check((q_norm_w is None) == (k_norm_w is None), "qk_norm_rope_store: q and k norm weights come together")
+    if q_norm_w is not None:
+        _check(q_norm_w.shape == (d,) and k_norm_w.shape == (d,) and q_norm_w.dtype == k_norm_w.dtype,
+               "qk_norm_rope_store: norm weights must be [head_dim] of one dtype")
+    max_pos = 0
+    if cos is not None:
+        _check(rotary_dim % 2 == 0 and 0 < rotary_dim <= d, "qk_norm_rope_store: rotary_dim must be even and <= head_dim")
+        _check(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.dim() == 2 and cos.shape == sin.shape
+               and cos.shape[1] == rotary_dim // 2, "qk_norm_rope_store: cos/sin must be float32 [positions, rotary_dim/2]")
+        max_pos = cos.shape[0]
+    else:
+        rotary_dim = 0
+    num_pages = 0
+    if slots is not None:
+        _check(slots.dtype == torch.int32 and slots.shape == (T,), "qk_norm_rope_store: slots must be int32 [T]")
+        _check(k_cache is not None and k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype,
+               "qk_norm_rope_store: the cache must have the activation dtype")
+        num_pages = k_cache.shape[0]
+        _check(tuple(k_cache.shape) == (num_pages, n_kv, page_size, d) and tuple(v_cache.shape) == (num_pages, n_kv, d, page_size),
+               "qk_norm_rope_store: cache pages must be K [pages, n_kv, page, d] and V [pages, n_kv, d, page]")
+    q = torch.empty((T, n_q * d), dtype=qkv.dtype, device=qkv.device)
+    if T:
+        hip().call("spy_qknorm_rope_store", _ptr(qkv), _code(qkv, "qkv"), _ptr(q), ctypes.c_int(T), ctypes.c_int(n_q),
+                   ctypes.c_int(n_kv), ctypes.c_int(d), _ptr(q_norm_w), _ptr(k_norm_w),
+                   ctypes.c_int(-1 if q_norm_w is None else _code(q_norm_w, "q norm weight")), ctypes.c_float(eps),
+                   _ptr(cos), _ptr(sin), ctypes.c_int(rotary_dim), ctypes.c_int(max_pos), _ptr(positions),
+                   _ptr(k_cache if slots is not None else None), _ptr(v_cache if slots is not None else None),
+                   ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(slots), _Hip.stream())
+    return q
+
+
+class AttentionMeta:
+    """Batch description that the attention kernels read (all int32, on the device).
+
+    cu_q [S+1]: first query token of each entry;  pos0 [S]: position of that token in its request;
+    kv_len [S]: keys the request has after this step (pos0 + tokens of the entry);
+    block_table [S, max_blocks]: logical page -> physical page (-1 = none);
+    token_entry [T], positions [T]: per query token.
+    tiles: (tile_entry [N], tile_row0 [N]) 16-row tiles of (token, head-in-group) rows per entry,
+    built for one group size ``tiles_group``; None if not built.
+    Host-side: S, T, max_blocks, max_kv_len, max_q_len."""
+
+    def __init__(self, cu_q, pos0, kv_len, block_table, token_entry, positions, S, T, max_blocks, max_kv_len, max_q_len,
+                 tiles=None, tiles_group=0, num_tiles=0):
+        self.cu_q, self.pos0, self.kv_len, self.block_table = cu_q, pos0, kv_len, block_table
+        self.token_entry, self.positions = token_entry, positions
+        self.S, self.T, self.max_blocks, self.max_kv_len, self.max_q_len = S, T, max_blocks, max_kv_len, max_q_len
+        self.tiles, self.tiles_group, self.num_tiles = tiles, tiles_group, num_tiles
+
+
+MFMA_ATTENTION = True      # False forces the plain kernel for bfloat16 too (used by tests)
+DECODE_SPLIT_TARGET = 1024  # waves wanted in flight when all entries are single tokens
+
+
+def mfma_attention_ok(dtype, d: int, page_size: int) -> bool:
+    return MFMA_ATTENTION and dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256 and page_size % 8 == 0
+
+
+def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_size: int, meta: AttentionMeta,
+                    n_q: int, n_kv: int, d: int, scale: float, window: Optional[int]) -> torch.Tensor:
+    """Causal grouped-query attention of the step's query tokens over the paged cache
+    (which already holds this step's keys and values).  Query at position p reads keys
+    max(0, p - window + 1) .. p.  Scores, softmax and the weighted sum are float32."""
+    if _impl is not None:
+        return _impl.paged_attention(q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window)
+    _dev(q, k_cache, v_cache, meta.cu_q, meta.pos0, meta.kv_len, meta.block_table, meta.token_entry, meta.positions)
+    T, S = meta.T, meta.S
+    _check(q.shape == (T, n_q * d), "paged_attention: q must be [T, n_q d]")
+    _check(n_q % n_kv == 0, "paged_attention: n_q must be a multiple of n_kv")
+    num_pages = k_cache.shape[0]
+    _check(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "paged_attention: cache and q must have one dtype")
+    _check(tuple(k_cache.shape) == (num_pages, n_kv, page_size, d) and tuple(v_cache.shape) == (num_pages, n_kv, d, page_size),
+           "paged_attention: cache pages must be K [pages, n_kv, page, d] and V [pages, n_kv, d, page]")
+    for name, t, shape in (("cu_q", meta.cu_q, (S + 1,)), ("pos0", meta.pos0, (S,)), ("kv_len", meta.kv_len, (S,)),
+                           ("block_table", meta.block_table, (S, meta.max_blocks)), ("token_entry", meta.token_entry, (T,)),
+                           ("positions", meta.positions, (T,))):
+        _check(t.dtype == torch.int32 and tuple(t.shape) == shape, "paged_attention: %s must be int32 %s" % (name, shape))
+    _check(meta.max_kv_len <= meta.max_blocks * page_size, "paged_attention: block tables are shorter than the longest request")
+    win = 0 if window is None else int(window)
+    _check(win >= 0, "paged_attention: window must be positive")
+    out = torch.empty_like(q)
+    if T == 0:
+        return out
+    group = n_q // n_kv
+    if mfma_attention_ok(q.dtype, d, page_size) and meta.tiles is not None and meta.tiles_group == group:
+        tile_entry, tile_row0 = meta.tiles
+        _check(tile_entry.dtype == torch.int32 and tile_row0.dtype == torch.int32 and tile_entry.shape == (meta.num_tiles,)
+               and tile_row0.shape == (meta.num_tiles,), "paged_attention: tile lists must be int32 [num_tiles]")
+        splits = 1
+        if meta.max_q_len == 1:
+            # all single tokens: split the keys so that the chip is full, at least 64 keys a part
+            want = max(1, DECODE_SPLIT_TARGET // max(1, meta.num_tiles * n_kv))
+            splits = max(1, min(want, -(-meta.max_kv_len // 64), 64))
+        ws_floats = hip().lib.spy_attention_mfma_workspace(ctypes.c_int(meta.num_tiles), ctypes.c_int(n_kv), ctypes.c_int(d),
+                                                           ctypes.c_int(splits))
+        ws = torch.empty((max(1, ws_floats),), dtype=torch.float32, device=q.device)
+        hip().call("spy_attention_mfma", _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), ctypes.c_int(page_size),
+                   ctypes.c_int(num_pages), _ptr(meta.cu_q), _ptr(meta.pos0), _ptr(meta.kv_len), _ptr(meta.block_table),
+                   ctypes.c_int(meta.max_blocks), _ptr(tile_entry), _ptr(tile_row0), ctypes.c_int(meta.num_tiles),
+                   ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d),
+                   ctypes.c_float(scale), ctypes.c_int(win), ctypes.c_int(splits), _ptr(ws), _Hip.stream())
+        return out
+    hip().call("spy_attention_generic", _ptr(out), _ptr(q), _code(q, "q"), _ptr(k_cache), _ptr(v_cache),
+               ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(meta.kv_len), _ptr(meta.block_table),
+               ctypes.c_int(meta.max_blocks), _ptr(meta.token_entry), _ptr(meta.positions), ctypes.c_int(S), ctypes.c_int(T),
+               ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d), ctypes.c_float(scale), ctypes.c_int(win), _Hip.stream())
+    return out
+
+
+def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
+    """``gate_up [T, 2 I]`` = [gate | up]  ->  silu(gate) * up  [T, I], float32 arithmetic."""
+    if _impl is not None:
+        return _impl.swiglu(gate_up)
+    _dev(gate_up)
+    _check(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "swiglu: [T, 2 I] expected")
+    T, I = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((T, I), dtype=gate_up.dtype, device=gate_up.device)
+    if T * I:
+        hip().call("spy_swiglu", _ptr(gate_up), _ptr(out), _code(gate_up, "gate_up"), ctypes.c_int(T), ctypes.c_int(I),
+                   _Hip.stream())
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
+    """Row r: temperature[r] == 0 -> first maximum of logits[r]; else the token whose cumulative
+    probability of softmax(logits[r] / temperature[r]), over ascending token ids, first exceeds
+    u[r] in [0, 1).  int32 [R]."""
+    if _impl is not None:
+        return _impl.sample(logits, temperature, u)
+    _dev(logits, temperature, u)
+    _check(logits.dtype == torch.float32 and logits.dim() == 2, "sample: logits must be float32 [R, V]")
+    R, V = logits.shape
+    _check(temperature.dtype == torch.float32 and temperature.shape == (R,) and u.dtype == torch.float32 and u.shape == (R,),
+           "sample: temperature and u must be float32 [R]")
+    _check(V > 0, "sample: empty vocabulary")
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    if R:
+        hip().call("spy_sample", _ptr(logits), _ptr(temperature), _ptr(u), _ptr(out), ctypes.c_int(R), ctypes.c_int(V),
+                   _Hip.stream())
+    return out

@@ -1,0 +1,78 @@
+"""Grouped-query attention over the paged cache.
+
+Per step: fused q/k/v projection; per-head RMS norm of q and k (optional;
+before the rotation, src/models/qwen3.hpp:160-194); rotation; keys and values
+of all tokens of the step written to their pages before any query reads
+(src/backends/cpu/cpu_attention.cpp:61-68); then every query reads its keys
+through its request's block table with the causal mask ``key <= position``
+(:98-111), scale 1/sqrt(d) after the dot product (:59, :110), kv head
+``h * n_kv / n_q`` (:96); output projection.  One meaning for whole prompts,
+portions and single tokens.  ``window`` keeps only the last ``window`` keys.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from ..cache.spec import PagedKV
+from ..kernels import ops
+from ..weights.loader import WeightSpec
+from .base import Mixer, PositionEncoding
+
+
+class PagedAttention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 position: Optional[PositionEncoding], qk_norm_eps: Optional[float] = None,
+                 window: Optional[int] = None, scale: Optional[float] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
+        self.position = position
+        self.qk_norm_eps = qk_norm_eps
+        self.window = window
+        self.scale = 1.0 / math.sqrt(head_dim) if scale is None else float(scale)
+        self.w_qkv = self.w_o = self.q_norm = self.k_norm = None
+
+    # ---- weights ---------------------------------------------------------
+    def weight_specs(self, prefix):
+        H, nq, nkv, d = self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim
+        specs = [WeightSpec(prefix + ".q_proj.weight", (nq * d, H)), WeightSpec(prefix + ".k_proj.weight", (nkv * d, H)),
+                 WeightSpec(prefix + ".v_proj.weight", (nkv * d, H)), WeightSpec(prefix + ".o_proj.weight", (H, nq * d))]
+        if self.qk_norm_eps is not None:
+            specs += [WeightSpec(prefix + ".q_norm.weight", (d,), "norm"), WeightSpec(prefix + ".k_norm.weight", (d,), "norm")]
+        return specs
+
+    def bind(self, prefix, weights):
+        q, k, v = (weights[prefix + ".%s_proj.weight" % n] for n in "qkv")
+        if not (q.dtype == k.dtype == v.dtype):
+            q, k, v = q.float(), k.float(), v.float()
+        # one product for q, k and v: rows [q heads | k heads | v heads]
+        self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
+        self.w_o = weights[prefix + ".o_proj.weight"]
+        if self.qk_norm_eps is not None:
+            self.q_norm, self.k_norm = weights[prefix + ".q_norm.weight"], weights[prefix + ".k_norm.weight"]
+            if self.q_norm.dtype != self.k_norm.dtype:
+                self.q_norm, self.k_norm = self.q_norm.float(), self.k_norm.float()
+
+    # ---- cache -----------------------------------------------------------
+    def cache_spec(self):
+        return PagedKV(self.num_kv_heads, self.head_dim, self.window)
+
+    def plan(self, batch) -> None:
+        batch.add_attention_tiles(self.num_heads // self.num_kv_heads)
+
+    # ---- step ------------------------------------------------------------
+    def forward(self, x, batch, cache, store=True):
+        nq, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
+        qkv = ops.linear(x, self.w_qkv)
+        rot = self.position.rotary() if self.position is not None else None
+        cos, sin, rdim = rot if rot is not None else (None, None, 0)
+        slots = batch.slot_mapping(cache.group) if store else None
+        q = ops.qk_norm_rope_store(qkv, nq, nkv, d, self.q_norm, self.k_norm,
+                                   self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
+                                   cos, sin, rdim, batch.positions, cache.k, cache.v, cache.page_size, slots)
+        meta = batch.attention_meta(cache.group, nq // nkv)
+        a = ops.paged_attention(q, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window)
+        return ops.linear(a, self.w_o)

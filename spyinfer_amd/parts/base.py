@@ -1,0 +1,91 @@
+"""Interfaces of the parts a decoder is put together from.
+
+A part knows its own sizes and constants (given to its constructor), the
+safetensors names and shapes of its weights under a prefix, and how to run on
+the tokens of a step.  No part knows which model it is in; the model picks the
+parts layer by layer from its configuration.
+
+All parts run on a flat batch of tokens ``[T, ...]`` described by a
+``StepBatch`` (``spyinfer_amd.engine.batch``).  The residual stream is
+float32; activations between parts have the run dtype (bfloat16 or float32).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..weights.loader import WeightSpec
+
+
+class Part:
+    """Common protocol: weights by name."""
+
+    def weight_specs(self, prefix: str) -> List[WeightSpec]:
+        """Tensors this part reads, with full names under ``prefix``."""
+        return []
+
+    def bind(self, prefix: str, weights: Dict[str, torch.Tensor]) -> None:
+        """Take the tensors named by ``weight_specs(prefix)`` (already on the device)."""
+
+
+class Norm(Part):
+    """y = norm(x) over the hidden dimension."""
+
+    def add_norm(self, resid: torch.Tensor, delta: Optional[torch.Tensor], out_dtype: torch.dtype,
+                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """resid += delta in float32 (in place, unless ``rows`` selects rows), then the norm of
+        the sum in ``out_dtype``.  Fusing the residual sum into the norm saves one pass over
+        the hidden state."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """How positions enter the model.  A rotary encoding hands its tables to the mixer,
+    which applies them to queries and keys; an encoding added to the embeddings
+    overrides ``on_embeddings``."""
+
+    def prepare(self, device, max_positions: int) -> None:
+        pass
+
+    def rotary(self):
+        """None, or (cos, sin, rotary_dim): float32 tables [positions, rotary_dim/2]."""
+        return None
+
+    def on_embeddings(self, hidden: torch.Tensor, batch) -> torch.Tensor:
+        return hidden
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a request (attention here)."""
+
+    def cache_spec(self):
+        """``PagedKV``, ``FixedState`` or None: what one layer of this mixer keeps per request."""
+        return None
+
+    def plan(self, batch) -> None:
+        """Called once per step and per distinct mixer before the batch goes to the device:
+        may add integer arrays to it with ``batch.add_array``."""
+
+    def forward(self, x: torch.Tensor, batch, cache, store: bool = True) -> torch.Tensor:
+        """x [T, H] (normed) -> [T, H].  ``cache`` is this call's layer cache
+        (``PagedKVLayer``/``StateLayer``/None).  ``store=False``: read the cache of
+        another layer without writing to it."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
+        """x [T, H] (normed) -> [T, H]."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arrangement of norm, mixer and feed-forward in one layer."""
+
+    mixer: Mixer
+
+    def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], batch, cache, store: bool = True):
+        """(residual stream, pending addend) -> (residual stream, pending addend).  The addend
+        is summed into the stream by the next norm."""
+        raise NotImplementedError

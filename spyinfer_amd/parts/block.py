@@ -1,0 +1,29 @@
+"""Pre-norm block: h += mixer(norm1(h)); h += ffn(norm2(h))  (src/models/qwen3.hpp:122-278).
+The sums are carried as a pending addend and folded into the next norm's kernel."""
+from __future__ import annotations
+
+from .base import Block, FeedForward, Mixer, Norm
+
+
+class PreNormBlock(Block):
+    def __init__(self, norm1: Norm, mixer: Mixer, norm2: Norm, ffn: FeedForward,
+                 names=("input_layernorm", "self_attn", "post_attention_layernorm", "mlp")):
+        self.norm1, self.mixer, self.norm2, self.ffn = norm1, mixer, norm2, ffn
+        self.names = names
+
+    def _parts(self, prefix):
+        return zip((self.norm1, self.mixer, self.norm2, self.ffn), (prefix + "." + n for n in self.names))
+
+    def weight_specs(self, prefix):
+        return [s for part, p in self._parts(prefix) for s in part.weight_specs(p)]
+
+    def bind(self, prefix, weights):
+        for part, p in self._parts(prefix):
+            part.bind(p, weights)
+
+    def forward(self, resid, delta, batch, cache, store=True):
+        act = batch.act_dtype
+        n1 = self.norm1.add_norm(resid, delta, act)
+        a = self.mixer.forward(n1, batch, cache, store)
+        n2 = self.norm2.add_norm(resid, a, act)
+        return resid, self.ffn.forward(n2, batch)

@@ -1,0 +1,43 @@
+"""Token embedding and output head.  h[t] = E[id[t]] with no scaling
+(src/models/qwen3.hpp:114-119); logits = norm(h) . W^T for the asked rows only, W = E when the
+model ties them (src/models/qwen3.hpp:46, 283-301)."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.loader import WeightSpec
+from .base import Part
+
+
+class TokenEmbedding(Part):
+    def __init__(self, vocab_size: int, hidden_size: int):
+        self.vocab_size, self.hidden_size = vocab_size, hidden_size
+        self.weight = None
+
+    def weight_specs(self, prefix):
+        return [WeightSpec(prefix + ".weight", (self.vocab_size, self.hidden_size))]
+
+    def bind(self, prefix, weights):
+        self.weight = weights[prefix + ".weight"]
+
+    def forward(self, ids):
+        return ops.embedding(ids, self.weight)
+
+
+class LMHead(Part):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding = None):
+        self.vocab_size, self.hidden_size, self.tied_to = vocab_size, hidden_size, tied_to
+        self.weight = None
+
+    def weight_specs(self, prefix):
+        if self.tied_to is not None:
+            # a tied checkpoint may store the head again; it is not read (src/models/qwen3.hpp:46)
+            return [WeightSpec(prefix + ".weight", (self.vocab_size, self.hidden_size), optional=True)]
+        return [WeightSpec(prefix + ".weight", (self.vocab_size, self.hidden_size))]
+
+    def bind(self, prefix, weights):
+        self.weight = self.tied_to.weight if self.tied_to is not None else weights[prefix + ".weight"]
+
+    def forward(self, normed):
+        return ops.linear(normed, self.weight, torch.float32)

@@ -1,0 +1,33 @@
+"""Gated feed-forward: down( silu(gate(x)) * up(x) ), no biases
+(src/models/qwen3.hpp:232-263; src/backends/cpu/x64/kernels.cpp:242-247).
+Gate and up run as one product with rows [gate | up]."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.loader import WeightSpec
+from .base import FeedForward
+
+
+class GatedMLP(FeedForward):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
+        if activation != "silu":
+            raise ValueError("GatedMLP: activation %r is not implemented" % activation)
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.w_gate_up = self.w_down = None
+
+    def weight_specs(self, prefix):
+        H, I = self.hidden_size, self.intermediate_size
+        return [WeightSpec(prefix + ".gate_proj.weight", (I, H)), WeightSpec(prefix + ".up_proj.weight", (I, H)),
+                WeightSpec(prefix + ".down_proj.weight", (H, I))]
+
+    def bind(self, prefix, weights):
+        g, u = weights[prefix + ".gate_proj.weight"], weights[prefix + ".up_proj.weight"]
+        if g.dtype != u.dtype:
+            g, u = g.float(), u.float()
+        self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
+        self.w_down = weights[prefix + ".down_proj.weight"]
+
+    def forward(self, x, batch):
+        return ops.linear(ops.swiglu(ops.linear(x, self.w_gate_up)), self.w_down)
