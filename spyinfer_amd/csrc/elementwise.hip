@@ -1,0 +1,191 @@
+// Embedding gather, RMS norm with the residual sum folded in, SwiGLU, and the fused
+// per-head norm + rotation + cache store.  All arithmetic is float32; a bfloat16 value is
+// rounded once, when it is written.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------------
+// out[t, :] = table[ids[t], :]  (float32 out: the start of the residual stream)
+template <typename TW>
+__global__ void embedding_kernel(float* __restrict__ out, const TW* __restrict__ table, const int* __restrict__ ids, int H, int V) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    float* o = out + (size_t)t * H;
+    if (id < 0 || id >= V) {
+        for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = 0.f;
+        return;
+    }
+    const TW* row = table + (size_t)id * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32<TW>(row[i]);
+}
+
+extern "C" int spy_embedding(float* out, const void* table, int table_dtype, const int* ids, int T, int H, int V, hipStream_t st) {
+    SPY_REQUIRE(T > 0 && H > 0 && V > 0, "spy_embedding: empty operand");
+    SPY_DISPATCH(table_dtype, TW, embedding_kernel<TW><<<T, 256, 0, st>>>(out, (const TW*)table, ids, H, V));
+    SPY_CHECK_LAUNCH("spy_embedding");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// x = resid[t] (+ delta[t]);  rows == null: resid[t] = x.  out[r] = (x / sqrt(mean(x^2) + eps)) * w
+template <typename TA, typename TW>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restrict__ delta, const TW* __restrict__ w, float eps,
+                                   TA* __restrict__ out, const int* __restrict__ rows, int T, int H) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    int t = r;
+    if (rows) {
+        t = rows[r];
+        if (t < 0 || t >= T) {   // never the case for a checked batch; write zeros rather than read outside
+            for (int i = threadIdx.x; i < H; i += blockDim.x) out[(size_t)r * H + i] = from_f32<TA>(0.f);
+            return;
+        }
+    }
+    float* x = resid + (size_t)t * H;
+    const TA* dl = delta ? delta + (size_t)t * H : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = x[i];
+        if (dl) v += to_f32<TA>(dl[i]);
+        if (dl && !rows) x[i] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+    TA* o = out + (size_t)r * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = x[i];
+        if (dl && rows) v += to_f32<TA>(dl[i]);
+        o[i] = from_f32<TA>((scale * v) * to_f32<TW>(w[i]));
+    }
+}
+
+extern "C" int spy_add_rmsnorm(float* resid, const void* delta, const void* w, int w_dtype, float eps, void* out, int out_dtype,
+                               const int* rows, int n_out, int T, int H, hipStream_t st) {
+    SPY_REQUIRE(n_out > 0 && T > 0 && H > 0, "spy_add_rmsnorm: empty operand");
+    const int threads = H >= 1024 ? 512 : 256;
+    SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW><<<n_out, threads, 0, st>>>(
+        resid, (const TA*)delta, (const TW*)w, eps, (TA*)out, rows, T, H))));
+    SPY_CHECK_LAUNCH("spy_add_rmsnorm");
+    return 0;
+}
+
+template <typename TA, typename TW>
+__global__ void rmsnorm_kernel(const TA* __restrict__ x, const TW* __restrict__ w, float eps, TA* __restrict__ out, int n) {
+    __shared__ float red[16];
+    const TA* xr = x + (size_t)blockIdx.x * n;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) { float v = to_f32<TA>(xr[i]); ss += v * v; }
+    ss = block_sum(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)n + eps);
+    TA* o = out + (size_t)blockIdx.x * n;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) o[i] = from_f32<TA>((scale * to_f32<TA>(xr[i])) * to_f32<TW>(w[i]));
+}
+
+extern "C" int spy_rmsnorm(const void* x, int x_dtype, const void* w, int w_dtype, float eps, void* out, int64_t rows, int n,
+                           hipStream_t st) {
+    SPY_REQUIRE(rows > 0 && rows < (1ll << 31) && n > 0, "spy_rmsnorm: bad sizes");
+    const int threads = n >= 1024 ? 512 : (n > 64 ? 256 : 64);
+    SPY_DISPATCH(x_dtype, TA, SPY_DISPATCH(w_dtype, TW, (rmsnorm_kernel<TA, TW><<<(unsigned)rows, threads, 0, st>>>(
+        (const TA*)x, (const TW*)w, eps, (TA*)out, n))));
+    SPY_CHECK_LAUNCH("spy_rmsnorm");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t, i] = silu(in[t, i]) * in[t, I + i]
+template <typename TA>
+__global__ void swiglu_kernel(const TA* __restrict__ in, TA* __restrict__ out, int T, int I) {
+    const size_t n = (size_t)T * I;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = idx / I, i = idx - t * I;
+        const float g = to_f32<TA>(in[t * 2 * I + i]);
+        const float u = to_f32<TA>(in[t * 2 * I + I + i]);
+        out[idx] = from_f32<TA>((g / (1.0f + expf(-g))) * u);
+    }
+}
+
+extern "C" int spy_swiglu(const void* in, void* out, int dtype, int T, int I, hipStream_t st) {
+    SPY_REQUIRE(T > 0 && I > 0, "spy_swiglu: empty operand");
+    const size_t n = (size_t)T * I;
+    const unsigned blocks = (unsigned)((n + 255) / 256 > 65536 ? 65536 : (n + 255) / 256);
+    SPY_DISPATCH(dtype, TA, swiglu_kernel<TA><<<blocks, 256, 0, st>>>((const TA*)in, (TA*)out, T, I));
+    SPY_CHECK_LAUNCH("spy_swiglu");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// One block (one wave) per (token, head of q|k|v).  q, k: optional RMS norm over the head, then
+// half-split rotation of the first `rot` dims: y[j] = x[j] c - x[j+rot/2] s; y[j+rot/2] = x[j] s + x[j+rot/2] c.
+// q -> q_out[t, h, :];  k -> K[page, h, off, :];  v -> V[page, h, :, off]  (values lie transposed in a page).
+#define QK_MAX_D 512
+template <typename TA, typename TW>
+__global__ void qknorm_rope_store_kernel(const TA* __restrict__ qkv, TA* __restrict__ q_out, int n_q, int n_kv, int d,
+                                         const TW* __restrict__ qw, const TW* __restrict__ kw, float eps,
+                                         const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, int max_pos,
+                                         const int* __restrict__ positions, TA* __restrict__ kc, TA* __restrict__ vc,
+                                         int P, int num_pages, const int* __restrict__ slots) {
+    __shared__ float y[QK_MAX_D];
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int width = (n_q + 2 * n_kv) * d;
+    const TA* x = qkv + (size_t)t * width + (size_t)h * d;
+    const bool is_q = h < n_q, is_k = !is_q && h < n_q + n_kv;
+    int page = -1, off = 0;
+    if (!is_q) {
+        if (!slots) return;
+        const int slot = slots[t];
+        if (slot < 0 || slot >= num_pages * P) return;
+        page = slot / P;
+        off = slot - page * P;
+    }
+    if (!is_q && !is_k) {   // values: a plain copy into the transposed page
+        const int hv = h - n_q - n_kv;
+        TA* dst = vc + ((size_t)page * n_kv + hv) * d * P + off;
+        for (int j = lane; j < d; j += 64) dst[(size_t)j * P] = x[j];
+        return;
+    }
+    float ss = 0.f;
+    for (int j = lane; j < d; j += 64) { const float v = to_f32<TA>(x[j]); y[j] = v; ss += v * v; }
+    const TW* w = is_q ? qw : kw;
+    if (w) {
+        ss = wave_sum(ss);
+        const float scale = 1.0f / sqrtf(ss / (float)d + eps);
+        for (int j = lane; j < d; j += 64) y[j] = (scale * y[j]) * to_f32<TW>(w[j]);
+    }
+    __syncthreads();
+    int p = positions[t];
+    p = p < 0 ? 0 : (p >= max_pos && max_pos > 0 ? max_pos - 1 : p);
+    const int half = rot >> 1;
+    TA* dst = is_q ? q_out + ((size_t)t * n_q + h) * d : kc + (((size_t)page * n_kv + (h - n_q)) * P + off) * d;
+    for (int j = lane; j < d; j += 64) {
+        float v;
+        if (j < half) {
+            const float c = cos_t[(size_t)p * half + j], s = sin_t[(size_t)p * half + j];
+            v = y[j] * c - y[j + half] * s;
+        } else if (j < rot) {
+            const float c = cos_t[(size_t)p * half + j - half], s = sin_t[(size_t)p * half + j - half];
+            v = y[j - half] * s + y[j] * c;
+        } else {
+            v = y[j];
+        }
+        dst[j] = from_f32<TA>(v);
+    }
+}
+
+extern "C" int spy_qknorm_rope_store(const void* qkv, int dtype, void* q_out, int T, int n_q, int n_kv, int d, const void* qw,
+                                     const void* kw, int w_dtype, float eps, const float* cos_t, const float* sin_t, int rot,
+                                     int max_pos, const int* positions, void* kc, void* vc, int P, int num_pages,
+                                     const int* slots, hipStream_t st) {
+    SPY_REQUIRE(T > 0 && n_q > 0 && n_kv > 0 && d > 0, "spy_qknorm_rope_store: empty operand");
+    SPY_REQUIRE(d <= QK_MAX_D, "spy_qknorm_rope_store: head_dim %d exceeds the supported %d", d, QK_MAX_D);
+    SPY_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "spy_qknorm_rope_store: rotary_dim %d does not fit head_dim %d", rot, d);
+    SPY_REQUIRE(rot == 0 || (cos_t && sin_t && max_pos > 0), "spy_qknorm_rope_store: rotation without tables");
+    SPY_REQUIRE(!slots || (kc && vc && P > 0 && num_pages > 0), "spy_qknorm_rope_store: slots without a cache");
+    SPY_REQUIRE(n_q + 2 * n_kv <= 65535, "spy_qknorm_rope_store: too many heads");
+    const dim3 grid(T, n_q + 2 * n_kv);
+    const int wd = w_dtype < 0 ? SPY_F32 : w_dtype;
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(wd, TW, (qknorm_rope_store_kernel<TA, TW><<<grid, 64, 0, st>>>(
+        (const TA*)qkv, (TA*)q_out, n_q, n_kv, d, (const TW*)qw, (const TW*)kw, eps, cos_t, sin_t, rot, max_pos, positions,
+        (TA*)kc, (TA*)vc, P, num_pages, slots))));
+    SPY_CHECK_LAUNCH("spy_qknorm_rope_store");
+    return 0;
+}

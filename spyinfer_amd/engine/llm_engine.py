@@ -1,0 +1,158 @@
+"""The programmatic entry point, in the manner of the reference's ``LLMEngine``
+(src/engine/llm_engine.hpp:18-58): add_request, append_to_request, step, is_request_finished,
+remove_request, get_output_tokens, has_unfinished_requests.  Requests are token ids (the
+reference tokenises text itself; tokenisation is outside this engine).  Options are the
+reference's ``Config`` fields (src/config.hpp:17-30), given as keyword arguments as the
+reference takes them in its parameter map (src/engine/llm_engine.cpp:11-16).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, NamedTuple, Optional, Sequence as Seq
+
+import torch
+
+from ..config.engine_config import EngineConfig
+from ..sampling.sampler import Sampler, SamplingParams
+from .batch import StepEntry
+from .runner import ModelRunner, load_model
+from .scheduler import Scheduler
+from .sequence import Sequence, SequenceStatus
+
+
+class StepOutput(NamedTuple):
+    request_id: int
+    token: int
+    finished: bool
+
+
+class LLMEngine:
+    def __init__(self, model_path: str, device="cuda:0", **params):
+        known = {f for f in EngineConfig.__dataclass_fields__}
+        bad = sorted(set(params) - known)
+        if bad:
+            raise TypeError("unknown engine option(s): %s; known: %s" % (", ".join(bad), ", ".join(sorted(known))))
+        self.config = EngineConfig(model=model_path, **params)
+        self.config.validate()
+        self.device = torch.device(device)
+        self.model = load_model(model_path, self.config.dtype, self.device)
+        mc = self.model.config
+        # as the reference: a request never outgrows the model's positions (src/config.hpp:12)
+        self.config.max_model_len = min(self.config.max_model_len, getattr(mc, "max_position_embeddings", 1 << 30))
+        num_pages = self.config.num_kvcache_blocks
+        if num_pages is None:
+            num_pages = self._pages_from_free_memory()
+        self.runner = ModelRunner(self.model, self.config.dtype, self.device, self.config.kvcache_block_size, num_pages,
+                                  self.config.max_num_seqs, self.config.max_num_batched_tokens)
+        self.scheduler = Scheduler(self.runner.manager, self.config.max_num_batched_tokens, self.config.max_num_seqs,
+                                   self.config.max_model_len)
+        self.sampler = Sampler(self.device)
+        self.eos_token_id = getattr(mc, "eos_token_id", -1)
+        self._sequences: Dict[int, Sequence] = {}
+        self._next_id = 0
+        self.stats = dict(steps=0, prefill_tokens=0, decode_tokens=0)
+
+    def _pages_from_free_memory(self) -> int:
+        per_page = ModelRunner.bytes_per_page(self.model, self.config.kvcache_block_size, self.config.dtype)
+        if per_page == 0:
+            return 1
+        if self.device.type == "cuda":
+            free, _total = torch.cuda.mem_get_info(self.device)
+        else:
+            free = 1 << 30
+        # room for the activations of one full step is left beside the pool
+        pages = int(free * self.config.gpu_memory_utilization * 0.9) // per_page
+        cap = -(-self.config.max_model_len // self.config.kvcache_block_size) * self.config.max_num_seqs
+        return max(1, min(pages, cap))
+
+    # ---- requests --------------------------------------------------------
+    def add_request(self, prompt_tokens: Seq[int], params: Optional[SamplingParams] = None) -> int:
+        params = params or SamplingParams()
+        params.validate()
+        rid = self._next_id
+        seq = Sequence(rid, [int(t) for t in prompt_tokens], params)
+        for t in seq.tokens:
+            if not (0 <= t < self.model.vocab_size):
+                raise ValueError("token id %d is outside the vocabulary of %d" % (t, self.model.vocab_size))
+        self.scheduler.add_sequence(seq)
+        self._next_id += 1
+        self._sequences[rid] = seq
+        return rid
+
+    def append_to_request(self, request_id: int, tokens: Seq[int], params: Optional[SamplingParams] = None) -> None:
+        """A further turn of a finished request (src/engine/llm_engine.cpp:40-73).  The reference keeps the
+        finished request's pages and prefills the new tokens only; here pages went back when it finished,
+        so the history is computed again.  The tokens that come out are the same."""
+        seq = self._sequences[request_id]
+        if seq.status is not SequenceStatus.FINISHED:
+            raise ValueError("request %d is still running" % request_id)
+        seq.tokens += [int(t) for t in tokens]
+        seq.num_prompt_tokens = len(seq.tokens)
+        if params is not None:
+            params.validate()
+            seq.params = params
+        seq.finish_reason = None
+        self.scheduler.add_sequence(seq)
+
+    def is_request_finished(self, request_id: int) -> bool:
+        return self._sequences[request_id].status is SequenceStatus.FINISHED
+
+    def has_unfinished_requests(self) -> bool:
+        return self.scheduler.has_unfinished()
+
+    def get_output_tokens(self, request_id: int) -> List[int]:
+        """Prompt and generated tokens, as the reference returns them (src/engine/llm_engine.cpp:139-147)."""
+        return list(self._sequences[request_id].tokens)
+
+    def get_generated_tokens(self, request_id: int) -> List[int]:
+        seq = self._sequences[request_id]
+        return seq.tokens[seq.num_prompt_tokens:]
+
+    def finish_reason(self, request_id: int) -> Optional[str]:
+        return self._sequences[request_id].finish_reason
+
+    def remove_request(self, request_id: int) -> None:
+        seq = self._sequences.pop(request_id)
+        if seq.status is not SequenceStatus.FINISHED:
+            self.scheduler.abort(seq)
+
+    # ---- one step --------------------------------------------------------
+    def step(self) -> List[StepOutput]:
+        scheduled = self.scheduler.schedule()
+        if not scheduled:
+            return []
+        entries = []
+        for sc in scheduled:
+            seq = sc.seq
+            lo = seq.num_computed
+            entries.append(StepEntry(seq.cache, seq.tokens[lo:lo + sc.num_tokens], [sc.num_tokens - 1] if sc.samples else []))
+        logits = self.runner.step(entries)
+        sampling = [sc.seq for sc in scheduled if sc.samples]
+        tokens = self.sampler.sample(
+            logits, [s.params.temperature for s in sampling],
+            [s.params.seed if s.params.seed is not None else self.config.seed + s.id for s in sampling],
+            [s.num_generated for s in sampling])
+        outputs = []
+        for seq, tok in zip(sampling, tokens):
+            seq.tokens.append(tok)
+            reason = None
+            # the end-of-sequence token stays in the request's tokens (src/engine/model_runner.cpp:141-151)
+            if tok == self.eos_token_id and not seq.params.ignore_eos:
+                reason = "eos"
+            elif seq.params.max_new_tokens is not None and seq.num_generated >= seq.params.max_new_tokens:
+                reason = "max_new_tokens"
+            elif len(seq) >= self.config.max_model_len:
+                reason = "max_model_len"
+            if reason:
+                self.scheduler.finish(seq, reason)
+            outputs.append(StepOutput(seq.id, tok, reason is not None))
+        self.stats["steps"] += 1
+        for sc in scheduled:
+            self.stats["decode_tokens" if sc.num_tokens == 1 and sc.samples else "prefill_tokens"] += sc.num_tokens
+        return outputs
+
+    def generate(self, prompts: Seq[Seq[int]], params: Optional[SamplingParams] = None) -> List[List[int]]:
+        """Convenience loop: all prompts at once, generated tokens of each."""
+        ids = [self.add_request(p, params) for p in prompts]
+        while any(not self.is_request_finished(i) for i in ids):
+            self.step()
+        return [self.get_generated_tokens(i) for i in ids]

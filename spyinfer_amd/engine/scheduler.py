@@ -1,0 +1,133 @@
+"""Continuous batching above the step function.
+
+Like the reference's scheduler (src/engine/scheduler.cpp:17-122) it keeps a waiting and a
+running queue, admits in arrival order while pages are free, and lets every running request
+take part in every step.  Beyond it: a token budget per step (``max_num_batched_tokens``,
+which the reference stores but never consults) under which prompts are cut into portions,
+a cap on running requests (``max_num_seqs``), and a decided answer when pages run out.
+
+One step holds, in this order:
+  1. one token for every running request that is decoding;
+  2. portions of running requests that still have prompt (or recomputation) left, in admission
+     order, each as large as the remaining budget allows;
+  3. newly admitted requests from the head of the waiting queue, while a slot, budget and pages
+     for their first portion are there.  The first one that does not fit stops admission
+     (arrival order is kept, as in the reference, scheduler.cpp:39-42).
+When pages run out for a running request, the request admitted last is preempted: its pages
+and slot are given back, it keeps all its tokens and goes to the FRONT of the waiting queue,
+and recomputes them when it is admitted again.  (The reference skips the token and
+desynchronises its batch, scheduler.cpp:79-86.)  A request that could never fit the pool is
+refused when it is added.
+"""
+from __future__ import annotations
+
+import collections
+from typing import Deque, List, NamedTuple
+
+from ..cache.manager import CacheManager
+from .sequence import Sequence, SequenceStatus
+
+
+class Scheduled(NamedTuple):
+    seq: Sequence
+    num_tokens: int        # tokens of seq.tokens[num_computed : num_computed + num_tokens] run in this step
+    samples: bool          # the portion reaches the request's last known token: a new token is sampled
+
+
+class Scheduler:
+    def __init__(self, manager: CacheManager, max_num_batched_tokens: int, max_num_seqs: int, max_model_len: int):
+        self.manager = manager
+        self.max_num_batched_tokens = max_num_batched_tokens
+        self.max_num_seqs = max_num_seqs
+        self.max_model_len = max_model_len
+        self.waiting: Deque[Sequence] = collections.deque()
+        self.running: List[Sequence] = []
+        self.num_preemptions = 0
+        self._admitted = 0
+
+    # ---- queues ----------------------------------------------------------
+    def add_sequence(self, seq: Sequence) -> None:
+        if len(seq) == 0:
+            raise ValueError("a request needs at least one prompt token")
+        if len(seq) >= self.max_model_len:
+            raise ValueError("the prompt has %d tokens; max_model_len is %d" % (len(seq), self.max_model_len))
+        limit = min(self.max_model_len, len(seq) + (seq.params.max_new_tokens or self.max_model_len))
+        if limit > self.manager.max_tokens_per_request():
+            raise ValueError("the request may reach %d tokens; the cache pool holds %d" % (limit, self.manager.max_tokens_per_request()))
+        seq.status = SequenceStatus.WAITING
+        self.waiting.append(seq)
+
+    def has_unfinished(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    def finish(self, seq: Sequence, reason: str) -> None:
+        """The request ends: what it holds goes back to the pools at once."""
+        seq.status = SequenceStatus.FINISHED
+        seq.finish_reason = reason
+        if seq in self.running:
+            self.running.remove(seq)
+        if seq.cache is not None and seq.cache.live:
+            self.manager.release(seq.cache)
+        seq.cache = None
+
+    def abort(self, seq: Sequence) -> None:
+        if seq in self.waiting:
+            self.waiting.remove(seq)
+        self.finish(seq, "removed")
+
+    def _preempt(self, seq: Sequence) -> None:
+        self.running.remove(seq)
+        self.manager.release(seq.cache)
+        seq.cache = None
+        seq.status = SequenceStatus.WAITING
+        seq.num_preemptions += 1
+        self.num_preemptions += 1
+        self.waiting.appendleft(seq)
+
+    # ---- one step --------------------------------------------------------
+    def schedule(self) -> List[Scheduled]:
+        budget = self.max_num_batched_tokens
+        out: List[Scheduled] = []
+        # 1 and 2: running requests, decoding ones first, each group in admission order
+        order = sorted(self.running, key=lambda s: (s.is_prefill, s.admit_order))
+        for seq in order:
+            if seq.status is not SequenceStatus.RUNNING:
+                continue                       # preempted while an earlier request was served
+            if budget <= 0:
+                break
+            left = len(seq) - seq.num_computed
+            n = min(left, budget)
+            while not self.manager.can_reserve(seq.cache, n):
+                victim = max(self.running, key=lambda s: s.admit_order)
+                if victim is seq and len(self.running) == 1:
+                    raise RuntimeError("request %d cannot get pages although it runs alone; the pool is too small" % seq.id)
+                for x in out:
+                    if x.seq is victim:    # a victim scheduled earlier in this step leaves it and returns its budget
+                        budget += x.num_tokens
+                out = [x for x in out if x.seq is not victim]
+                self._preempt(victim)
+                if victim is seq:
+                    break
+            if seq.status is not SequenceStatus.RUNNING:
+                continue
+            self.manager.reserve(seq.cache, n)
+            out.append(Scheduled(seq, n, n == left))
+            budget -= n
+        # 3: admission from the head of the waiting queue
+        while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs and self.manager.can_admit():
+            seq = self.waiting[0]
+            n = min(len(seq), budget)
+            cache = self.manager.admit(seq.id)
+            if not self.manager.can_reserve(cache, n):
+                self.manager.release(cache)
+                break
+            self.waiting.popleft()
+            seq.cache = cache
+            seq.status = SequenceStatus.RUNNING
+            seq.admit_order = self._admitted
+            self._admitted += 1
+            self.running.append(seq)
+            self.manager.reserve(cache, n)
+            out.append(Scheduled(seq, n, n == len(seq)))
+            budget -= n
+        return out

@@ -74,6 +74,9 @@ class _Hip:
         for name in ("spy_embedding", "spy_add_rmsnorm", "spy_rmsnorm", "spy_gemm", "spy_qknorm_rope_store",
                      "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_swiglu",
                      "spy_sample", "spy_gemm_skinny"):
+            if not hasattr(self.lib, name):
+                raise KernelError("the kernel library %s lacks %s: rebuild it (python -c 'import __graft_entry__ as g; g.build()')"
+                                  % (self.lib._name, name))
             getattr(self.lib, name).restype = ctypes.c_int64 if name.endswith("_workspace") else ctypes.c_int
 
     def call(self, name, *args):
@@ -157,7 +160,7 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
 #: reference sends m >= 8 to cuBLAS (src/backends/cuda/cuda_operator.cpp); below, to the hand-written
 #: streaming kernel.  Set by the engine after measuring; tests pin both paths.
 LIBRARY_GEMM_MIN_ROWS = 8
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 0
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
@@ -260,7 +263,7 @@ class AttentionMeta:
         self.tiles, self.tiles_group, self.num_tiles = tiles, tiles_group, num_tiles
 
 
-MFMA_ATTENTION = True      # False forces the plain kernel for bfloat16 too (used by tests)
+MFMA_ATTENTION = False     # False forces the plain kernel for bfloat16 too (used by tests)
 DECODE_SPLIT_TARGET = 1024  # waves wanted in flight when all entries are single tokens
 
 

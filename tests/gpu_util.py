@@ -1,0 +1,27 @@
+import pytest
+import torch
+
+
+def require_gpu():
+    """The GPU tests fail (not skip) when the kernel library cannot be loaded on a GPU box."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    from spyinfer_amd.kernels import ops
+    ops.install_test_double(None)
+    ops.hip()
+    return torch.device("cuda:0")
+
+
+TOL = {torch.float32: dict(atol=2e-5, rtol=2e-5), torch.bfloat16: dict(atol=2e-2, rtol=2e-2)}
+
+
+def close(got, ref, dtype, scale=1.0, what=""):
+    tol = TOL[dtype]
+    got, ref = got.detach().double().cpu(), ref.detach().double().cpu()
+    err = (got - ref).abs()
+    lim = tol["atol"] * scale + tol["rtol"] * ref.abs()
+    bad = ~(err <= lim)
+    if bad.any():
+        idx = torch.nonzero(bad)[0].tolist()
+        raise AssertionError("%s: first wrong element at %s: got %r, expected %r (%d of %d wrong, max err %.3g)"
+                             % (what, idx, got[tuple(idx)].item(), ref[tuple(idx)].item(), int(bad.sum()), bad.numel(), err.max().item()))

@@ -1,0 +1,335 @@
+"""Each HIP kernel alone against a plain float64/float32 torch formula of the same operation, at
+sizes other than the engine's: sizes that are no power of two, one row, many rows, odd head
+counts and groups, pages of several sizes."""
+import math
+
+import pytest
+import torch
+
+from tests.gpu_util import close, require_gpu
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def rnd(shape, dtype, dev, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).to(dev)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,H,V", [(1, 64, 10), (37, 200, 331), (300, 4096, 1000)])
+def test_embedding(dtype, T, H, V):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    table = rnd((V, H), dtype, dev, 1)
+    ids = torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(2)).int().to(dev)
+    out = ops.embedding(ids, table)
+    assert out.dtype == torch.float32
+    assert torch.equal(out.cpu(), table.cpu()[ids.cpu().long()].float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("wdtype", DTYPES)
+@pytest.mark.parametrize("T,H,eps", [(1, 64, 1e-6), (19, 200, 1e-5), (130, 4096, 1e-6), (3, 5120, 1e-2)])
+def test_add_rms_norm(dtype, wdtype, T, H, eps):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    resid = rnd((T, H), torch.float32, dev, 3, 2.0)
+    delta = rnd((T, H), dtype, dev, 4)
+    w = (1 + 0.1 * rnd((H,), torch.float32, dev, 5)).to(wdtype)
+    x = resid.double() + delta.double()
+    ref = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w.double()
+    r2 = resid.clone()
+    out = ops.add_rms_norm(r2, delta, w, eps, dtype)
+    close(out, ref, dtype, what="add_rms_norm")
+    close(r2, x, torch.float32, what="residual sum")
+    # rows: only those rows, residual untouched; no delta
+    rows = torch.tensor([T - 1, 0, T // 2], dtype=torch.int32, device=dev)
+    r3 = resid.clone()
+    out = ops.add_rms_norm(r3, delta, w, eps, dtype, rows)
+    close(out, ref[rows.long()], dtype, what="add_rms_norm rows")
+    assert torch.equal(r3, resid)
+    x0 = resid.double()
+    out = ops.add_rms_norm(r3, None, w, eps, dtype)
+    close(out, x0 / torch.sqrt((x0 * x0).mean(-1, keepdim=True) + eps) * w.double(), dtype, what="rms_norm without delta")
+    assert torch.equal(r3, resid)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rms_norm_eps_matters(dtype):
+    """A tiny row tells eps 1e-6 from 1e-5; an all-zero row gives zeros."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    x = torch.full((2, 96), 1e-3, dtype=dtype, device=dev)
+    x[1] = 0
+    w = torch.ones(96, dtype=dtype, device=dev)
+    a = ops.rms_norm(x, w, 1e-6).float()
+    b = ops.rms_norm(x, w, 1e-5).float()
+    xv = float(x[0, 0])
+    assert abs(a[0, 0].item() - xv / math.sqrt(xv * xv + 1e-6)) < 1e-2
+    assert abs(b[0, 0].item() - xv / math.sqrt(xv * xv + 1e-5)) < 1e-2
+    assert a[0, 0].item() > 2 * b[0, 0].item()
+    assert torch.all(a[1] == 0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 8, 10), (2, 4, 3), (4, 1024, 1024), (9, 1024, 1030), (120, 100, 1000), (1, 331, 88),
+                                   (65, 200, 136), (7, 4096, 4096), (33, 160, 96)])
+def test_linear(dtype, M, N, K):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    x = rnd((M, K), dtype, dev, 6)
+    w = rnd((N, K), dtype, dev, 7, 0.05)
+    ref = x.double() @ w.double().t()
+    for od in (dtype, torch.float32):
+        out = ops.linear(x, w, od)
+        assert out.dtype == od and out.shape == (M, N)
+        close(out, ref, dtype if od == dtype else (torch.float32 if dtype == torch.float32 else torch.bfloat16),
+              scale=math.sqrt(K) * 0.05, what="linear %s->%s" % (dtype, od))
+
+
+def test_linear_reference_vector():
+    """test/test_linear.cpp:53-60 of the reference: x . W^T before the bias."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    x = torch.tensor([[1., 2, 3], [4, 5, 6]], device=dev)
+    w = torch.tensor([[1., 2, 3], [4, 5, 6], [7, 8, 9], [10, 11, 12]], device=dev)
+    assert ops.linear(x, w).cpu().tolist() == [[14, 32, 50, 68], [32, 77, 122, 167]]
+
+
+def test_linear_float32_is_true_float32():
+    """No reduced-precision matrix mode: products of numbers that need 24 bits come out exact."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    x = torch.tensor([[1.0 + 2 ** -20, 1.0]], device=dev)
+    w = torch.tensor([[1.0, -1.0]], device=dev)
+    assert ops.linear(x, w).item() == 2 ** -20
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_linear_mixed_weight_dtype(dtype):
+    """A weight stored in 32-bit stays so, beside bfloat16 activations."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    x = rnd((5, 72), dtype, dev, 8)
+    w = rnd((40, 72), torch.float32, dev, 9)
+    close(ops.linear(x, w), x.double() @ w.double().t(), dtype, scale=8.0, what="mixed linear")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu(dtype):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    # ramp of the reference's test (test/test_swiglu.cpp:43-46)
+    n = 100100
+    i = torch.arange(n)
+    gate = ((i % 100).float() / 10.0 - 5.0)
+    up = ((i % 70).float() / 15.0 - 2.0)
+    T, I = 100, 1001
+    gu = torch.cat([gate.view(T, I), up.view(T, I)], dim=1).to(dtype).to(dev)
+    out = ops.swiglu(gu)
+    g, u = gu[:, :I].double(), gu[:, I:].double()
+    close(out, g / (1 + torch.exp(-g)) * u, dtype, what="swiglu")
+    edge = torch.tensor([[0.0, 30.0, -30.0, 3.0, 3.0, 3.0]], dtype=dtype, device=dev)
+    o = ops.swiglu(edge).float().cpu()[0]
+    assert o[0] == 0 and abs(o[1] - 90) < 0.5 and abs(o[2]) < 1e-6
+
+
+def plain_qk(qkv, n_q, n_kv, d, qw, kw, eps, theta, rot, pos):
+    T = qkv.shape[0]
+    x = qkv.double()
+    q = x[:, :n_q * d].view(T, n_q, d)
+    k = x[:, n_q * d:(n_q + n_kv) * d].view(T, n_kv, d)
+    v = x[:, (n_q + n_kv) * d:].view(T, n_kv, d)
+    if qw is not None:
+        q = q / torch.sqrt((q * q).mean(-1, keepdim=True) + eps) * qw.double()
+        k = k / torch.sqrt((k * k).mean(-1, keepdim=True) + eps) * kw.double()
+    if rot:
+        half = rot // 2
+        freq = theta ** (-torch.arange(half, dtype=torch.float64) / half)
+        ang = pos.double()[:, None] * freq[None]
+        # complex form of the half-split rotation: (x[j] + i x[j + half]) * exp(i p freq_j)
+        def r(t):
+            z = torch.complex(t[..., :half], t[..., half:rot]) * torch.polar(torch.ones_like(ang), ang)[:, None, :]
+            return torch.cat([z.real, z.imag, t[..., rot:]], -1)
+        q, k = r(q), r(k)
+    return q, k, v
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_q,n_kv,d,rot,P,norm", [(4, 2, 16, 16, 16, True), (8, 2, 32, 32, 8, True), (6, 3, 48, 48, 16, True),
+                                                   (3, 1, 80, 40, 4, False), (32, 8, 128, 128, 16, True), (5, 5, 256, 256, 32, True)])
+def test_qk_norm_rope_store(dtype, n_q, n_kv, d, rot, P, norm):
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.parts.rotary import RotaryEmbedding
+    dev = require_gpu()
+    T, pages, theta, eps = 23, 9, 12345.0, 1e-5
+    qkv = rnd((T, (n_q + 2 * n_kv) * d), dtype, dev, 10)
+    qw = (1 + 0.2 * rnd((d,), torch.float32, dev, 11)).to(dtype) if norm else None
+    kw = (1 + 0.2 * rnd((d,), torch.float32, dev, 12)).to(dtype) if norm else None
+    pos = torch.randint(0, 500, (T,), generator=torch.Generator().manual_seed(13)).int()
+    rope = RotaryEmbedding(d, theta, rot)
+    rope.prepare(dev, 512)
+    slots = torch.randperm(pages * P, generator=torch.Generator().manual_seed(14))[:T].int()
+    slots[3] = -1
+    kc = torch.full((pages, n_kv, P, d), 7.0, dtype=dtype, device=dev)
+    vc = torch.full((pages, n_kv, d, P), 7.0, dtype=dtype, device=dev)
+    q = ops.qk_norm_rope_store(qkv, n_q, n_kv, d, qw, kw, eps, rope.cos, rope.sin, rot, pos.to(dev), kc, vc, P, slots.to(dev))
+    rq, rk, rv = plain_qk(qkv.cpu(), n_q, n_kv, d, None if qw is None else qw.cpu(), None if kw is None else kw.cpu(), eps, theta, rot, pos)
+    # angles reach 500 rad in float32: allow for their rounding (|x| * 500 * 2^-24 * few)
+    close(q.view(T, n_q, d), rq, dtype, scale=8.0, what="q")
+    kc_ref = torch.full((pages, n_kv, P, d), 7.0, dtype=torch.float64)
+    vc_ref = torch.full((pages, n_kv, d, P), 7.0, dtype=torch.float64)
+    for t in range(T):
+        s = int(slots[t])
+        if s >= 0:
+            kc_ref[s // P, :, s % P, :] = rk[t]
+            vc_ref[s // P, :, :, s % P] = rv[t]
+    close(kc, kc_ref, dtype, scale=8.0, what="k cache")
+    assert torch.equal(vc.cpu().double(), vc_ref.to(dtype).double()), "values must be stored unchanged"
+
+
+def plain_paged_attention(q, kc, vc, P, bt, token_entry, positions, n_q, n_kv, d, scale, window):
+    T = q.shape[0]
+    out = torch.zeros(T, n_q, d, dtype=torch.float64)
+    qd = q.double().view(T, n_q, d)
+    for t in range(T):
+        s, p = int(token_entry[t]), int(positions[t])
+        lo = 0 if not window else max(0, p - window + 1)
+        keys = range(lo, p + 1)
+        K = torch.stack([kc[bt[s][c // P], :, c % P, :] for c in keys]).double()
+        V = torch.stack([vc[bt[s][c // P], :, :, c % P] for c in keys]).double()
+        for h in range(n_q):
+            g = h * n_kv // n_q
+            pr = torch.softmax((K[:, g] @ qd[t, h]) * scale, 0)
+            out[t, h] = pr @ V[:, g]
+    return out.view(T, n_q * d)
+
+
+def make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed, window=None, spike=False):
+    """entries: list of (tokens already cached, tokens in this step).  Pages are dealt in a random
+    order; unused pages and slots hold NaN."""
+    from spyinfer_amd.kernels.ops import AttentionMeta
+    g = torch.Generator().manual_seed(seed)
+    total_pages = sum(-(-(a + n) // P) for a, n in entries) + 3
+    order = torch.randperm(total_pages, generator=g).tolist()
+    kc = torch.full((total_pages, n_kv, P, d), float("nan"), dtype=dtype)
+    vc = torch.full((total_pages, n_kv, d, P), float("nan"), dtype=dtype)
+    bt, cu, pos0, kvl, te, ps = [], [0], [], [], [], []
+    maxb = max(-(-(a + n) // P) for a, n in entries)
+    for s, (a, n) in enumerate(entries):
+        nb = -(-(a + n) // P)
+        pages = [order.pop() for _ in range(nb)]
+        bt.append(pages + [-1] * (maxb - nb))
+        for c in range(a + n):
+            kc[pages[c // P], :, c % P, :] = torch.randn(n_kv, d, generator=g).to(dtype)
+            vc[pages[c // P], :, :, c % P] = torch.randn(n_kv, d, generator=g).to(dtype)
+        cu.append(cu[-1] + n); pos0.append(a); kvl.append(a + n)
+        te += [s] * n; ps += list(range(a, a + n))
+    T = cu[-1]
+    q = torch.randn(T, n_q * d, generator=g).to(dtype)
+    if spike:
+        # one far key per request gets a score that stands out: a kernel that skips or misplaces it fails
+        for s, (a, n) in enumerate(entries):
+            if a + n > 3:
+                c = 1
+                t = cu[s + 1] - 1
+                for h in range(n_q):
+                    gk = h * n_kv // n_q
+                    kc[bt[s][c // P], gk, c % P, :] = (q[t].view(n_q, d)[h].float() * 1.5).to(dtype)
+    G = n_q // n_kv
+    tile_entry, tile_row0 = [], []
+    for s, (a, n) in enumerate(entries):
+        for r0 in range(0, n * G, 16):
+            tile_entry.append(s); tile_row0.append(r0)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    meta = AttentionMeta(i32(cu), i32(pos0), i32(kvl), i32(bt), i32(te), i32(ps), len(entries), T, maxb, max(kvl),
+                         max(n for _, n in entries), (i32(tile_entry), i32(tile_row0)), G, len(tile_entry))
+    return q, kc, vc, bt, te, ps, meta
+
+
+ATT_CASES = [
+    # n_q, n_kv, d, P, entries (cached, new), window
+    (4, 2, 16, 16, [(0, 5)], None),
+    (8, 2, 32, 8, [(0, 1), (0, 40), (7, 2)], None),
+    (6, 3, 48, 16, [(0, 70), (33, 1), (100, 1), (15, 17)], None),
+    (32, 8, 128, 16, [(300, 1), (17, 1), (0, 33)], None),
+    (5, 5, 64, 32, [(0, 50), (90, 3)], None),
+    (16, 1, 80, 16, [(130, 1), (0, 21)], None),
+    (8, 4, 128, 16, [(0, 150), (140, 10), (149, 1)], 37),
+    (4, 4, 256, 64, [(60, 9), (0, 3)], None),
+    (3, 1, 112, 4, [(0, 19), (30, 1)], 8),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", range(len(ATT_CASES)))
+@pytest.mark.parametrize("mfma", [False, True])
+def test_paged_attention(dtype, case, mfma):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    n_q, n_kv, d, P, entries, window = ATT_CASES[case]
+    if mfma and not (dtype == torch.bfloat16 and d % 16 == 0 and P % 8 == 0):
+        pytest.skip("the MFMA kernel takes bfloat16, head sizes in steps of 16 and pages of a multiple of 8")
+    q, kc, vc, bt, te, ps, meta = make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed=case, window=window, spike=True)
+    scale = 1.0 / math.sqrt(d)
+    ref = plain_paged_attention(q, kc, vc, P, bt, te, ps, n_q, n_kv, d, scale, window)
+    old = ops.MFMA_ATTENTION
+    ops.MFMA_ATTENTION = mfma
+    try:
+        out = ops.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), P, meta, n_q, n_kv, d, scale, window)
+    finally:
+        ops.MFMA_ATTENTION = old
+    close(out, ref, dtype, scale=2.0, what="attention case %d" % case)
+
+
+def test_attention_without_rotation_is_library_sdpa():
+    """One request from an empty cache equals softmax(QK^T / sqrt(d) + causal) V of a library routine."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    n_q, n_kv, d, P, n = 4, 2, 32, 16, 45
+    q, kc, vc, bt, te, ps, meta = make_attention_case(torch.float32, dev, n_q, n_kv, d, P, [(0, n)], seed=99)
+    K = torch.stack([kc[bt[0][c // P], :, c % P, :] for c in range(n)])      # [n, n_kv, d]
+    V = torch.stack([vc[bt[0][c // P], :, :, c % P] for c in range(n)])
+    Kr = K.repeat_interleave(n_q // n_kv, dim=1).transpose(0, 1)             # [n_q, n, d]
+    Vr = V.repeat_interleave(n_q // n_kv, dim=1).transpose(0, 1)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.view(n, n_q, d).transpose(0, 1), Kr, Vr, is_causal=True)
+    out = ops.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), P, meta, n_q, n_kv, d, 1 / math.sqrt(d), None)
+    close(out.view(n, n_q, d), ref.transpose(0, 1), torch.float32, what="sdpa")
+
+
+@pytest.mark.parametrize("V", [7, 384, 151936])
+def test_sample(V):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    g = torch.Generator().manual_seed(V)
+    R = 9
+    logits = torch.randn(R, V, generator=g) * 2
+    logits[0, :] = 1.5                      # all equal: the first wins
+    logits[1, V - 1] = 50; logits[1, V // 2] = 50
+    temp = torch.tensor([0, 0, 0, 0.8, 0.8, 1.3, 0.05, 1.0, 1.0])
+    u = torch.tensor([0, 0, 0, 0.0, 0.999, 0.5, 0.7, 0.25, 0.75])
+    out = ops.sample(logits.to(dev), temp.to(dev), u.to(dev)).cpu()
+    assert out[0] == 0 and out[1] == V // 2 and out[2] == int(torch.argmax(logits[2]))
+    for r in range(3, R):
+        p = torch.softmax(logits[r].double() / float(temp[r]), 0)
+        c = torch.cumsum(p, 0)
+        k = int(out[r])
+        lo = float(c[k - 1]) if k > 0 else 0.0
+        # the chosen id's cumulative interval holds u (up to float32 rounding of the sums)
+        assert lo - 1e-4 <= float(u[r]) <= float(c[k]) + 1e-4, (r, k, lo, float(c[k]), float(u[r]))
+        assert p[k] > 0
+
+
+def test_sample_frequencies():
+    """Empirical frequencies on a 4-token distribution follow softmax(logits / T)."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    R = 4000
+    logits = torch.tensor([0.0, 1.0, 2.0, -1.0]).repeat(R, 1)
+    u = torch.rand(R, generator=torch.Generator().manual_seed(0))
+    out = ops.sample(logits.to(dev), torch.full((R,), 0.7).to(dev), u.to(dev)).cpu().long()
+    freq = torch.bincount(out, minlength=4).double() / R
+    p = torch.softmax(logits[0].double() / 0.7, 0)
+    assert (freq - p).abs().max() < 0.03
