@@ -1,0 +1,107 @@
+"""Generation through the entry point on the CPU stand-in for the kernels: greedy tokens equal
+the plain implementation's whatever the budget, the pool or the company; temperature sampling
+does not depend on the batch."""
+import pytest
+import torch
+
+from spyinfer_amd.sampling import SamplingParams, uniform_for
+from tests.configs import INIT, TINY_A, TINY_B
+from tests.plain.qwen3_plain import PlainQwen3
+
+
+@pytest.fixture(scope="module")
+def folder_a(tmp_path_factory):
+    from spyinfer_amd.weights import write_random_model
+    return write_random_model(str(tmp_path_factory.mktemp("gen_a")), TINY_A, 31, torch.bfloat16, **INIT)
+
+
+@pytest.fixture(scope="module")
+def folder_b(tmp_path_factory):
+    from spyinfer_amd.weights import write_random_model
+    return write_random_model(str(tmp_path_factory.mktemp("gen_b")), TINY_B, 32, torch.bfloat16, **INIT)
+
+
+def prompts(vocab, lengths, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, vocab, (n,), generator=g).tolist() for n in lengths]
+
+
+def test_greedy_equals_plain_under_every_schedule(folder_a, emu_ops):
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    ps = prompts(256, [5, 17, 33, 60])
+    plain = PlainQwen3(folder_a)
+    want = [plain.greedy(p, 16) for p in ps]
+    sp = SamplingParams(max_new_tokens=16, ignore_eos=True)
+    for opts in (dict(), dict(max_num_batched_tokens=32), dict(max_num_batched_tokens=7, max_num_seqs=3),
+                 dict(num_kvcache_blocks=7, max_num_batched_tokens=24)):      # 7 pages of 16: preemption
+        kw = dict(dtype="float32", device="cpu", max_model_len=128, num_kvcache_blocks=40, max_num_seqs=8)
+        kw.update(opts)
+        eng = LLMEngine(folder_a, **kw)
+        got = eng.generate(ps, sp)
+        assert got == want, opts
+        assert eng.runner.manager.num_free_pages() == [kw["num_kvcache_blocks"]]
+        if "num_kvcache_blocks" in opts:
+            assert eng.scheduler.num_preemptions > 0
+        eng.runner.manager.check()
+
+
+def test_temperature_is_independent_of_the_batch(folder_b, emu_ops):
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    ps = prompts(384, [1, 40, 130], seed=2)
+    sp = SamplingParams(temperature=0.8, max_new_tokens=24, ignore_eos=True)
+    kw = dict(dtype="float32", device="cpu", max_model_len=256, kvcache_block_size=8, num_kvcache_blocks=80, seed=9)
+    together = LLMEngine(folder_b, max_num_batched_tokens=32, **kw).generate(ps, sp)
+    alone = []
+    for i, p in enumerate(ps):
+        eng = LLMEngine(folder_b, **kw)
+        eng._next_id = i                       # same request id -> same stream of uniform numbers
+        alone.append(eng.generate([p], sp)[0])
+    assert together == alone
+    assert len({tuple(x) for x in together}) == 3
+
+
+def test_finishing(folder_b, emu_ops):
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    eng = LLMEngine(folder_b, dtype="float32", device="cpu", max_model_len=12, kvcache_block_size=8, num_kvcache_blocks=8)
+    plain = PlainQwen3(folder_b)
+    p = prompts(384, [6], seed=3)[0]
+    first = plain.greedy(p, 1)[0]
+    eng.eos_token_id = first                   # the first generated token ends the request and is kept
+    rid = eng.add_request(p)
+    while not eng.is_request_finished(rid):
+        eng.step()
+    assert eng.get_output_tokens(rid) == p + [first] and eng.finish_reason(rid) == "eos"
+    rid = eng.add_request(p, SamplingParams(ignore_eos=True))
+    while not eng.is_request_finished(rid):
+        eng.step()
+    assert len(eng.get_output_tokens(rid)) == 12 and eng.finish_reason(rid) == "max_model_len"
+    # a further turn of a finished request
+    eng.config.max_model_len = eng.scheduler.max_model_len = 40
+    rid = eng.add_request(p, SamplingParams(max_new_tokens=3, ignore_eos=True))
+    while not eng.is_request_finished(rid):
+        eng.step()
+    turn1 = eng.get_output_tokens(rid)
+    eng.append_to_request(rid, [9, 8, 7], SamplingParams(max_new_tokens=2, ignore_eos=True))
+    while not eng.is_request_finished(rid):
+        eng.step()
+    assert eng.get_output_tokens(rid)[:len(turn1) + 3] == turn1 + [9, 8, 7]
+    assert eng.get_output_tokens(rid)[len(turn1) + 3:] == plain.greedy(turn1 + [9, 8, 7], 2)
+    eng.remove_request(rid)
+    assert not eng.has_unfinished_requests()
+    with pytest.raises(TypeError, match="known"):
+        LLMEngine(folder_b, device="cpu", page_size=4)
+    with pytest.raises(ValueError, match="vocabulary"):
+        eng.add_request([999])
+
+
+def test_uniform_numbers():
+    us = [uniform_for(3, i) for i in range(2000)]
+    assert all(0.0 <= u < 1.0 for u in us) and abs(sum(us) / len(us) - 0.5) < 0.03
+    assert uniform_for(3, 5) == uniform_for(3, 5) != uniform_for(4, 5)
+
+
+def test_cli_usage(capsys):
+    from spyinfer_amd.__main__ import main
+    assert main([]) == 1
+    assert main(["-m", "x", "-b", "cuda"]) == 1
+    assert "Available backends: hip" in capsys.readouterr().err
