@@ -1,0 +1,160 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X.
+
+Default: the Qwen3-8B shape of BASELINE.json configs[2] (36 layers, hidden 4096, 32 query and
+8 key/value heads of 128, intermediate 12288, vocabulary 151936, untied head) with random
+bfloat16 weights; 8 requests with 1024-token random prompts decode through the engine's own step
+(scheduler, step function, cache, kernels, device sampling).  A "step" is one decode step.
+Prints ONE JSON line: decoded tokens per second, plus the prefill of 2048 tokens, the decode
+step's HBM roofline, and decode at batch 1 and 64.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--dtype bfloat16|float32]
+"""
+import argparse
+import json
+import sys
+import time
+
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+MODEL_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_act="silu", num_hidden_layers=36, hidden_size=4096,
+                num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936,
+                rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960,
+                bos_token_id=151643, eos_token_id=151645)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (both numbers are reported)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=1024)
+    ap.add_argument("--context", type=int, default=4096, help="max_model_len")
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--points", default="1,64", help="further decode batch sizes to report (empty: none)")
+    ap.add_argument("--enforce-eager", action="store_true")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
+        return 2
+
+    import torch
+
+    from spyinfer_amd.cache.spec import PagedKV
+    from spyinfer_amd.config.registry import architecture_of
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.sampling import SamplingParams
+    from spyinfer_amd.weights.random_init import random_tensors_on_device
+
+    ops.hip()
+    dev = torch.device("cuda:0")
+    raw = dict(MODEL_8B)
+    model_layers = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    arch = architecture_of(raw)
+    cfg = arch.config_cls.from_dict(raw)
+    model = arch.build(cfg)
+    run_dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    weights = random_tensors_on_device(model.weight_specs(), args.seed, run_dtype, dev)
+    model.bind(weights, dev)
+    del weights
+    torch.cuda.empty_cache()
+
+    points = [int(x) for x in args.points.split(",") if x.strip()]
+    max_batch = max([args.batch] + points)
+    page = 16
+    pages_per_req = -(-args.context // page)
+    eng = LLMEngine.__new__(LLMEngine)
+    eng._init_with_model(model, dev, dtype=args.dtype, max_model_len=args.context, kvcache_block_size=page,
+                         num_kvcache_blocks=pages_per_req * max_batch + 8, max_num_seqs=max_batch,
+                         max_num_batched_tokens=max(16384, args.prefill_tokens), enforce_eager=args.enforce_eager, seed=args.seed)
+    g = torch.Generator().manual_seed(args.seed)
+
+    def prompts(n, length):
+        return [torch.randint(0, cfg.vocab_size, (length,), generator=g).tolist() for _ in range(n)]
+
+    act_bytes = 2 if args.dtype == "bfloat16" else 4
+    L, H, I, V = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    nq, nkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    layer_params = H * (nq + 2 * nkv) * d + nq * d * H + 3 * H * I + 2 * H + 2 * d
+    weight_bytes = (L * layer_params + H + V * H) * act_bytes              # every weight a decode step uses, once
+    kv_bytes_per_token = sum(2 * s.num_kv_heads * s.head_dim * act_bytes for s in model.cache_specs() if isinstance(s, PagedKV))
+
+    def decode_run(batch, steps, warmup):
+        """tokens/s, ms/step, mean context over the timed steps."""
+        ids = [eng.add_request(p, SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + 1, ignore_eos=True))
+               for p in prompts(batch, args.prompt_len)]
+        while any(s.is_prefill or s.num_generated == 0 for s in (eng._sequences[i] for i in ids)):
+            eng.step()                                                       # prompts, in portions under the budget
+        for _ in range(warmup):
+            eng.step()
+        ctx0 = sum(len(eng._sequences[i]) for i in ids) / batch
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            out = eng.step()
+            assert len(out) == batch
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        ctx1 = sum(len(eng._sequences[i]) for i in ids) / batch
+        for i in ids:
+            eng.remove_request(i)
+        return batch * steps / dt, dt / steps * 1e3, (ctx0 + ctx1) / 2
+
+    def prefill_run(tokens, repeats=3):
+        best = None
+        for _ in range(repeats + 1):
+            rc = eng.runner.manager.admit("prefill")
+            eng.runner.manager.reserve(rc, tokens)
+            toks = prompts(1, tokens)[0]
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            logits = eng.runner.step([StepEntry(rc, toks, [tokens - 1])])
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            eng.runner.manager.release(rc)
+            assert logits.shape == (1, V)
+            best = dt if best is None else min(best, dt)       # the first run also warms the library up
+        return best
+
+    value, ms, ctx = decode_run(args.batch, args.steps, args.warmup)
+    step_bytes = weight_bytes + args.batch * ctx * kv_bytes_per_token
+    achieved = step_bytes / (ms * 1e-3) / 1e9
+    pf = prefill_run(args.prefill_tokens)
+    T = args.prefill_tokens
+    linear_flops = 2 * T * L * (H * (nq + 2 * nkv) * d + nq * d * H + 3 * H * I) + 2 * V * H
+    attn_flops = L * 4 * d * nq * T * (T + 1) / 2
+    pf_flops = linear_flops + attn_flops
+    extra = {}
+    for b in points:
+        v, _, _ = decode_run(b, max(8, args.steps // 2), max(4, args.warmup // 2))
+        extra["decode_b%d" % b] = round(v, 1)
+    line = {
+        "metric": "decode tok/s at batch %d (Qwen3-8B shape, %d-token prompts)" % (args.batch, args.prompt_len),
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, uniform-random token ids)",
+        "config": {"model": "Qwen3-8B shape", "layers": L, "layers_of_model": model_layers, "hidden": H, "q_heads": nq,
+                   "kv_heads": nkv, "head_dim": d, "intermediate": I, "vocab": V, "global_batch": args.batch,
+                   "seq_len": args.context, "prompt_len": args.prompt_len, "mean_context": round(ctx, 1), "page_size": page,
+                   "graphs": not args.enforce_eager, "parallelism": "single GPU"},
+        "prefill": {"value": round(T / pf, 1), "tokens": T, "ms": round(pf * 1e3, 3),
+                    "frac": round(pf_flops / pf / PEAK_FLOPS[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "points": extra,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -31,10 +31,18 @@ class LLMEngine:
         bad = sorted(set(params) - known)
         if bad:
             raise TypeError("unknown engine option(s): %s; known: %s" % (", ".join(bad), ", ".join(sorted(known))))
-        self.config = EngineConfig(model=model_path, **params)
+        config = EngineConfig(model=model_path, **params)
+        config.validate()
+        self._init_with_model(load_model(model_path, config.dtype, torch.device(device)), device, **params)
+        self.config.model = model_path
+
+    def _init_with_model(self, model, device, **params) -> None:
+        """Set the engine up around a model whose weights are already bound (measurements make
+        their weights on the device instead of reading a folder)."""
+        self.config = EngineConfig(**params)
         self.config.validate()
         self.device = torch.device(device)
-        self.model = load_model(model_path, self.config.dtype, self.device)
+        self.model = model
         mc = self.model.config
         # as the reference: a request never outgrows the model's positions (src/config.hpp:12)
         self.config.max_model_len = min(self.config.max_model_len, getattr(mc, "max_position_embeddings", 1 << 30))

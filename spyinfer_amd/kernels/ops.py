@@ -156,11 +156,12 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return out
 
 
-#: at or above this many rows a bfloat16 product goes to the library (hipBLASLt via torch), as the
-#: reference sends m >= 8 to cuBLAS (src/backends/cuda/cuda_operator.cpp); below, to the hand-written
-#: streaming kernel.  Set by the engine after measuring; tests pin both paths.
-LIBRARY_GEMM_MIN_ROWS = 8
-SKINNY_MAX_ROWS = 0
+#: A bfloat16 product with at most this many rows runs on the hand-written streaming MFMA kernel
+#: (decode); above, the library product (hipBLASLt via torch) stands, as the reference sends
+#: m >= 8 to cuBLAS (src/backends/cuda/cuda_operator.cpp).  float32 results of bfloat16 operands
+#: (logits) always come from the hand-written kernels, which keep the float32 sums.
+SKINNY_MAX_ROWS = 16
+SKINNY_MAX_ROWS_F32_OUT = 64
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
@@ -180,22 +181,17 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     if M == 0:
         return torch.empty((0, N), dtype=out_dtype, device=x.device)
     all_bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-    if all_bf16 and M <= SKINNY_MAX_ROWS and (M < LIBRARY_GEMM_MIN_ROWS or out_dtype == torch.float32 or _skinny_preferred(M, N, K)) \
-            and K % 8 == 0:
+    if all_bf16 and K % 8 == 0 and M <= (SKINNY_MAX_ROWS_F32_OUT if out_dtype == torch.float32 else SKINNY_MAX_ROWS):
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         hip().call("spy_gemm_skinny", _ptr(x), _ptr(w), _ptr(out), _code(out, "out"), ctypes.c_int(M), ctypes.c_int(N),
                    ctypes.c_int(K), _Hip.stream())
         return out
-    if all_bf16 and out_dtype == torch.bfloat16 and M >= LIBRARY_GEMM_MIN_ROWS:
+    if all_bf16 and out_dtype == torch.bfloat16 and M > SKINNY_MAX_ROWS:
         return torch.matmul(x, w.t())
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     hip().call("spy_gemm", _ptr(x), _code(x, "x"), _ptr(w), _code(w, "w"), _ptr(out), _code(out, "out"),
                ctypes.c_int(M), ctypes.c_int(N), ctypes.c_int(K), _Hip.stream())
     return out
-
-
-def _skinny_preferred(M, N, K) -> bool:
-    return True
 
 
 def qk_norm_rope_store(qkv: torch.Tensor, n_q: int, n_kv: int, d: int, q_norm_w, k_norm_w, eps: float,

@@ -52,6 +52,27 @@ def random_tensors(specs: Iterable[WeightSpec], seed: int, dtype: torch.dtype = 
     return out
 
 
+def random_tensors_on_device(specs: Iterable[WeightSpec], seed: int, dtype: torch.dtype, device,
+                             matrix_std: float = 0.02, norm_mean: float = 1.0, norm_std: float = 0.0) -> Dict[str, torch.Tensor]:
+    """Random weights made on the device itself, for measurements at sizes whose files would take
+    minutes to write and read.  Same distributions as ``random_tensors``, other values."""
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    out = {}
+    for s in specs:
+        if s.optional:
+            continue
+        if s.role == "table":
+            out[s.name] = torch.randint(0, 2, s.shape, generator=g, dtype=torch.int32, device=device)
+        elif s.role == "norm":
+            out[s.name] = (norm_mean + norm_std * torch.randn(s.shape, generator=g, dtype=torch.float32, device=device)).to(dtype)
+        else:
+            t = torch.empty(s.shape, dtype=dtype, device=device)
+            t.normal_(0.0, matrix_std, generator=g)
+            out[s.name] = t
+    return out
+
+
 def write_random_model(folder: str, config: dict, seed: int, dtype: torch.dtype = torch.bfloat16, **init) -> str:
     """``config`` is the config.json content (with ``architectures``).  Returns ``folder``."""
     from ..config.registry import architecture_of
