@@ -1,3 +1,262 @@
+// Paged attention on MFMA for bfloat16: one wave per (16-row tile, kv head, part of the keys).
+//
+// Rows of a tile are (token, query head of the kv head's group) pairs of one batch entry, token
+// major: row r -> token r / G, head hk * G + r % G.  So a decoded token fills G rows, a prompt
+// portion of n tokens n * G rows, and one kernel serves single tokens, portions and their mix.
+//
+// Per block of 32 keys, with v_mfma_f32_16x16x32_bf16 (operand lane layout: lane % 16 = row or
+// column, lane / 16 = which 8 of the 32 k values):
+//   S^T = K . Q^T   two MFMA tiles (a, b).  Tile a takes keys c0 + 8(r/4) + r%4, tile b those + 4,
+//                   so that lane (q row, g) ends up with the scores of keys c0 + 8g .. c0 + 8g + 7.
+//   softmax         running maximum and sum per q row, float32; the maximum is combined over the
+//                   four lanes of a row (g) with two lane exchanges.
+//   O^T += V^T . P^T   P^T needs exactly those 8 keys per lane as its 8 k values: no data movement.
+//                   V^T comes from the cache, where values lie [d][key] within a page: lane
+//                   (d row, g) loads the 8 keys c0 + 8g .. +7 of row d with one 16-byte load.
+// Keys lie [key][d] within a page: lane (key, g) loads 16 bytes K[key][32 kk + 8 g ..].
+// With several parts per tile the partial (O, m, l) go to a workspace and a second kernel merges.
 #include "common.h"
-extern "C" int64_t spy_attention_mfma_workspace(int num_tiles, int n_kv, int d, int splits) { return 0; }
-extern "C" int spy_attention_mfma() { return spy_fail("spy_attention_mfma: not built yet"); }
+#include <math.h>
+
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
+__device__ __forceinline__ bf16x8_t zero8() { return bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
+
+template <int DMAX>
+__global__ __launch_bounds__(64) void attention_mfma_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+    int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
+    int n_q, int n_kv, int d, float scale, int window, int splits, float* __restrict__ ws) {
+    constexpr int KK = DMAX / 32;   // 32-wide chunks of the head dim for Q.K
+    constexpr int DT = DMAX / 16;   // 16-row tiles of the head dim for P.V
+    const int tile = blockIdx.x, hk = blockIdx.y, sp = blockIdx.z;
+    const int lane = threadIdx.x, r16 = lane & 15, g = lane >> 4;
+    const int s = tile_entry[tile];
+    const int row0 = tile_row0[tile];
+    const int G = n_q / n_kv;
+    const int q0 = cu_q[s];
+    const int n = cu_q[s + 1] - q0;
+    const int nrows = n * G;
+    const int p0 = pos0[s];
+    const int kvl = kv_len[s];
+    const int* bt = block_table + (size_t)s * max_blocks;
+
+    // this lane's query row (as column of S^T and O^T)
+    const int row = row0 + r16;
+    const bool row_ok = row < nrows;
+    const int tq = row_ok ? row / G : 0;
+    const int head = hk * G + (row_ok ? row % G : 0);
+    const int pos = p0 + tq;
+    const int lo_row = window > 0 ? max(0, pos - window + 1) : 0;
+
+    bf16x8_t bq[KK];
+    {
+        const bf16_t* qp = q + ((size_t)(q0 + tq) * n_q + head) * d;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const int dofs = kk * 32 + 8 * g;
+            bq[kk] = (row_ok && dofs < d) ? *reinterpret_cast<const bf16x8_t*>(qp + dofs) : zero8();
+        }
+    }
+    // keys this tile can see: from the first row's window start to the last row's position
+    const int last_row = min(nrows, row0 + 16) - 1;
+    const int hi = min(p0 + last_row / G, kvl - 1);
+    int lo = window > 0 ? max(0, p0 + row0 / G - window + 1) : 0;
+    lo &= ~31;
+    const int nblk = hi >= lo ? (hi - lo) / 32 + 1 : 0;
+    const int per = (nblk + splits - 1) / splits;
+    const int b_begin = sp * per, b_end = min(nblk, b_begin + per);
+
+    f32x4_t acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    for (int b = b_begin; b < b_end; ++b) {
+        const int c0 = lo + 32 * b;
+        // ---- S^T = K . Q^T ------------------------------------------------------------------
+        const int key_a = c0 + 8 * (r16 >> 2) + (r16 & 3);      // tile a; tile b is key_a + 4 (same page: P % 8 == 0)
+        int kpage = -1;
+        if (key_a < kvl) kpage = bt[key_a / P];
+        const bool k_ok = kpage >= 0 && kpage < num_pages;
+        const bf16_t* kp = kc + (((size_t)(k_ok ? kpage : 0) * n_kv + hk) * P + key_a % P) * d;
+        f32x4_t sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const int dofs = kk * 32 + 8 * g;
+            bf16x8_t ka = zero8(), kb = zero8();
+            if (k_ok && dofs < d) {
+                ka = *reinterpret_cast<const bf16x8_t*>(kp + dofs);
+                if (key_a + 4 < kvl) kb = *reinterpret_cast<const bf16x8_t*>(kp + 4 * d + dofs);
+            }
+            if (kk * 32 < d) {
+                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, bq[kk], sa, 0, 0, 0);
+                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, bq[kk], sb, 0, 0, 0);
+            }
+        }
+        // ---- V^T fragments (issued early; used after the softmax) ----------------------------
+        const int key_v = c0 + 8 * g;                             // this lane's 8 keys
+        int vpage = -1;
+        if (key_v < kvl) vpage = bt[key_v / P];
+        const bool v_ok = vpage >= 0 && vpage < num_pages;
+        const int v_valid = min(8, kvl - key_v);                  // keys of the group that exist (slots beyond hold anything)
+        const bf16_t* vp = vc + (((size_t)(v_ok ? vpage : 0) * n_kv + hk) * d) * P + key_v % P;
+        bf16x8_t vt[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const int dd = dt * 16 + r16;
+            vt[dt] = (v_ok && dd < d) ? *reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P) : zero8();
+        }
+        if (v_ok && v_valid < 8) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (j >= v_valid) vt[dt][j] = 0;
+        }
+        // ---- softmax over this lane's 8 keys of its q row --------------------------------------
+        float sc[8];
+        float bmax = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int key = c0 + 8 * g + j;
+            const float v = (j < 4 ? sa[j] : sb[j - 4]) * scale;
+            const bool ok = row_ok && key <= pos && key >= lo_row && key < kvl;
+            sc[j] = ok ? v : -INFINITY;
+            bmax = fmaxf(bmax, sc[j]);
+        }
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+        const float m_new = fmaxf(m, bmax);
+        float alpha = 1.f;
+        bf16x8_t pb = zero8();
+        if (m_new != -INFINITY) {
+            alpha = (m == -INFINITY) ? 0.f : __expf(m - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float pj = (sc[j] == -INFINITY) ? 0.f : __expf(sc[j] - m_new);
+                psum += pj;
+                pb[j] = (short)f32_to_bf16(pj);
+            }
+            l = l * alpha + psum;
+            m = m_new;
+        }
+        // ---- O^T = O^T * alpha + V^T . P^T -----------------------------------------------------
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            if (dt * 16 < d) {
+                acc[dt] *= alpha;
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt], pb, acc[dt], 0, 0, 0);
+            }
+        }
+    }
+    // the four lanes of a row hold partial sums of l
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+
+    if (splits == 1) {
+        if (!row_ok) return;
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        bf16_t* op = out + ((size_t)(q0 + tq) * n_q + head) * d;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const int dd = dt * 16 + 4 * g;
+            if (dd < d) {
+                uint2 w;
+                w.x = (uint32_t)f32_to_bf16(acc[dt][0] * inv) | ((uint32_t)f32_to_bf16(acc[dt][1] * inv) << 16);
+                w.y = (uint32_t)f32_to_bf16(acc[dt][2] * inv) | ((uint32_t)f32_to_bf16(acc[dt][3] * inv) << 16);
+                *reinterpret_cast<uint2*>(op + dd) = w;
+            }
+        }
+        return;
+    }
+    // partial result: ws[((tile * n_kv + hk) * splits + sp)] = { O[16][DMAX], m[16], l[16] }
+    float* w = ws + (((size_t)tile * n_kv + hk) * splits + sp) * (16 * (DMAX + 2));
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const int dd = dt * 16 + 4 * g;
+        *reinterpret_cast<f32x4_t*>(w + r16 * DMAX + dd) = acc[dt];
+    }
+    if (g == 0) {
+        w[16 * DMAX + r16] = m;
+        w[16 * DMAX + 16 + r16] = l;
+    }
+}
+
+// Merge the parts of each (tile, kv head): O = sum_i O_i e^(m_i - M) / sum_i l_i e^(m_i - M).
+template <int DMAX>
+__global__ __launch_bounds__(256) void attention_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws,
+                                                              const int* __restrict__ cu_q, const int* __restrict__ tile_entry,
+                                                              const int* __restrict__ tile_row0, int n_q, int n_kv, int d, int splits) {
+    __shared__ float wgt[64 * 16];     // weight of part i for row r: [i][r], up to 64 parts
+    __shared__ float inv_l[16];
+    const int tile = blockIdx.x, hk = blockIdx.y, tid = threadIdx.x;
+    const int s = tile_entry[tile], row0 = tile_row0[tile];
+    const int G = n_q / n_kv;
+    const int q0 = cu_q[s];
+    const int nrows = (cu_q[s + 1] - q0) * G;
+    const float* base = ws + ((size_t)tile * n_kv + hk) * splits * (16 * (DMAX + 2));
+    if (tid < 16) {
+        float M = -INFINITY;
+        for (int i = 0; i < splits; ++i) M = fmaxf(M, base[(size_t)i * (16 * (DMAX + 2)) + 16 * DMAX + tid]);
+        float L = 0.f;
+        for (int i = 0; i < splits; ++i) {
+            const float* w = base + (size_t)i * (16 * (DMAX + 2));
+            const float mi = w[16 * DMAX + tid];
+            const float e = (mi == -INFINITY) ? 0.f : __expf(mi - M);
+            wgt[i * 16 + tid] = e;
+            L += w[16 * DMAX + 16 + tid] * e;
+        }
+        inv_l[tid] = L > 0.f ? 1.0f / L : 0.f;
+    }
+    __syncthreads();
+    for (int e = tid; e < 16 * d; e += 256) {
+        const int r = e / d, dd = e - r * d;
+        const int row = row0 + r;
+        if (row >= nrows) continue;
+        float o = 0.f;
+        for (int i = 0; i < splits; ++i) o += base[(size_t)i * (16 * (DMAX + 2)) + r * DMAX + dd] * wgt[i * 16 + r];
+        const int tq = row / G, head = hk * G + row % G;
+        out[((size_t)(q0 + tq) * n_q + head) * d + dd] = f32_to_bf16(o * inv_l[r]);
+    }
+}
+
+static int dmax_of(int d) { return d <= 64 ? 64 : (d <= 128 ? 128 : 256); }
+
+extern "C" int64_t spy_attention_mfma_workspace(int num_tiles, int n_kv, int d, int splits) {
+    if (splits <= 1) return 0;
+    return (int64_t)num_tiles * n_kv * splits * 16 * (dmax_of(d) + 2);
+}
+
+extern "C" int spy_attention_mfma(void* out, const void* q, const void* kc, const void* vc, int P, int num_pages, const int* cu_q,
+                                  const int* pos0, const int* kv_len, const int* block_table, int max_blocks, const int* tile_entry,
+                                  const int* tile_row0, int num_tiles, int S, int T, int n_q, int n_kv, int d, float scale,
+                                  int window, int splits, float* ws, hipStream_t st) {
+    SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
+                "spy_attention_mfma: empty operand");
+    SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 256, "spy_attention_mfma: head_dim %d is not a multiple of 16 in 16..256", d);
+    SPY_REQUIRE(P % 8 == 0, "spy_attention_mfma: page size %d is not a multiple of 8", P);
+    SPY_REQUIRE(n_q % n_kv == 0, "spy_attention_mfma: n_q %d is not a multiple of n_kv %d", n_q, n_kv);
+    SPY_REQUIRE(splits >= 1 && splits <= 64, "spy_attention_mfma: %d parts (1..64 allowed)", splits);
+    SPY_REQUIRE(splits == 1 || ws, "spy_attention_mfma: parts without a workspace");
+    SPY_REQUIRE(n_kv <= 65535, "spy_attention_mfma: too many kv heads");
+    const dim3 grid(num_tiles, n_kv, splits);
+    const dim3 mgrid(num_tiles, n_kv);
+#define ATT_CASE(DM)                                                                                                          \
+    attention_mfma_kernel<DM><<<grid, 64, 0, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, P,    \
+                                                   num_pages, cu_q, pos0, kv_len, block_table, max_blocks, tile_entry,        \
+                                                   tile_row0, n_q, n_kv, d, scale, window, splits, ws);                       \
+    if (splits > 1)                                                                                                           \
+        attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits);
+    switch (dmax_of(d)) {
+        case 64: ATT_CASE(64) break;
+        case 128: ATT_CASE(128) break;
+        default: ATT_CASE(256) break;
+    }
+#undef ATT_CASE
+    SPY_CHECK_LAUNCH("spy_attention_mfma");
+    return 0;
+}

@@ -259,7 +259,7 @@ class AttentionMeta:
         self.tiles, self.tiles_group, self.num_tiles = tiles, tiles_group, num_tiles
 
 
-MFMA_ATTENTION = False     # False forces the plain kernel for bfloat16 too (used by tests)
+MFMA_ATTENTION = True      # False forces the plain kernel for bfloat16 too (used by tests)
 DECODE_SPLIT_TARGET = 1024  # waves wanted in flight when all entries are single tokens
 
 

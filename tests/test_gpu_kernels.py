@@ -260,6 +260,8 @@ ATT_CASES = [
     (8, 4, 128, 16, [(0, 150), (140, 10), (149, 1)], 37),
     (4, 4, 256, 64, [(60, 9), (0, 3)], None),
     (3, 1, 112, 4, [(0, 19), (30, 1)], 8),
+    (32, 8, 128, 16, [(1151, 1), (70, 1), (2000, 1), (0, 1)], None),      # single tokens only: keys split into parts
+    (6, 2, 96, 8, [(700, 1), (333, 1)], 100),
 ]
 
 
