@@ -87,6 +87,7 @@ class RequestCache:
         self.tables: List[List[int]] = [[] for _ in range(num_groups)]
         self.fresh = True            # no step has run yet: state slots must be reset
         self.live = True
+        self.versions = [0] * num_groups   # bumped whenever a table changes (lets callers cache copies)
 
     def pages_held(self, group: int) -> List[int]:
         return [p for p in self.tables[group] if p >= 0]
@@ -158,6 +159,8 @@ class CacheManager:
         for n, g in zip(need, self.page_groups):
             for _ in range(n):
                 rc.tables[g.index].append(g.pool.allocate())
+            if n:
+                rc.versions[g.index] += 1
         rc.reserved = max(rc.reserved, n_tokens)
 
     def commit(self, rc: RequestCache, n_tokens: int) -> None:
@@ -173,6 +176,7 @@ class CacheManager:
                 if table[i] >= 0:
                     g.pool.free(table[i])
                     table[i] = -1
+                    rc.versions[g.index] += 1
 
     def release(self, rc: RequestCache) -> None:
         """The request ends (or is preempted): everything it holds goes back."""
@@ -184,6 +188,7 @@ class CacheManager:
                 if p >= 0:
                     g.pool.free(p)
             rc.tables[g.index] = []
+            rc.versions[g.index] += 1
         self.slots.free(rc.slot)
         rc.live = False
         rc.num_tokens = 0

@@ -12,6 +12,7 @@ from __future__ import annotations
 
 from typing import Dict, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, RequestCache
@@ -34,18 +35,36 @@ class StepEntry:
                 raise ValueError("wanted place %d is outside the entry's %d tokens" % (w, len(self.tokens)))
 
 
+def _table_row(rc: RequestCache, group: int) -> np.ndarray:
+    """The request's block table of a group as an int32 array, cached until the table changes."""
+    cache = rc.__dict__.setdefault("_rows", {})
+    hit = cache.get(group)
+    if hit is None or hit[0] != rc.versions[group]:
+        hit = (rc.versions[group], np.asarray(rc.tables[group], dtype=np.int32))
+        cache[group] = hit
+    return hit[1]
+
+
 class StepBatch:
     def __init__(self, entries: Sequence[StepEntry], manager: CacheManager, act_dtype: torch.dtype, device,
-                 vocab_size: Optional[int] = None, min_max_blocks: int = 0):
+                 vocab_size: Optional[int] = None, fixed_max_blocks: int = 0):
+        """``fixed_max_blocks`` > 0: block tables have exactly that width (and attention splits its
+        keys into a number of parts that does not depend on the lengths), so that steps with the
+        same numbers of entries, tokens and wanted rows have one memory layout: what a captured
+        graph needs."""
         self.entries = list(entries)
         self.act_dtype = act_dtype
         self.device = torch.device(device)
-        self.S = len(self.entries)
-        self._arrays: Dict[str, List[int]] = {}
+        self.S = S = len(self.entries)
+        self.fixed_shape = fixed_max_blocks > 0
+        self._arrays: Dict[str, np.ndarray] = {}
         self._dev: Dict[str, torch.Tensor] = {}
         self._tiles: Dict[int, int] = {}
         seen = set()
-        token_ids, positions, token_entry, cu_q, pos0, kv_len, slot_ids, fresh, rows = [], [], [], [0], [], [], [], [], []
+        lens = np.empty(S, dtype=np.int32)
+        pos0 = np.empty(S, dtype=np.int32)
+        slot_ids = np.empty(S, dtype=np.int32)
+        fresh = np.empty(S, dtype=np.int32)
         for s, e in enumerate(self.entries):
             rc = e.cache
             if id(rc) in seen:
@@ -56,60 +75,66 @@ class StepBatch:
             n = len(e.tokens)
             if n > rc.reserved:
                 raise ValueError("request %r runs %d tokens but pages are reserved for %d" % (rc.request_id, n, rc.reserved))
-            if vocab_size is not None:
-                for t in e.tokens:
-                    if not (0 <= t < vocab_size):
-                        raise ValueError("token id %r of request %r is outside the vocabulary of %d" % (t, rc.request_id, vocab_size))
-            base = len(token_ids)
-            token_ids += e.tokens
-            positions += range(rc.num_tokens, rc.num_tokens + n)
-            token_entry += [s] * n
-            cu_q.append(base + n)
-            pos0.append(rc.num_tokens)
-            kv_len.append(rc.num_tokens + n)
-            slot_ids.append(rc.slot)
-            fresh.append(1 if rc.fresh else 0)
-            rows += [base + w for w in e.want]
-        self.T, self.R = len(token_ids), len(rows)
-        self.max_q_len = max((len(e.tokens) for e in self.entries), default=0)
-        self.max_kv_len = max(kv_len, default=0)
-        self.host = dict(token_ids=token_ids, positions=positions, token_entry=token_entry, cu_q=cu_q, pos0=pos0,
-                         kv_len=kv_len, slot_ids=slot_ids, fresh=fresh, logit_rows=rows)
-        for k, v in self.host.items():
-            self._arrays[k] = v
+            lens[s], pos0[s], slot_ids[s], fresh[s] = n, rc.num_tokens, rc.slot, 1 if rc.fresh else 0
+        cu_q = np.zeros(S + 1, dtype=np.int32)
+        np.cumsum(lens, out=cu_q[1:])
+        self.T = T = int(cu_q[-1])
+        token_ids = np.fromiter((t for e in self.entries for t in e.tokens), dtype=np.int64, count=T)
+        if vocab_size is not None and T and (token_ids.min() < 0 or token_ids.max() >= vocab_size):
+            bad = token_ids[(token_ids < 0) | (token_ids >= vocab_size)][0]
+            raise ValueError("token id %d is outside the vocabulary of %d" % (int(bad), vocab_size))
+        token_entry = np.repeat(np.arange(S, dtype=np.int32), lens)
+        positions = (np.arange(T, dtype=np.int32) - cu_q[:-1][token_entry] + pos0[token_entry]).astype(np.int32)
+        rows = np.fromiter((int(cu_q[s]) + w for s, e in enumerate(self.entries) for w in e.want), dtype=np.int32)
+        self.R = int(rows.shape[0])
+        kv_len = pos0 + lens
+        self.max_q_len = int(lens.max()) if S else 0
+        self.max_kv_len = int(kv_len.max()) if S else 0
+        self.lens = lens
+        for name, arr in (("token_ids", token_ids.astype(np.int32)), ("positions", positions), ("token_entry", token_entry),
+                          ("cu_q", cu_q), ("pos0", pos0), ("kv_len", kv_len.astype(np.int32)), ("slot_ids", slot_ids),
+                          ("fresh", fresh), ("logit_rows", rows)):
+            self._arrays[name] = arr
         # per page group: block tables padded with -1, and the slot of every token of the step
         self.max_blocks = []
         for g in manager.page_groups:
-            width = max([len(e.cache.tables[g.index]) for e in self.entries] + [min_max_blocks, 1])
-            table, slots = [], []
-            for e in self.entries:
-                t = e.cache.tables[g.index]
-                table += t + [-1] * (width - len(t))
-                for p in range(e.cache.num_tokens, e.cache.num_tokens + len(e.tokens)):
-                    slots.append(manager.slot_of_token(e.cache, g.index, p))
+            tables = [_table_row(e.cache, g.index) for e in self.entries]
+            width = max([len(t) for t in tables] + [1])
+            if fixed_max_blocks:
+                if width > fixed_max_blocks:
+                    raise ValueError("a block table has %d pages, the fixed width is %d" % (width, fixed_max_blocks))
+                width = fixed_max_blocks
+            table = np.full((S, width), -1, dtype=np.int32)
+            for s, t in enumerate(tables):
+                table[s, :len(t)] = t
+            P = g.page_size
+            pages = table[token_entry, positions // P] if T else np.empty(0, dtype=np.int32)
+            if T and pages.min() < 0:
+                t = int(np.argmin(pages))
+                raise ValueError("position %d of request %r has no page in group %d"
+                                 % (int(positions[t]), self.entries[int(token_entry[t])].cache.request_id, g.index))
             self.max_blocks.append(width)
-            self._arrays["block_table_%d" % g.index] = table
-            self._arrays["slot_mapping_%d" % g.index] = slots
+            self._arrays["block_table_%d" % g.index] = table.reshape(-1)
+            self._arrays["slot_mapping_%d" % g.index] = (pages * P + positions % P).astype(np.int32)
         self.num_groups = len(manager.page_groups)
 
     # ---- additions by parts, before upload ---------------------------------
-    def add_array(self, name: str, values: List[int]) -> None:
+    def add_array(self, name: str, values) -> None:
         if self._dev:
             raise RuntimeError("the batch is already on the device")
-        self._arrays[name] = list(values)
+        self._arrays[name] = np.asarray(values, dtype=np.int32).reshape(-1)
 
     def add_attention_tiles(self, group_size: int) -> None:
         """16-row tiles over each entry's rows (token-major, head-in-group minor) for a
         query-head group of ``group_size``."""
         if group_size in self._tiles:
             return
-        tile_entry, tile_row0 = [], []
-        for s, e in enumerate(self.entries):
-            nrows = len(e.tokens) * group_size
-            for r0 in range(0, nrows, ROWS_PER_TILE):
-                tile_entry.append(s)
-                tile_row0.append(r0)
-        self._tiles[group_size] = len(tile_entry)
+        ntiles = (self.lens.astype(np.int64) * group_size + ROWS_PER_TILE - 1) // ROWS_PER_TILE
+        tile_entry = np.repeat(np.arange(self.S, dtype=np.int32), ntiles)
+        first = np.zeros(self.S + 1, dtype=np.int64)
+        np.cumsum(ntiles, out=first[1:])
+        tile_row0 = ((np.arange(int(first[-1]), dtype=np.int64) - first[:-1][tile_entry]) * ROWS_PER_TILE).astype(np.int32)
+        self._tiles[group_size] = int(first[-1])
         self.add_array("tile_entry_%d" % group_size, tile_entry)
         self.add_array("tile_row0_%d" % group_size, tile_row0)
 
@@ -118,29 +143,33 @@ class StepBatch:
         """name -> (offset, length) in the packed buffer; every array starts at a multiple of 4 ints."""
         off, out = 0, {}
         for name, vals in self._arrays.items():
-            out[name] = (off, len(vals))
-            off += (len(vals) + 3) // 4 * 4
+            out[name] = (off, int(vals.shape[0]))
+            off += (int(vals.shape[0]) + 3) // 4 * 4
         return out, max(off, 4)
 
-    def upload(self, device_buffer: Optional[torch.Tensor] = None, pinned: Optional[torch.Tensor] = None) -> None:
+    def layout_key(self):
+        return tuple((name, int(v.shape[0])) for name, v in self._arrays.items())
+
+    def pack_into(self, host: torch.Tensor):
+        """Write all arrays into the int32 host tensor; returns (layout, total ints)."""
         layout, total = self.layout()
-        flat = [0] * total
+        if host.numel() < total:
+            raise ValueError("the step's metadata (%d ints) exceeds the buffer (%d)" % (total, host.numel()))
+        flat = host.numpy()
         for name, (off, n) in layout.items():
             flat[off:off + n] = self._arrays[name]
-        host = torch.tensor(flat, dtype=torch.int32)
-        if device_buffer is None:
-            dev = host.to(self.device)
-        else:
-            if device_buffer.numel() < total:
-                raise ValueError("the step's metadata (%d ints) exceeds the device buffer (%d)" % (total, device_buffer.numel()))
-            dev = device_buffer[:total]
-            if pinned is not None:
-                pinned[:total].copy_(host)
-                dev.copy_(pinned[:total], non_blocking=True)
-            else:
-                dev.copy_(host)
+        return layout, total
+
+    def bind_device(self, dev: torch.Tensor, layout) -> None:
         for name, (off, n) in layout.items():
             self._dev[name] = dev[off:off + n]
+
+    def upload(self) -> None:
+        """Simple path: a fresh host tensor, one copy to the device."""
+        _layout, total = self.layout()
+        host = torch.empty(total, dtype=torch.int32)
+        layout, total = self.pack_into(host)
+        self.bind_device(host.to(self.device), layout)
 
     def __getattr__(self, name):
         dev = self.__dict__.get("_dev", {})
@@ -164,4 +193,4 @@ class StepBatch:
             n_tiles = self._tiles[group_size]
         return AttentionMeta(self._dev["cu_q"], self._dev["pos0"], self._dev["kv_len"], self.block_table(group),
                              self._dev["token_entry"], self._dev["positions"], self.S, self.T, self.max_blocks[group],
-                             self.max_kv_len, self.max_q_len, tiles, group_size, n_tiles)
+                             self.max_kv_len, self.max_q_len, tiles, group_size, n_tiles, fixed_shape=self.fixed_shape)

@@ -50,7 +50,8 @@ class LLMEngine:
         if num_pages is None:
             num_pages = self._pages_from_free_memory()
         self.runner = ModelRunner(self.model, self.config.dtype, self.device, self.config.kvcache_block_size, num_pages,
-                                  self.config.max_num_seqs, self.config.max_num_batched_tokens)
+                                  self.config.max_num_seqs, self.config.max_num_batched_tokens,
+                                  enforce_eager=self.config.enforce_eager, max_model_len=self.config.max_model_len)
         self.scheduler = Scheduler(self.runner.manager, self.config.max_num_batched_tokens, self.config.max_num_seqs,
                                    self.config.max_model_len)
         self.sampler = Sampler(self.device)

@@ -44,7 +44,10 @@ def load_model(folder: str, dtype, device) -> DecoderModel:
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, dtype, device, page_size: int, num_pages: int, max_num_seqs: int,
-                 max_num_batched_tokens: int = 16384):
+                 max_num_batched_tokens: int = 16384, enforce_eager: bool = True, max_model_len: Optional[int] = None):
+        """``enforce_eager=False``: steps that hold single tokens only (decoding) are captured in
+        HIP graphs, one per number of entries and wanted rows, and replayed; their block tables
+        then have the fixed width that ``max_model_len`` needs."""
         self.model = model
         self.act_dtype = resolve_dtype(dtype)
         self.device = torch.device(device)
@@ -52,6 +55,14 @@ class ModelRunner:
         self.manager = CacheManager(model.cache_specs(), page_size, num_pages, max_num_seqs)
         self.storage = CacheStorage(self.manager, self.act_dtype, self.device)
         self.steps_run = 0
+        self.use_graphs = (not enforce_eager) and self.device.type == "cuda"
+        limit = max_model_len or model.max_positions or num_pages * page_size
+        self.fixed_max_blocks = min(-(-limit // page_size), max(1, num_pages))
+        self._graphs = {}
+        self._seen = {}
+        self._pinned = None
+        self._copied = None
+        self.graph_replays = 0
 
     @staticmethod
     def bytes_per_page(model: DecoderModel, page_size: int, dtype) -> int:
@@ -62,23 +73,77 @@ class ModelRunner:
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run the entries' tokens as one batch.  Pages for them must have been reserved
         (``manager.reserve``).  Returns float32 logits [wanted rows, vocab] in the order of the
-        entries and of their ``want``; afterwards the tokens count as cached."""
+        entries and of their ``want`` (valid until the next step); afterwards the tokens count
+        as cached."""
         entries = list(entries)
         if not entries:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
-        batch = StepBatch(entries, self.manager, self.act_dtype, self.device, self.model.vocab_size)
+        graphable = self.use_graphs and all(len(e.tokens) == 1 for e in entries) \
+            and all(len(t) <= self.fixed_max_blocks for e in entries for t in e.cache.tables)
+        batch = StepBatch(entries, self.manager, self.act_dtype, self.device, self.model.vocab_size,
+                          self.fixed_max_blocks if graphable else 0)
         if batch.T > self.max_num_batched_tokens:
             raise ValueError("the step holds %d tokens, max_num_batched_tokens is %d" % (batch.T, self.max_num_batched_tokens))
         if self.model.max_positions and batch.max_kv_len > self.model.max_positions:
             raise ValueError("a request would reach %d tokens, the model's positions end at %d"
                              % (batch.max_kv_len, self.model.max_positions))
         self.model.plan(batch)
-        batch.upload()
         self._reset_fresh_state(batch)
-        logits = self.model.forward(batch, self.storage)
+        if graphable:
+            logits = self._step_graph(batch)
+        else:
+            if self.device.type == "cuda":
+                self._upload(batch, None)
+            else:
+                batch.upload()
+            logits = self.model.forward(batch, self.storage)
         for e in entries:
             self.manager.commit(e.cache, len(e.tokens))
         self.steps_run += 1
+        return logits
+
+    # ---- metadata to the device ----------------------------------------------
+    def _upload(self, batch: StepBatch, dev_buf: Optional[torch.Tensor]) -> None:
+        """Pack the batch's arrays into pinned host memory and copy them with one transfer."""
+        _layout, total = batch.layout()
+        if self._pinned is None or self._pinned.numel() < total:
+            self._pinned = torch.empty(max(total, 1 << 16), dtype=torch.int32, pin_memory=True)
+            self._copied = None
+        if self._copied is not None:
+            self._copied.synchronize()          # the last transfer has read the pinned buffer
+        layout, total = batch.pack_into(self._pinned)
+        if dev_buf is None:
+            dev_buf = torch.empty(total, dtype=torch.int32, device=self.device)
+        dev_buf[:total].copy_(self._pinned[:total], non_blocking=True)
+        self._copied = torch.cuda.Event()
+        self._copied.record()
+        batch.bind_device(dev_buf, layout)
+
+    # ---- graphs -----------------------------------------------------------------
+    def _step_graph(self, batch: StepBatch) -> torch.Tensor:
+        key = batch.layout_key()
+        held = self._graphs.get(key)
+        if held is not None:
+            graph, dev_buf, logits = held
+            self._upload(batch, dev_buf)
+            graph.replay()
+            self.graph_replays += 1
+            return logits
+        if self._seen.get(key, 0) < 1:
+            # first step of this shape: run it kernel by kernel (this also warms the library up)
+            self._seen[key] = 1
+            self._upload(batch, None)
+            return self.model.forward(batch, self.storage)
+        _layout, total = batch.layout()
+        dev_buf = torch.empty(total, dtype=torch.int32, device=self.device)
+        self._upload(batch, dev_buf)
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(batch, self.storage)
+        self._graphs[key] = (graph, dev_buf, logits)
+        graph.replay()                          # capture launches nothing: this replay is the step
+        self.graph_replays += 1
         return logits
 
     def _reset_fresh_state(self, batch: StepBatch) -> None:

@@ -252,11 +252,13 @@ class AttentionMeta:
     Host-side: S, T, max_blocks, max_kv_len, max_q_len."""
 
     def __init__(self, cu_q, pos0, kv_len, block_table, token_entry, positions, S, T, max_blocks, max_kv_len, max_q_len,
-                 tiles=None, tiles_group=0, num_tiles=0):
+                 tiles=None, tiles_group=0, num_tiles=0, fixed_shape=False):
         self.cu_q, self.pos0, self.kv_len, self.block_table = cu_q, pos0, kv_len, block_table
         self.token_entry, self.positions = token_entry, positions
         self.S, self.T, self.max_blocks, self.max_kv_len, self.max_q_len = S, T, max_blocks, max_kv_len, max_q_len
         self.tiles, self.tiles_group, self.num_tiles = tiles, tiles_group, num_tiles
+        #: True: launch shapes must not depend on the requests' lengths (the step is captured in a graph)
+        self.fixed_shape = fixed_shape
 
 
 MFMA_ATTENTION = True      # False forces the plain kernel for bfloat16 too (used by tests)
@@ -301,7 +303,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         if meta.max_q_len == 1:
             # all single tokens: split the keys so that the chip is full, at least 64 keys a part
             want = max(1, DECODE_SPLIT_TARGET // max(1, meta.num_tiles * n_kv))
-            splits = max(1, min(want, -(-meta.max_kv_len // 64), 64))
+            by_len = 64 if meta.fixed_shape else -(-meta.max_kv_len // 64)
+            splits = max(1, min(want, by_len, 64))
         ws_floats = hip().lib.spy_attention_mfma_workspace(ctypes.c_int(meta.num_tiles), ctypes.c_int(n_kv), ctypes.c_int(d),
                                                            ctypes.c_int(splits))
         ws = torch.empty((max(1, ws_floats),), dtype=torch.float32, device=q.device)

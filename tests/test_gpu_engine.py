@@ -1,0 +1,232 @@
+"""The engine on the GPU: greedy generation through the entry point, graphs against eager steps,
+long decoding, the first tokens of a sequence, and a toy architecture with a stateful mixer that is
+registered, built and stepped without a change to the framework's files."""
+import dataclasses
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from tests import replay_cases as rc
+from tests.configs import INIT, TINY_A, TINY_B, TINY_C
+from tests.gpu_util import require_gpu
+from tests.plain.qwen3_plain import PlainQwen3
+
+pytestmark = pytest.mark.gpu
+TOL = {"float32": dict(atol=1e-4, rtol=1e-4), "bfloat16": dict(atol=8e-2, rtol=2e-2)}
+
+
+@pytest.fixture(scope="module")
+def folder_c(tmp_path_factory):
+    from spyinfer_amd.weights import write_random_model
+    return write_random_model(str(tmp_path_factory.mktemp("eng_c")), TINY_C, 61, torch.bfloat16, **INIT)
+
+
+@pytest.fixture(scope="module")
+def folder_a(tmp_path_factory):
+    from spyinfer_amd.weights import write_random_model
+    return write_random_model(str(tmp_path_factory.mktemp("eng_a")), TINY_A, 62, torch.bfloat16, **INIT)
+
+
+def prompts(vocab, lengths, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, vocab, (n,), generator=g).tolist() for n in lengths]
+
+
+@pytest.mark.parametrize("eager", [True, False])
+def test_greedy_float32_equals_plain(folder_a, eager):
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    require_gpu()
+    ps = prompts(256, [5, 17, 33, 60], 1)
+    plain = PlainQwen3(folder_a)
+    want = [plain.greedy(p, 16) for p in ps]
+    for opts in (dict(), dict(max_num_batched_tokens=24, num_kvcache_blocks=7)):
+        kw = dict(dtype="float32", max_model_len=128, num_kvcache_blocks=40, max_num_seqs=8, enforce_eager=eager)
+        kw.update(opts)
+        eng = LLMEngine(folder_a, **kw)
+        assert eng.generate(ps, SamplingParams(max_new_tokens=16, ignore_eos=True)) == want
+        if not eager:
+            assert eng.runner.graph_replays > 0
+        eng.runner.manager.check()
+
+
+def test_greedy_bfloat16_follows_plain(folder_a):
+    """bfloat16 may leave the plain tokens only where the plain logits nearly tie."""
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    require_gpu()
+    ps = prompts(256, [5, 17, 33, 60], 2)
+    plain = PlainQwen3(folder_a)
+    eng = LLMEngine(folder_a, dtype="bfloat16", max_model_len=128, num_kvcache_blocks=40, max_num_seqs=8)
+    got = eng.generate(ps, SamplingParams(max_new_tokens=16, ignore_eos=True))
+    same = 0
+    for p, g in zip(ps, got):
+        toks = list(p)
+        for t in g:
+            logits = plain.forward(toks)[-1]
+            best = int(torch.argmax(logits))
+            if t != best:
+                assert float(logits[best] - logits[t]) < 0.1, "a bfloat16 token differs where the plain logits are apart"
+                break
+            same += 1
+            toks.append(t)
+    assert same >= 40
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(folder_c, dtype):
+    """Decode steps from a captured graph, replayed many times with the program's own work between
+    them, give what eager steps give, step by step."""
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.runner import ModelRunner, load_model
+    dev = require_gpu()
+    model = load_model(folder_c, dtype, dev)
+    ps = prompts(331, [40, 3, 130], 3)
+    runs = []
+    for eager in (True, False):
+        runner = ModelRunner(model, dtype, dev, 16, 64, 4, enforce_eager=eager, max_model_len=320)
+        caches = [runner.manager.admit(i) for i in range(3)]
+        for c, p in zip(caches, ps):
+            runner.manager.reserve(c, len(p))
+        runner.step([StepEntry(c, p, []) for c, p in zip(caches, ps)])
+        g = torch.Generator().manual_seed(4)
+        outs = []
+        for i in range(40):
+            toks = torch.randint(0, 331, (3,), generator=g).tolist()
+            for c in caches:
+                runner.manager.reserve(c, 1)
+            outs.append(runner.step([StepEntry(c, [t], [0]) for c, t in zip(caches, toks)]).cpu().clone())
+            _ = torch.randn(1000, device=dev).sum().item()          # other work and a synchronisation between replays
+        runs.append(outs)
+        if not eager:
+            assert runner.graph_replays >= 38
+    # graph steps split the keys into a fixed number of parts, eager steps by length: in bfloat16 the two
+    # round differently, each within the distance that is allowed against the plain implementation
+    tol = TOL[dtype]
+    for i, (a, b) in enumerate(zip(*runs)):
+        assert torch.allclose(a, b, atol=tol["atol"], rtol=tol["rtol"]), "step %d: graph and eager differ by %g" % (i, (a - b).abs().max())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(folder_c, dtype, tmp_path):
+    require_gpu()
+    reqs = rc.random_requests(331, [500, 1, 2], seed=8)
+    plain = PlainQwen3(folder_c)
+    ref = {rid: plain.forward(t) for rid, t in reqs.items()}
+    steps = rc.bulk_tail(reqs, tail=480)                 # 20 tokens at once, then 480 one by one
+    rc.run_replay_inprocess(folder_c, dtype, str(tmp_path), steps, rc.max_live_tokens(steps))
+    got = rc.collect(str(tmp_path), steps, 331)
+    assert len(got) == 503
+    rc.compare(got, ref, what="long decoding " + dtype, **TOL[dtype])
+
+
+def test_temperature_through_entry_point(folder_a):
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    require_gpu()
+    ps = prompts(256, [9, 30], 5)
+    sp = SamplingParams(temperature=0.8, max_new_tokens=12, ignore_eos=True)
+    kw = dict(dtype="float32", max_model_len=128, num_kvcache_blocks=40, seed=3)
+    a = LLMEngine(folder_a, **kw).generate(ps, sp)
+    b = LLMEngine(folder_a, max_num_batched_tokens=8, **kw).generate(ps, sp)
+    assert a == b and a[0] != a[1]
+    greedy = LLMEngine(folder_a, **kw).generate(ps, SamplingParams(max_new_tokens=12, ignore_eos=True))
+    assert greedy != a
+
+
+# ---------------------------------------------------------------------------------------------
+# A toy architecture defined here: blocks whose mixer keeps a running mean of its inputs per
+# request (state of fixed size in a slot) beside ordinary attention blocks.
+
+def _toy_parts():
+    from spyinfer_amd.cache import FixedState
+    from spyinfer_amd.config import ModelConfig
+    from spyinfer_amd.models import DecoderModel, LayerCall
+    from spyinfer_amd.parts import GatedMLP, LMHead, PagedAttention, PreNormBlock, RMSNorm, RotaryEmbedding, TokenEmbedding
+    from spyinfer_amd.parts.base import Mixer
+    from spyinfer_amd.weights import WeightSpec
+
+    class RunningMean(Mixer):
+        """out[t] = gain * mean of the request's inputs up to t.  State: [H] sums and one count."""
+
+        def __init__(self, hidden):
+            self.hidden = hidden
+
+        def weight_specs(self, prefix):
+            return [WeightSpec(prefix + ".gain", (self.hidden,), "norm")]
+
+        def bind(self, prefix, weights):
+            self.gain = weights[prefix + ".gain"]
+
+        def cache_spec(self):
+            return FixedState((self.hidden + 1,), "float32")
+
+        def forward(self, x, batch, cache, store=True):
+            out = torch.empty_like(x)
+            cu = batch.host_cu_q
+            for s, e in enumerate(batch.entries):
+                st = cache.state[e.cache.slot]
+                xs = x[cu[s]:cu[s + 1]].float()
+                sums = torch.cumsum(xs, 0) + st[:self.hidden]
+                cnt = st[self.hidden] + torch.arange(1, xs.shape[0] + 1, device=x.device, dtype=torch.float32)
+                out[cu[s]:cu[s + 1]] = (sums / cnt[:, None] * self.gain.float()).to(x.dtype)
+                if store:
+                    st[:self.hidden] = sums[-1]
+                    st[self.hidden] = cnt[-1]
+            return out
+
+        def plan(self, batch):
+            batch.host_cu_q = [0] + list(np.cumsum(batch.lens))
+
+    @dataclasses.dataclass
+    class ToyConfig(ModelConfig):
+        hidden_size: int = 0
+        num_hidden_layers: int = 0
+        vocab_size: int = 0
+        intermediate_size: int = 0
+
+    def build(cfg):
+        emb = TokenEmbedding(cfg.vocab_size, cfg.hidden_size)
+        rope = RotaryEmbedding(16, 10000.0)
+        layers = []
+        for i in range(cfg.num_hidden_layers):
+            mixer = RunningMean(cfg.hidden_size) if i % 2 == 0 else PagedAttention(cfg.hidden_size, 4, 2, 16, rope, window=24)
+            layers.append(PreNormBlock(RMSNorm(cfg.hidden_size, 1e-5), mixer, RMSNorm(cfg.hidden_size, 1e-5),
+                                       GatedMLP(cfg.hidden_size, cfg.intermediate_size)))
+        # the run order names layer 1 twice (its weights run again with a cache of their own)
+        order = [LayerCall(0, 0), LayerCall(1, 1), LayerCall(2, 2), LayerCall(1, 3)]
+        return DecoderModel(cfg, emb, rope, layers, RMSNorm(cfg.hidden_size, 1e-5), LMHead(cfg.vocab_size, cfg.hidden_size, tied_to=emb),
+                            schedule=order, max_positions=512)
+
+    return ToyConfig, build
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_with_state(dtype, tmp_path):
+    from spyinfer_amd.config import register_architecture, unregister_architecture
+    from spyinfer_amd.weights import write_random_model
+    require_gpu()
+    ToyConfig, build = _toy_parts()
+    register_architecture("ToyRunningMeanLM", ToyConfig, build)
+    try:
+        cfg = dict(architectures=["ToyRunningMeanLM"], hidden_size=64, num_hidden_layers=3, vocab_size=97, intermediate_size=80)
+        folder = write_random_model(str(tmp_path / "toy"), cfg, 71, torch.bfloat16, **INIT)
+        reqs = rc.random_requests(97, [70, 9, 41, 120, 33], seed=9)
+        outs = {}
+        for mode in ("whole", "portions", "mixed"):
+            steps = getattr(rc, mode)(reqs)
+            out = str(tmp_path / mode)
+            rc.run_replay_inprocess(folder, dtype, out, steps, rc.max_live_tokens(steps))
+            outs[mode] = rc.collect(out, steps, 97)
+        tol = TOL[dtype]
+        for mode in ("portions", "mixed"):
+            for key, row in outs[mode].items():
+                assert np.allclose(row, outs["whole"][key], atol=tol["atol"], rtol=tol["rtol"]), (mode, key)
+        # the state matters: a request's logits differ from those of its second half alone
+        first = next(iter(reqs))
+        assert not np.allclose(outs["whole"][(first, 40)], outs["whole"][(first, 5)], atol=1e-3)
+    finally:
+        unregister_architecture("ToyRunningMeanLM")
