@@ -90,7 +90,7 @@ def main() -> int:
 
     def decode_run(batch, steps, warmup):
         """tokens/s, ms/step, mean context over the timed steps."""
-        ids = [eng.add_request(p, SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + 1, ignore_eos=True))
+        ids = [eng.add_request(p, SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + 64, ignore_eos=True))
                for p in prompts(batch, args.prompt_len)]
         while any(s.is_prefill or s.num_generated == 0 for s in (eng._sequences[i] for i in ids)):
             eng.step()                                                       # prompts, in portions under the budget

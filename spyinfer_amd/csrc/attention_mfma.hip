@@ -1,4 +1,5 @@
-// Paged attention on MFMA for bfloat16: one wave per (16-row tile, kv head, part of the keys).
+// Paged attention on MFMA for bfloat16: one block of AW waves per (16-row tile, kv head, part of
+// the keys); the waves take the part's 32-key blocks in turn and merge through LDS at the end.
 //
 // Rows of a tile are (token, query head of the kv head's group) pairs of one batch entry, token
 // major: row r -> token r / G, head hk * G + r % G.  So a decoded token fills G rows, a prompt
@@ -23,16 +24,20 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
 __device__ __forceinline__ bf16x8_t zero8() { return bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
 
+#define AW 4   // waves per block
+
 template <int DMAX>
-__global__ __launch_bounds__(64) void attention_mfma_kernel(
+__global__ __launch_bounds__(AW * 64) void attention_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
     int n_q, int n_kv, int d, float scale, int window, int splits, float* __restrict__ ws) {
     constexpr int KK = DMAX / 32;   // 32-wide chunks of the head dim for Q.K
     constexpr int DT = DMAX / 16;   // 16-row tiles of the head dim for P.V
+    extern __shared__ float lds[];   // (AW - 1) * (DT * 4 + 2) * 64 floats: the other waves' O, m, l
     const int tile = blockIdx.x, hk = blockIdx.y, sp = blockIdx.z;
-    const int lane = threadIdx.x, r16 = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: loops over it stay scalar
+    const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
     const int s = tile_entry[tile];
     const int row0 = tile_row0[tile];
     const int G = n_q / n_kv;
@@ -74,7 +79,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
     for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
-    for (int b = b_begin; b < b_end; ++b) {
+    for (int b = b_begin + wave; b < b_end; b += AW) {
         const int c0 = lo + 32 * b;
         // ---- S^T = K . Q^T ------------------------------------------------------------------
         const int key_a = c0 + 8 * (r16 >> 2) + (r16 & 3);      // tile a; tile b is key_a + 4 (same page: P % 8 == 0)
@@ -157,6 +162,38 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
 
+    // merge the waves of the block: wave 0 takes the others' (O, m, l) from LDS, lane for lane
+    {
+        constexpr int PER = DT * 4 + 2;
+        if (wave > 0) {
+            float* mine = lds + (size_t)(wave - 1) * PER * 64;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) mine[(dt * 4 + i) * 64 + lane] = acc[dt][i];
+            mine[(DT * 4) * 64 + lane] = m;
+            mine[(DT * 4 + 1) * 64 + lane] = l;
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 1; w < AW; ++w) {
+            const float* other = lds + (size_t)(w - 1) * PER * 64;
+            const float mo = other[(DT * 4) * 64 + lane];
+            const float lo_ = other[(DT * 4 + 1) * 64 + lane];
+            const float mn = fmaxf(m, mo);
+            if (mn == -INFINITY) continue;
+            const float a = (m == -INFINITY) ? 0.f : __expf(m - mn);
+            const float bsc = (mo == -INFINITY) ? 0.f : __expf(mo - mn);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[dt][i] = acc[dt][i] * a + other[(dt * 4 + i) * 64 + lane] * bsc;
+            l = l * a + lo_ * bsc;
+            m = mn;
+        }
+    }
+
     if (splits == 1) {
         if (!row_ok) return;
         const float inv = l > 0.f ? 1.0f / l : 0.f;
@@ -213,10 +250,10 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(bf16_t* __restrict
         inv_l[tid] = L > 0.f ? 1.0f / L : 0.f;
     }
     __syncthreads();
-    for (int e = tid; e < 16 * d; e += 256) {
+    const int valid = min(16, nrows - row0);
+    for (int e = tid; e < valid * d; e += 256) {
         const int r = e / d, dd = e - r * d;
         const int row = row0 + r;
-        if (row >= nrows) continue;
         float o = 0.f;
         for (int i = 0; i < splits; ++i) o += base[(size_t)i * (16 * (DMAX + 2)) + r * DMAX + dd] * wgt[i * 16 + r];
         const int tq = row / G, head = hk * G + row % G;
@@ -246,7 +283,7 @@ extern "C" int spy_attention_mfma(void* out, const void* q, const void* kc, cons
     const dim3 grid(num_tiles, n_kv, splits);
     const dim3 mgrid(num_tiles, n_kv);
 #define ATT_CASE(DM)                                                                                                          \
-    attention_mfma_kernel<DM><<<grid, 64, 0, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, P,    \
+    attention_mfma_kernel<DM><<<grid, AW * 64, (AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, P,    \
                                                    num_pages, cu_q, pos0, kv_len, block_table, max_blocks, tile_entry,        \
                                                    tile_row0, n_q, n_kv, d, scale, window, splits, ws);                       \
     if (splits > 1)                                                                                                           \

@@ -27,7 +27,30 @@ extern "C" int spy_embedding(float* out, const void* table, int table_dtype, con
 
 // ---------------------------------------------------------------------------------------------
 // x = resid[t] (+ delta[t]);  rows == null: resid[t] = x.  out[r] = (x / sqrt(mean(x^2) + eps)) * w
-template <typename TA, typename TW>
+// One block per row.  The row is read once and kept in registers (4 values per thread and pass,
+// up to NORM_PASSES passes); longer rows are read again for the second pass.
+#define NORM_PASSES 8
+template <typename TA> struct Vec4;
+template <> struct Vec4<float> {
+    typedef float4 type;
+    static __device__ __forceinline__ void load(const float* p, float* v) { const float4 t = *reinterpret_cast<const float4*>(p); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+    static __device__ __forceinline__ void store(float* p, const float* v) { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
+};
+template <> struct Vec4<bf16_t> {
+    static __device__ __forceinline__ void load(const bf16_t* p, float* v) {
+        const uint2 t = *reinterpret_cast<const uint2*>(p);
+        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, const float* v) {
+        uint2 t;
+        t.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+        t.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+        *reinterpret_cast<uint2*>(p) = t;
+    }
+};
+
+template <typename TA, typename TW, bool VEC>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restrict__ delta, const TW* __restrict__ w, float eps,
                                    TA* __restrict__ out, const int* __restrict__ rows, int T, int H) {
     __shared__ float red[16];
@@ -42,16 +65,52 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
     }
     float* x = resid + (size_t)t * H;
     const TA* dl = delta ? delta + (size_t)t * H : nullptr;
+    TA* o = out + (size_t)r * H;
+    const bool write_back = dl && !rows;
+    if (VEC) {
+        // H % 4 == 0 and 16-byte aligned rows (checked by the launcher); the row fits the register passes
+        float v[NORM_PASSES][4];
+        float ss = 0.f;
+#pragma unroll
+        for (int p = 0; p < NORM_PASSES; ++p) {
+            const int i = (p * blockDim.x + threadIdx.x) * 4;
+            if (i < H) {
+                Vec4<float>::load(x + i, v[p]);
+                if (dl) {
+                    float d4[4];
+                    Vec4<TA>::load(dl + i, d4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[p][e] += d4[e];
+                }
+                if (write_back) Vec4<float>::store(x + i, v[p]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ss += v[p][e] * v[p][e];
+            }
+        }
+        ss = block_sum(ss, red);
+        const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+        for (int p = 0; p < NORM_PASSES; ++p) {
+            const int i = (p * blockDim.x + threadIdx.x) * 4;
+            if (i < H) {
+                float w4[4], y[4];
+                Vec4<TW>::load(w + i, w4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) y[e] = (scale * v[p][e]) * w4[e];
+                Vec4<TA>::store(o + i, y);
+            }
+        }
+        return;
+    }
     float ss = 0.f;
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
         float v = x[i];
         if (dl) v += to_f32<TA>(dl[i]);
-        if (dl && !rows) x[i] = v;
+        if (write_back) x[i] = v;
         ss += v * v;
     }
     ss = block_sum(ss, red);
     const float scale = 1.0f / sqrtf(ss / (float)H + eps);
-    TA* o = out + (size_t)r * H;
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
         float v = x[i];
         if (dl && rows) v += to_f32<TA>(dl[i]);
@@ -62,9 +121,17 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TA* __restri
 extern "C" int spy_add_rmsnorm(float* resid, const void* delta, const void* w, int w_dtype, float eps, void* out, int out_dtype,
                                const int* rows, int n_out, int T, int H, hipStream_t st) {
     SPY_REQUIRE(n_out > 0 && T > 0 && H > 0, "spy_add_rmsnorm: empty operand");
-    const int threads = H >= 1024 ? 512 : 256;
-    SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW><<<n_out, threads, 0, st>>>(
-        resid, (const TA*)delta, (const TW*)w, eps, (TA*)out, rows, T, H))));
+    const int threads = H >= 2048 ? 256 : (H >= 512 ? 128 : 64);
+    const bool aligned = H % 4 == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)delta % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
+                         ((uintptr_t)out % 16) == 0;
+    const bool vec = aligned && H <= threads * 4 * NORM_PASSES;
+    if (vec) {
+        SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW, true><<<n_out, threads, 0, st>>>(
+            resid, (const TA*)delta, (const TW*)w, eps, (TA*)out, rows, T, H))));
+    } else {
+        SPY_DISPATCH(out_dtype, TA, SPY_DISPATCH(w_dtype, TW, (add_rmsnorm_kernel<TA, TW, false><<<n_out, 512, 0, st>>>(
+            resid, (const TA*)delta, (const TW*)w, eps, (TA*)out, rows, T, H))));
+    }
     SPY_CHECK_LAUNCH("spy_add_rmsnorm");
     return 0;
 }

@@ -25,7 +25,8 @@ template <int MT, int NT, int WAVES, typename TC>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                                  TC* __restrict__ C, int M, int N, int K) {
     __shared__ float red[(WAVES - 1) * NT * MT * 64 * 4];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // the wave index is the same in all lanes: keep it in a scalar register so that loops over it are scalar too
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int r = lane & 15, g = lane >> 4;
     const int n_base = blockIdx.x * (16 * NT);
     f32x4_t acc[NT][MT];
@@ -34,41 +35,90 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    const bf16_t* wrow[NT];
-    bool wok[NT];
+    // Rows beyond N or M are clamped to the last row: their products land in outputs that are
+    // never stored, and the main loop needs no per-lane predicates.  Addresses are a base that is
+    // the same in all lanes (it advances with the chunk) plus a 32-bit lane offset that never
+    // changes, so the loop recomputes no per-lane address.
+    const char* wbase = reinterpret_cast<const char*>(W) + (size_t)n_base * K * 2;
+    const char* xbase = reinterpret_cast<const char*>(X);
+    unsigned woff[NT], xoff[MT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        const int n = n_base + nt * 16 + r;
-        wok[nt] = n < N;
-        wrow[nt] = W + (size_t)(wok[nt] ? n : 0) * K;
-    }
-    const bf16_t* xrow[MT];
+    for (int nt = 0; nt < NT; ++nt) woff[nt] = (unsigned)(min(n_base + nt * 16 + r, N - 1) - n_base) * (unsigned)K * 2u + 16u * g;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) xoff[mt] = (unsigned)min(mt * 16 + r, M - 1) * (unsigned)K * 2u + 16u * g;
+    // lanes whose row of X does not exist load nothing (their columns of the result are not stored):
+    // with few rows most lanes of the X loads stay idle, which the memory pipeline notices
     bool xok[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int m = mt * 16 + r;
-        xok[mt] = m < M;
-        xrow[mt] = X + (size_t)(xok[mt] ? m : 0) * K;
-    }
+    for (int mt = 0; mt < MT; ++mt) xok[mt] = mt * 16 + r < M;
+    const bf16_t* wrow[NT];
+    const bf16_t* xrow[MT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) wrow[nt] = reinterpret_cast<const bf16_t*>(wbase + woff[nt]);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) xrow[mt] = reinterpret_cast<const bf16_t*>(xbase + xoff[mt]);
 
-    for (int kc = wave * SK_CHUNK; kc < K; kc += WAVES * SK_CHUNK) {
-        bf16x8_t a[NT][4], b[MT][4];
+    bf16x8_t a0[NT][4], b0[MT][4], a1[NT][4], b1[MT][4];
+#define SK_LOAD(A, B, CHUNK)                                                                         \
+    {                                                                                                \
+        const char* wb_ = wbase + (size_t)(CHUNK) * (SK_CHUNK * 2);                                  \
+        const char* xb_ = xbase + (size_t)(CHUNK) * (SK_CHUNK * 2);                                  \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                              \
+            _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                        \
+                A[nt][j] = *reinterpret_cast<const bf16x8_t*>(wb_ + woff[nt] + 64 * j);              \
+            _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                        \
+                B[mt][j] = load8(reinterpret_cast<const bf16_t*>(xb_ + xoff[mt] + 64 * j), xok[mt]); \
+        }                                                                                            \
+    }
+#define SK_MFMA(A, B, ACC)                                                                           \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                    \
+        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                            \
+            _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                        \
+                ACC[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[nt][j], B[mt][j], ACC[nt][mt], 0, 0, 0);
+
+    // Full chunks, two per round with accumulators of their own (added at the end).  The loop is
+    // kept this plain on purpose: a version that issued the next round's loads before this round's
+    // products was compiled into code that overwrote live registers.
+    f32x4_t acc2[NT][MT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc2[nt][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const int nfull = K / SK_CHUNK;
+    int c = wave;
+    for (; c + WAVES < nfull; c += 2 * WAVES) {     // two chunks of this wave per round: 8 loads of W per lane in flight
+        SK_LOAD(a0, b0, c)
+        SK_LOAD(a1, b1, c + WAVES)
+        SK_MFMA(a0, b0, acc)
+        SK_MFMA(a1, b1, acc2)
+    }
+    if (c < nfull) {
+        SK_LOAD(a0, b0, c)
+        SK_MFMA(a0, b0, acc)
+    }
+#undef SK_LOAD
+#undef SK_MFMA
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] += acc2[nt][mt];
+    // the rest of K (fewer than 128 values; K is a multiple of 8), by the wave whose turn it is
+    if (nfull * SK_CHUNK < K && wave == nfull % WAVES) {
+        const int kc = nfull * SK_CHUNK;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int k = kc + 32 * j + 8 * g;
-            const bool kok = k < K;          // K is a multiple of 8: a lane's 8 elements are all inside or all outside
+            const bool kok = kc + 32 * j + 8 * g < K;
+            bf16x8_t a[NT], b[MT];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) a[nt][j] = load8(wrow[nt] + k, kok && wok[nt]);
+            for (int nt = 0; nt < NT; ++nt) a[nt] = load8(wrow[nt] + kc + 32 * j, kok);
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) b[mt][j] = load8(xrow[mt] + k, kok && xok[mt]);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
+            for (int mt = 0; mt < MT; ++mt) b[mt] = load8(xrow[mt] + kc + 32 * j, kok && xok[mt]);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
-                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], b[mt][j], acc[nt][mt], 0, 0, 0);
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt], b[mt], acc[nt][mt], 0, 0, 0);
+        }
     }
 
     if (WAVES > 1) {
@@ -114,11 +164,20 @@ static void launch_skinny(const bf16_t* X, const bf16_t* W, void* C, int M, int 
 
 template <int MT, typename TC>
 static void pick_skinny(const bf16_t* X, const bf16_t* W, void* C, int M, int N, int K, hipStream_t st) {
-    const int tiles = (N + 15) / 16;
-    // many rows of W: two tiles per wave halve the traffic of X; few rows: more waves share K
-    if (tiles >= 2048 && MT <= 2) launch_skinny<MT, 2, 4, TC>(X, W, C, M, N, K, st);
-    else if (tiles >= 1024) launch_skinny<MT, 1, 4, TC>(X, W, C, M, N, K, st);
-    else launch_skinny<MT, 1, 8, TC>(X, W, C, M, N, K, st);
+    // Measured on MI355X at the Qwen3-8B shapes (N 4096..151936, K 4096..12288) with 1 and 8 rows:
+    // one 16-row tile per block and 8 waves sharing K was the best or within 3 % of it everywhere.
+    launch_skinny<MT, 1, 8, TC>(X, W, C, M, N, K, st);
+}
+
+// Explicit configuration, for tuning runs: MT = 1 only.
+extern "C" int spy_gemm_skinny_cfg(const void* X, const void* W, void* C, int M, int N, int K, int nt, int waves, hipStream_t st) {
+    SPY_REQUIRE(M > 0 && M <= 16 && K % 8 == 0, "spy_gemm_skinny_cfg: M <= 16 and K %% 8 == 0 expected");
+    const bf16_t* x = (const bf16_t*)X;
+    const bf16_t* w = (const bf16_t*)W;
+#define CFG(NT_, W_) if (nt == NT_ && waves == W_) { launch_skinny<1, NT_, W_, bf16_t>(x, w, C, M, N, K, st); SPY_CHECK_LAUNCH("cfg"); return 0; }
+    CFG(1, 2) CFG(1, 4) CFG(1, 8) CFG(1, 16) CFG(2, 2) CFG(2, 4) CFG(2, 8) CFG(2, 16) CFG(4, 2) CFG(4, 4) CFG(4, 8)
+#undef CFG
+    return spy_fail("spy_gemm_skinny_cfg: no such configuration");
 }
 
 extern "C" int spy_gemm_skinny(const void* X, const void* W, void* C, int c_dtype, int M, int N, int K, hipStream_t st) {

@@ -1,79 +1,146 @@
 // Token choice on the device: first maximum (greedy), or the inverse CDF of softmax(logits / T)
-// over ascending token ids at a given uniform number u.  One block per row of logits.
+// over ascending token ids at a given uniform number u.
+// Two kernels: (1) every row is cut into SM_CHUNKS contiguous chunks of ids, one block per chunk
+// finds the chunk's first maximum and, for T > 0, its sum of exp((x - chunk max) / T);
+// (2) one wave per row merges the chunks in id order, finds the chunk that holds u * total and
+// walks it.  All sums run over ascending ids, so the choice is a function of (logits, T, u) alone.
 #include "common.h"
 #include <math.h>
 
-#define SM_THREADS 1024
+#define SM_CHUNKS 64
+#define SM_THREADS 256
 
-__global__ __launch_bounds__(SM_THREADS) void sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
-                                                            const float* __restrict__ uniform, int* __restrict__ out, int V) {
-    __shared__ float red[16];
-    __shared__ float best_v[16];
-    __shared__ int best_i[16];
-    __shared__ float part[SM_THREADS];
-    __shared__ int chosen;
-    const int r = blockIdx.x, tid = threadIdx.x;
+__device__ __forceinline__ void better(float& v, int& i, float ov, int oi) {
+    // the greater value wins, on ties the lower id; an id is "unset" as INT_MAX; a NaN never wins
+    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+}
+
+__global__ __launch_bounds__(SM_THREADS) void sample_chunks_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                                                                   float* __restrict__ pmax, int* __restrict__ pidx,
+                                                                   float* __restrict__ psum, int V) {
+    __shared__ float sv[SM_THREADS / 64];
+    __shared__ int si[SM_THREADS / 64];
+    __shared__ float red[SM_THREADS / 64];
+    const int c = blockIdx.x, r = blockIdx.y, tid = threadIdx.x;
+    const int chunk = (V + SM_CHUNKS - 1) / SM_CHUNKS;
+    const int b = min(V, c * chunk), e = min(V, b + chunk);
     const float* x = logits + (size_t)r * V;
-    const float temp = temperature[r];
-    // each thread owns a contiguous run of ids, so that sums walk the ids in ascending order
-    const int chunk = (V + SM_THREADS - 1) / SM_THREADS;
-    const int b = min(V, tid * chunk), e = min(V, b + chunk);
     float mv = -INFINITY;
     int mi = 0x7fffffff;
-    for (int i = b; i < e; ++i) {
-        const float v = x[i];
-        if (v > mv || (mi == 0x7fffffff && !(v < mv))) { mv = v; mi = i; }   // first maximum; a NaN row still yields an id
-    }
-    // wave: keep the greater value, on ties the lower id
+    for (int i = b + tid; i < e; i += SM_THREADS) better(mv, mi, x[i], i);
     for (int o = 32; o > 0; o >>= 1) {
         const float ov = __shfl_xor(mv, o, 64);
         const int oi = __shfl_xor(mi, o, 64);
-        if (ov > mv || (ov == mv && oi < mi)) { mv = ov; mi = oi; }
+        better(mv, mi, ov, oi);
     }
-    if ((tid & 63) == 0) { best_v[tid >> 6] = mv; best_i[tid >> 6] = mi; }
+    if ((tid & 63) == 0) { sv[tid >> 6] = mv; si[tid >> 6] = mi; }
     __syncthreads();
-    mv = best_v[0]; mi = best_i[0];
-    for (int w = 1; w < SM_THREADS / 64; ++w)
-        if (best_v[w] > mv || (best_v[w] == mv && best_i[w] < mi)) { mv = best_v[w]; mi = best_i[w]; }
+    mv = sv[0]; mi = si[0];
+    for (int w = 1; w < SM_THREADS / 64; ++w) better(mv, mi, sv[w], si[w]);
+    const float temp = temperature[r];
+    float s = 0.f;
+    if (temp > 0.f && mi != 0x7fffffff) {
+        const float inv_t = 1.0f / temp;
+        for (int i = b + tid; i < e; i += SM_THREADS) s += expf((x[i] - mv) * inv_t);
+        s = block_sum(s, red);
+    }
+    if (tid == 0) {
+        pmax[r * SM_CHUNKS + c] = mv;
+        pidx[r * SM_CHUNKS + c] = mi;
+        psum[r * SM_CHUNKS + c] = s;
+    }
+}
+
+__global__ __launch_bounds__(64) void sample_pick_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                                                         const float* __restrict__ uniform, const float* __restrict__ pmax,
+                                                         const int* __restrict__ pidx, const float* __restrict__ psum,
+                                                         int* __restrict__ out, int V) {
+    __shared__ float mass[SM_CHUNKS];
+    __shared__ float lsum[64];
+    const int r = blockIdx.x, lane = threadIdx.x;
+    float mv = pmax[r * SM_CHUNKS + lane];
+    int mi = pidx[r * SM_CHUNKS + lane];
+    const float cmax = mv;
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(mv, o, 64);
+        const int oi = __shfl_xor(mi, o, 64);
+        better(mv, mi, ov, oi);
+    }
+    const int greedy = mi == 0x7fffffff ? 0 : mi;
+    const float temp = temperature[r];
     if (!(temp > 0.f)) {
-        if (tid == 0) out[r] = mi == 0x7fffffff ? 0 : mi;
+        if (lane == 0) out[r] = greedy;
         return;
     }
     const float inv_t = 1.0f / temp;
-    float s = 0.f;
-    for (int i = b; i < e; ++i) s += expf((x[i] - mv) * inv_t);
-    part[tid] = s;
-    const float total = block_sum(s, red);
-    if (tid == 0) chosen = -1;
+    // mass of each chunk relative to the row maximum
+    mass[lane] = (cmax == -INFINITY) ? 0.f : psum[r * SM_CHUNKS + lane] * expf((cmax - mv) * inv_t);
     __syncthreads();
+    float total = 0.f;
+    for (int c = 0; c < SM_CHUNKS; ++c) total += mass[c];
     const float target = uniform[r] * total;
-    // exclusive prefix of the per-thread sums, in id order (one wave scans the 1024 partial sums)
-    if (tid < 64) {
+    int chosen_chunk = -1;
+    float before = 0.f;
+    {
         float run = 0.f;
-        for (int i = 0; i < tid * (SM_THREADS / 64); ++i) run += part[i];   // prefix before this lane's 16 partials
-        for (int i = tid * (SM_THREADS / 64); i < (tid + 1) * (SM_THREADS / 64); ++i) {
-            const float nxt = run + part[i];
-            const int bi = min(V, i * chunk), ei = min(V, bi + chunk);
-            if (bi < ei && target >= run && target < nxt && chosen < 0) {
-                // this run of ids holds the target: walk it
-                float acc = run;
-                int pick = ei - 1;
-                for (int j = bi; j < ei; ++j) {
-                    acc += expf((x[j] - mv) * inv_t);
-                    if (target < acc) { pick = j; break; }
-                }
-                atomicCAS(&chosen, -1, pick);
-            }
+        for (int c = 0; c < SM_CHUNKS; ++c) {
+            const float nxt = run + mass[c];
+            if (chosen_chunk < 0 && mass[c] > 0.f && target < nxt) { chosen_chunk = c; before = run; }
             run = nxt;
         }
     }
+    if (chosen_chunk < 0) {          // rounding pushed the target to the very end: the row's maximum stands in
+        if (lane == 0) out[r] = greedy;
+        return;
+    }
+    const int chunk = (V + SM_CHUNKS - 1) / SM_CHUNKS;
+    const int b = min(V, chosen_chunk * chunk), e = min(V, b + chunk);
+    const float* x = logits + (size_t)r * V;
+    // every lane sums a contiguous run of the chunk, then the runs are walked in order
+    const int per = (e - b + 63) / 64;
+    const int lb = min(e, b + lane * per), le = min(e, lb + per);
+    float s = 0.f;
+    for (int i = lb; i < le; ++i) s += expf((x[i] - mv) * inv_t);
+    lsum[lane] = s;
     __syncthreads();
-    if (tid == 0) out[r] = chosen >= 0 ? chosen : (mi == 0x7fffffff ? 0 : mi);
+    if (lane == 0) {
+        float run = before;
+        int pick = -1, last_pos = -1;
+        for (int w = 0; w < 64 && pick < 0; ++w) {
+            const float nxt = run + lsum[w];
+            if (lsum[w] > 0.f) {
+                const int wb = min(e, b + w * per), we = min(e, wb + per);
+                if (target < nxt) {
+                    float acc = run;
+                    for (int i = wb; i < we; ++i) {
+                        const float p = expf((x[i] - mv) * inv_t);
+                        acc += p;
+                        if (p > 0.f) last_pos = i;
+                        if (target < acc) { pick = i; break; }
+                    }
+                    if (pick < 0) pick = last_pos;   // the run's sum and its walk rounded apart
+                } else {
+                    last_pos = we - 1;
+                }
+            }
+            run = nxt;
+        }
+        out[r] = pick >= 0 ? pick : (last_pos >= 0 ? last_pos : greedy);
+    }
 }
 
-extern "C" int spy_sample(const float* logits, const float* temperature, const float* uniform, int* out, int R, int V, hipStream_t st) {
+extern "C" int64_t spy_sample_workspace(int R) { return (int64_t)R * SM_CHUNKS * 3; }
+
+extern "C" int spy_sample(const float* logits, const float* temperature, const float* uniform, int* out, int R, int V, float* ws,
+                          hipStream_t st) {
     SPY_REQUIRE(R > 0 && V > 0, "spy_sample: empty operand");
-    sample_kernel<<<R, SM_THREADS, 0, st>>>(logits, temperature, uniform, out, V);
+    SPY_REQUIRE(R <= 65535, "spy_sample: too many rows");
+    SPY_REQUIRE(ws, "spy_sample: no workspace");
+    float* pmax = ws;
+    int* pidx = reinterpret_cast<int*>(ws + (size_t)R * SM_CHUNKS);
+    float* psum = ws + (size_t)2 * R * SM_CHUNKS;
+    sample_chunks_kernel<<<dim3(SM_CHUNKS, R), SM_THREADS, 0, st>>>(logits, temperature, pmax, pidx, psum, V);
+    sample_pick_kernel<<<R, 64, 0, st>>>(logits, temperature, uniform, pmax, pidx, psum, out, V);
     SPY_CHECK_LAUNCH("spy_sample");
     return 0;
 }

@@ -73,7 +73,7 @@ class _Hip:
         self.lib.spy_last_error.restype = ctypes.c_char_p
         for name in ("spy_embedding", "spy_add_rmsnorm", "spy_rmsnorm", "spy_gemm", "spy_qknorm_rope_store",
                      "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_swiglu",
-                     "spy_sample", "spy_gemm_skinny"):
+                     "spy_sample", "spy_sample_workspace", "spy_gemm_skinny"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: rebuild it (python -c 'import __graft_entry__ as g; g.build()')"
                                   % (self.lib._name, name))
@@ -262,7 +262,7 @@ class AttentionMeta:
 
 
 MFMA_ATTENTION = True      # False forces the plain kernel for bfloat16 too (used by tests)
-DECODE_SPLIT_TARGET = 1024  # waves wanted in flight when all entries are single tokens
+DECODE_SPLIT_TARGET = 768   # blocks (of 4 waves) wanted in flight when all entries are single tokens
 
 
 def mfma_attention_ok(dtype, d: int, page_size: int) -> bool:
@@ -301,10 +301,10 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                and tile_row0.shape == (meta.num_tiles,), "paged_attention: tile lists must be int32 [num_tiles]")
         splits = 1
         if meta.max_q_len == 1:
-            # all single tokens: split the keys so that the chip is full, at least 64 keys a part
+            # all single tokens: split the keys so that the chip is full; a block of 4 waves wants 128 keys at least
             want = max(1, DECODE_SPLIT_TARGET // max(1, meta.num_tiles * n_kv))
-            by_len = 64 if meta.fixed_shape else -(-meta.max_kv_len // 64)
-            splits = max(1, min(want, by_len, 64))
+            by_len = 16 if meta.fixed_shape else -(-meta.max_kv_len // 128)
+            splits = max(1, min(want, by_len, 16))
         ws_floats = hip().lib.spy_attention_mfma_workspace(ctypes.c_int(meta.num_tiles), ctypes.c_int(n_kv), ctypes.c_int(d),
                                                            ctypes.c_int(splits))
         ws = torch.empty((max(1, ws_floats),), dtype=torch.float32, device=q.device)
@@ -349,6 +349,7 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor) -> 
     _check(V > 0, "sample: empty vocabulary")
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     if R:
+        ws = torch.empty((hip().lib.spy_sample_workspace(ctypes.c_int(R)),), dtype=torch.float32, device=logits.device)
         hip().call("spy_sample", _ptr(logits), _ptr(temperature), _ptr(u), _ptr(out), ctypes.c_int(R), ctypes.c_int(V),
-                   _Hip.stream())
+                   _ptr(ws), _Hip.stream())
     return out
