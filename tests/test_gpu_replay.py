@@ -49,6 +49,50 @@ def test_replay_matches_plain(dtype, name, mode, models, tmp_path):
     rc.compare(got, ref, what="%s/%s/%s" % (name, mode, dtype), **TOL[dtype])
 
 
+@pytest.fixture(scope="module")
+def sharp_model(tmp_path_factory):
+    """Config C with the q and k norm weights scaled up, so that scores are large and the softmax is
+    peaked: single far keys carry most of the weight, and a key that is skipped, read from the wrong
+    page or masked by mistake changes the logits by far more than the tolerance."""
+    from safetensors.torch import load_file
+    from spyinfer_amd.weights import write_file, write_random_model
+    folder = write_random_model(str(tmp_path_factory.mktemp("model_sharp")), TINY_C, 77, torch.bfloat16, **INIT)
+    path = os.path.join(folder, "model.safetensors")
+    w = {k: v.clone() for k, v in load_file(path).items()}
+    for k in w:
+        if k.endswith("q_norm.weight") or k.endswith("k_norm.weight"):
+            w[k] = (w[k].float() * 2.0).to(torch.bfloat16)
+    write_file(path, w)
+    reqs = rc.random_requests(TINY_C["vocab_size"], [600, 333, 150, 420, 64, 257], seed=6)
+    plain = PlainQwen3(folder)
+    return folder, reqs, {rid: plain.forward(t) for rid, t in reqs.items()}
+
+
+def test_sharp_attention_is_really_sharp(sharp_model):
+    """The construction does what it says: in the plain model, dropping one far key changes logits visibly."""
+    folder, reqs, ref = sharp_model
+    plain = PlainQwen3(folder)
+    toks = reqs["r2"]
+    full = plain.forward(toks)[-1]
+    for drop in (1, 17, 75):                                # one key of 150 removed (later positions shift by one too)
+        cut = plain.forward(toks[:drop] + toks[drop + 1:])[-1]
+        assert (full - cut).abs().max() > 0.5
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", ["bulk_tail", "portions", "mixed"])
+def test_replay_with_sharp_attention_over_hundreds_of_keys(dtype, mode, sharp_model, tmp_path):
+    require_gpu()
+    folder, reqs, ref = sharp_model
+    steps = getattr(rc, mode)(reqs)
+    rc.run_replay_inprocess(folder, dtype, str(tmp_path), steps, rc.max_live_tokens(steps))
+    got = rc.collect(str(tmp_path), steps, TINY_C["vocab_size"])
+    # A peaked softmax amplifies the bfloat16 rounding of q and k: the CPU model of that rounding differs from
+    # the plain implementation by up to 0.14 here, a dropped key by more than 0.5 (test above).
+    tol = dict(TOL[dtype]) if dtype == "float32" else dict(atol=0.28, rtol=0.02)
+    rc.compare(got, ref, what="sharp/%s/%s" % (mode, dtype), **tol)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(dtype, models, tmp_path):
     """bin/trace_run as a user starts it: a process of its own, steps on standard input."""
