@@ -1,0 +1,249 @@
+// Paged attention on MFMA for entries with many query rows (prompt portions): a block of 4 waves
+// works on 128 rows of one entry and one kv head, 32 rows (two 16-row MFMA tiles) per wave.  Rows
+// are (token, query head of the group) pairs as in attention_mfma.hip.  Keys and values of 64 keys
+// at a time are gathered through the block table into LDS once per block (prefetched into
+// registers while the previous 64 keys are worked on) and shared by the 8 row tiles; every K and V
+// fragment that a wave reads from LDS serves both of its row tiles.
+//
+// MFMA arrangement as in attention_mfma.hip: S^T = K . Q^T in two tiles whose key order leaves
+// lane (q row, g) with the scores of 8 consecutive keys, which are exactly the 8 k-values that
+// lane must supply of P^T in O^T += V^T . P^T.  In LDS the keys of a 32-key half are stored in the
+// order the two S^T tiles read them (rows 0..15 tile a, 16..31 tile b), which makes the 16-byte
+// reads of 16 lanes hit 16 different bank groups.
+#include "common.h"
+#include <math.h>
+
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
+#define PF_WAVES 4
+#define PF_ROWS 128      // rows per block
+#define PF_KEYS 64       // keys staged per round
+
+__device__ __forceinline__ bf16x8_t pf_zero8() { return bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
+
+template <int DMAX>
+__global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+    int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
+    int n_q, int n_kv, int d, float scale, int window) {
+    constexpr int KK = DMAX / 32, DT = DMAX / 16;
+    constexpr int KLD = DMAX + 8;            // bf16 per staged key row
+    constexpr int VLD = PF_KEYS + 8;         // bf16 per staged value row (one head dim, 64 keys)
+    constexpr int NV = DMAX / 32;            // 16-byte vectors per thread and operand per round (64 keys * DMAX / 8 / 256)
+    __shared__ __attribute__((aligned(16))) bf16_t ks[PF_KEYS * KLD];
+    __shared__ __attribute__((aligned(16))) bf16_t vs[DMAX * VLD];
+
+    const int tile = blockIdx.x, hk = blockIdx.y;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    const int s = tile_entry[tile];
+    const int row0 = tile_row0[tile];
+    const int G = n_q / n_kv;
+    const int q0 = cu_q[s];
+    const int nrows = (cu_q[s + 1] - q0) * G;
+    const int p0 = pos0[s];
+    const int kvl = kv_len[s];
+    const int* bt = block_table + (size_t)s * max_blocks;
+    const int d8 = d >> 3;
+
+    // this lane's two query rows
+    bool row_ok[2];
+    int tq[2], head[2], pos[2], lo_row[2];
+    bf16x8_t bq[2][KK];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int row = row0 + 32 * wave + 16 * t + r16;
+        row_ok[t] = row < nrows;
+        tq[t] = row_ok[t] ? row / G : 0;
+        head[t] = hk * G + (row_ok[t] ? row % G : 0);
+        pos[t] = p0 + tq[t];
+        lo_row[t] = window > 0 ? max(0, pos[t] - window + 1) : 0;
+        const bf16_t* qp = q + ((size_t)(q0 + tq[t]) * n_q + head[t]) * d;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const int dofs = kk * 32 + 8 * g;
+            bq[t][kk] = (row_ok[t] && dofs < d) ? *reinterpret_cast<const bf16x8_t*>(qp + dofs) : pf_zero8();
+        }
+    }
+    // keys the block can see, and those this wave can see (wave-uniform)
+    const int blk_last_row = min(nrows, row0 + PF_ROWS) - 1;
+    const int hi = min(p0 + blk_last_row / G, kvl - 1);
+    int lo = window > 0 ? max(0, p0 + row0 / G - window + 1) : 0;
+    lo &= ~(PF_KEYS - 1);
+    const int nblk = hi >= lo ? (hi - lo) / PF_KEYS + 1 : 0;
+    const int w_first_row = row0 + 32 * wave;
+    const int w_last_row = min(nrows, w_first_row + 32) - 1;
+    const int w_hi = w_last_row >= w_first_row ? p0 + w_last_row / G : -1;               // last key any row of the wave reads
+    const int w_lo = window > 0 ? max(0, p0 + w_first_row / G - window + 1) : 0;           // first key any row of the wave reads
+
+    f32x4_t acc[2][DT];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[t][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+
+    bf16x8_t pk[NV], pv[NV];
+    // gather 64 keys' K and V into registers: vector v = tid + 256 i
+    //   K: key = v / d8, chunk = v % d8            (16 bytes of one key row)
+    //   V: kgrp = v % 8, dd = v / 8                (8 keys of one head dim)
+#define PF_PREFETCH(C0)                                                                                       \
+    _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                          \
+        const int v = tid + 256 * i;                                                                          \
+        pk[i] = pf_zero8();                                                                                   \
+        pv[i] = pf_zero8();                                                                                   \
+        if (v < PF_KEYS * d8) {                                                                               \
+            const int key = (C0) + v / d8, ch = v % d8;                                                       \
+            if (key < kvl) {                                                                                  \
+                const int page = bt[key / P];                                                                 \
+                if (page >= 0 && page < num_pages)                                                            \
+                    pk[i] = *reinterpret_cast<const bf16x8_t*>(kc + (((size_t)page * n_kv + hk) * P + key % P) * d + ch * 8); \
+            }                                                                                                 \
+            const int kg = v & 7, dd = v >> 3;                                                                \
+            const int key0 = (C0) + 8 * kg;                                                                   \
+            if (key0 < kvl) {                                                                                 \
+                const int page = bt[key0 / P];                                                                \
+                if (page >= 0 && page < num_pages) {                                                          \
+                    bf16x8_t x = *reinterpret_cast<const bf16x8_t*>(vc + (((size_t)page * n_kv + hk) * d + dd) * P + key0 % P); \
+                    const int valid = kvl - key0;      /* slots beyond the request's keys hold anything */     \
+                    if (valid < 8) { _Pragma("unroll") for (int j = 0; j < 8; ++j) if (j >= valid) x[j] = 0; } \
+                    pv[i] = x;                                                                                \
+                }                                                                                             \
+            }                                                                                                 \
+        }                                                                                                     \
+    }
+
+    if (nblk > 0) PF_PREFETCH(lo)
+    for (int b = 0; b < nblk; ++b) {
+        const int c0 = lo + PF_KEYS * b;
+        __syncthreads();                               // the previous round's readers are done
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int v = tid + 256 * i;
+            if (v < PF_KEYS * d8) {
+                const int key = v / d8, ch = v % d8;   // key local to the round, 0..63
+                const int k32 = key & 31;
+                // row order inside a 32-key half: tile a reads keys 8j + {0..3}, tile b keys 8j + {4..7}
+                const int rho = (key & 32) + (((k32 & 7) < 4) ? (4 * (k32 >> 3) + (k32 & 3)) : (16 + 4 * (k32 >> 3) + (k32 & 3)));
+                *reinterpret_cast<bf16x8_t*>(ks + rho * KLD + ch * 8) = pk[i];
+                const int kg = v & 7, dd = v >> 3;
+                *reinterpret_cast<bf16x8_t*>(vs + dd * VLD + 8 * kg) = pv[i];
+            }
+        }
+        __syncthreads();
+        if (b + 1 < nblk) PF_PREFETCH(c0 + PF_KEYS)
+
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int h0 = c0 + 32 * half;
+            if (h0 > w_hi || h0 + 31 < w_lo) continue;             // no row of this wave reads these keys (wave-uniform)
+            // ---- S^T = K . Q^T for both row tiles ------------------------------------------------
+            f32x4_t sa[2], sb[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) { sa[t] = f32x4_t{0.f, 0.f, 0.f, 0.f}; sb[t] = f32x4_t{0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                if (kk * 32 < d) {
+                    // columns at and beyond d were never staged: they must read as zero, not as what LDS held before
+                    const bool in_d = kk * 32 + 8 * g < d;
+                    const bf16x8_t ka = in_d ? *reinterpret_cast<const bf16x8_t*>(ks + (32 * half + r16) * KLD + kk * 32 + 8 * g) : pf_zero8();
+                    const bf16x8_t kb = in_d ? *reinterpret_cast<const bf16x8_t*>(ks + (32 * half + 16 + r16) * KLD + kk * 32 + 8 * g) : pf_zero8();
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        sa[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, bq[t][kk], sa[t], 0, 0, 0);
+                        sb[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, bq[t][kk], sb[t], 0, 0, 0);
+                    }
+                }
+            }
+            // ---- softmax: this lane has keys h0 + 8 g .. + 7 of its rows ----------------------------
+            bf16x8_t pb[2];
+            float alpha[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                float sc[8];
+                float bmax = -INFINITY;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int key = h0 + 8 * g + j;
+                    const float v = (j < 4 ? sa[t][j] : sb[t][j - 4]) * scale;
+                    const bool ok = row_ok[t] && key <= pos[t] && key >= lo_row[t] && key < kvl;
+                    sc[j] = ok ? v : -INFINITY;
+                    bmax = fmaxf(bmax, sc[j]);
+                }
+                bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
+                bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+                const float m_new = fmaxf(m[t], bmax);
+                alpha[t] = 1.f;
+                pb[t] = pf_zero8();
+                if (m_new != -INFINITY) {
+                    alpha[t] = (m[t] == -INFINITY) ? 0.f : __expf(m[t] - m_new);
+                    float psum = 0.f;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float pj = (sc[j] == -INFINITY) ? 0.f : __expf(sc[j] - m_new);
+                        psum += pj;
+                        pb[t][j] = (short)f32_to_bf16(pj);
+                    }
+                    l[t] = l[t] * alpha[t] + psum;
+                    m[t] = m_new;
+                }
+            }
+            // ---- O^T = O^T * alpha + V^T . P^T ---------------------------------------------------------
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                if (dt * 16 < d) {
+                    const bf16x8_t vt = *reinterpret_cast<const bf16x8_t*>(vs + (dt * 16 + r16) * VLD + 32 * half + 8 * g);
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        acc[t][dt] *= alpha[t];
+                        acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pb[t], acc[t][dt], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+#undef PF_PREFETCH
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        float lt = l[t];
+        lt += __shfl_xor(lt, 16, 64);
+        lt += __shfl_xor(lt, 32, 64);
+        if (!row_ok[t]) continue;
+        const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+        bf16_t* op = out + ((size_t)(q0 + tq[t]) * n_q + head[t]) * d;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const int dd = dt * 16 + 4 * g;
+            if (dd < d) {
+                uint2 w;
+                w.x = (uint32_t)f32_to_bf16(acc[t][dt][0] * inv) | ((uint32_t)f32_to_bf16(acc[t][dt][1] * inv) << 16);
+                w.y = (uint32_t)f32_to_bf16(acc[t][dt][2] * inv) | ((uint32_t)f32_to_bf16(acc[t][dt][3] * inv) << 16);
+                *reinterpret_cast<uint2*>(op + dd) = w;
+            }
+        }
+    }
+}
+
+extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, const void* vc, int P, int num_pages, const int* cu_q,
+                                     const int* pos0, const int* kv_len, const int* block_table, int max_blocks,
+                                     const int* tile_entry, const int* tile_row0, int num_tiles, int S, int T, int n_q, int n_kv,
+                                     int d, float scale, int window, hipStream_t st) {
+    SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
+                "spy_attention_prefill: empty operand");
+    SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "spy_attention_prefill: head_dim %d is not a multiple of 16 in 16..128", d);
+    SPY_REQUIRE(P % 8 == 0, "spy_attention_prefill: page size %d is not a multiple of 8", P);
+    SPY_REQUIRE(n_q % n_kv == 0, "spy_attention_prefill: n_q %d is not a multiple of n_kv %d", n_q, n_kv);
+    SPY_REQUIRE(n_kv <= 65535, "spy_attention_prefill: too many kv heads");
+    const dim3 grid(num_tiles, n_kv);
+#define PF_CASE(DM)                                                                                                              \
+    attention_prefill_kernel<DM><<<grid, PF_WAVES * 64, 0, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, \
+                                                                 P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,      \
+                                                                 tile_entry, tile_row0, n_q, n_kv, d, scale, window);
+    if (d <= 64) { PF_CASE(64) } else { PF_CASE(128) }
+#undef PF_CASE
+    SPY_CHECK_LAUNCH("spy_attention_prefill");
+    return 0;
+}

@@ -18,7 +18,9 @@ import torch
 from ..cache.manager import CacheManager, RequestCache
 from ..kernels.ops import AttentionMeta
 
-ROWS_PER_TILE = 16   # rows of (token, head-in-group) pairs that one attention wave works on
+ROWS_PER_TILE = 16        # rows of (token, head-in-group) pairs in a small attention tile
+ROWS_PER_BIG_TILE = 128   # rows in a tile of the prefill attention kernel
+BIG_MIN_ROWS = 64         # entries with at least this many rows go to the prefill kernel
 
 
 class StepEntry:
@@ -124,19 +126,25 @@ class StepBatch:
             raise RuntimeError("the batch is already on the device")
         self._arrays[name] = np.asarray(values, dtype=np.int32).reshape(-1)
 
-    def add_attention_tiles(self, group_size: int) -> None:
-        """16-row tiles over each entry's rows (token-major, head-in-group minor) for a
-        query-head group of ``group_size``."""
+    def add_attention_tiles(self, group_size: int, big_tiles: bool = True) -> None:
+        """Tiles over each entry's rows (token-major, head-in-group minor) for a query-head group of
+        ``group_size``: entries with at least BIG_MIN_ROWS rows are cut into 128-row tiles (the
+        LDS-sharing prefill kernel), the others into 16-row tiles (one block of waves each)."""
         if group_size in self._tiles:
             return
-        ntiles = (self.lens.astype(np.int64) * group_size + ROWS_PER_TILE - 1) // ROWS_PER_TILE
-        tile_entry = np.repeat(np.arange(self.S, dtype=np.int32), ntiles)
-        first = np.zeros(self.S + 1, dtype=np.int64)
-        np.cumsum(ntiles, out=first[1:])
-        tile_row0 = ((np.arange(int(first[-1]), dtype=np.int64) - first[:-1][tile_entry]) * ROWS_PER_TILE).astype(np.int32)
-        self._tiles[group_size] = int(first[-1])
-        self.add_array("tile_entry_%d" % group_size, tile_entry)
-        self.add_array("tile_row0_%d" % group_size, tile_row0)
+        rows = self.lens.astype(np.int64) * group_size
+        big = (rows >= BIG_MIN_ROWS) & bool(big_tiles)
+        counts = {}
+        for kind, size, mask in (("small", ROWS_PER_TILE, ~big), ("big", ROWS_PER_BIG_TILE, big)):
+            ntiles = np.where(mask, (rows + size - 1) // size, 0)
+            tile_entry = np.repeat(np.arange(self.S, dtype=np.int32), ntiles)
+            first = np.zeros(self.S + 1, dtype=np.int64)
+            np.cumsum(ntiles, out=first[1:])
+            tile_row0 = ((np.arange(int(first[-1]), dtype=np.int64) - first[:-1][tile_entry]) * size).astype(np.int32)
+            counts[kind] = int(first[-1])
+            self.add_array("tile_entry_%s_%d" % (kind, group_size), tile_entry)
+            self.add_array("tile_row0_%s_%d" % (kind, group_size), tile_row0)
+        self._tiles[group_size] = counts
 
     # ---- to the device -------------------------------------------------------
     def layout(self):
@@ -187,10 +195,11 @@ class StepBatch:
         return self._dev["block_table_%d" % group].view(self.S, self.max_blocks[group])
 
     def attention_meta(self, group: int, group_size: int) -> AttentionMeta:
-        tiles, n_tiles = None, 0
+        tiles = None
         if group_size in self._tiles:
-            tiles = (self._dev["tile_entry_%d" % group_size], self._dev["tile_row0_%d" % group_size])
-            n_tiles = self._tiles[group_size]
+            tiles = {}
+            for kind, n in self._tiles[group_size].items():
+                tiles[kind] = (self._dev["tile_entry_%s_%d" % (kind, group_size)], self._dev["tile_row0_%s_%d" % (kind, group_size)], n)
         return AttentionMeta(self._dev["cu_q"], self._dev["pos0"], self._dev["kv_len"], self.block_table(group),
                              self._dev["token_entry"], self._dev["positions"], self.S, self.T, self.max_blocks[group],
-                             self.max_kv_len, self.max_q_len, tiles, group_size, n_tiles, fixed_shape=self.fixed_shape)
+                             self.max_kv_len, self.max_q_len, tiles, group_size, fixed_shape=self.fixed_shape)

@@ -72,7 +72,8 @@ class _Hip:
         self.lib = _build.load()
         self.lib.spy_last_error.restype = ctypes.c_char_p
         for name in ("spy_embedding", "spy_add_rmsnorm", "spy_rmsnorm", "spy_gemm", "spy_qknorm_rope_store",
-                     "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_swiglu",
+                     "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_prefill",
+                     "spy_swiglu",
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: rebuild it (python -c 'import __graft_entry__ as g; g.build()')"
@@ -247,22 +248,31 @@ class AttentionMeta:
     kv_len [S]: keys the request has after this step (pos0 + tokens of the entry);
     block_table [S, max_blocks]: logical page -> physical page (-1 = none);
     token_entry [T], positions [T]: per query token.
-    tiles: (tile_entry [N], tile_row0 [N]) 16-row tiles of (token, head-in-group) rows per entry,
-    built for one group size ``tiles_group``; None if not built.
+    tiles: {"small": (tile_entry [N], tile_row0 [N], N), "big": (...)}: 16-row tiles of (token,
+    head-in-group) rows for entries with few rows and 128-row tiles for entries with many, built
+    for one group size ``tiles_group``; None if not built.
     Host-side: S, T, max_blocks, max_kv_len, max_q_len."""
 
     def __init__(self, cu_q, pos0, kv_len, block_table, token_entry, positions, S, T, max_blocks, max_kv_len, max_q_len,
-                 tiles=None, tiles_group=0, num_tiles=0, fixed_shape=False):
+                 tiles=None, tiles_group=0, fixed_shape=False):
         self.cu_q, self.pos0, self.kv_len, self.block_table = cu_q, pos0, kv_len, block_table
         self.token_entry, self.positions = token_entry, positions
         self.S, self.T, self.max_blocks, self.max_kv_len, self.max_q_len = S, T, max_blocks, max_kv_len, max_q_len
-        self.tiles, self.tiles_group, self.num_tiles = tiles, tiles_group, num_tiles
+        self.tiles, self.tiles_group = tiles, tiles_group
         #: True: launch shapes must not depend on the requests' lengths (the step is captured in a graph)
         self.fixed_shape = fixed_shape
 
 
 MFMA_ATTENTION = True      # False forces the plain kernel for bfloat16 too (used by tests)
 DECODE_SPLIT_TARGET = 768   # blocks (of 4 waves) wanted in flight when all entries are single tokens
+
+
+PREFILL_ATTENTION_MAX_HEAD_DIM = 128
+
+
+def prefill_attention_ok(d: int) -> bool:
+    """Whether entries with many rows may be cut into 128-row tiles for this head size."""
+    return d <= PREFILL_ATTENTION_MAX_HEAD_DIM
 
 
 def mfma_attention_ok(dtype, d: int, page_size: int) -> bool:
@@ -296,23 +306,35 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         return out
     group = n_q // n_kv
     if mfma_attention_ok(q.dtype, d, page_size) and meta.tiles is not None and meta.tiles_group == group:
-        tile_entry, tile_row0 = meta.tiles
-        _check(tile_entry.dtype == torch.int32 and tile_row0.dtype == torch.int32 and tile_entry.shape == (meta.num_tiles,)
-               and tile_row0.shape == (meta.num_tiles,), "paged_attention: tile lists must be int32 [num_tiles]")
-        splits = 1
-        if meta.max_q_len == 1:
-            # all single tokens: split the keys so that the chip is full; a block of 4 waves wants 128 keys at least
-            want = max(1, DECODE_SPLIT_TARGET // max(1, meta.num_tiles * n_kv))
-            by_len = 16 if meta.fixed_shape else -(-meta.max_kv_len // 128)
-            splits = max(1, min(want, by_len, 16))
-        ws_floats = hip().lib.spy_attention_mfma_workspace(ctypes.c_int(meta.num_tiles), ctypes.c_int(n_kv), ctypes.c_int(d),
-                                                           ctypes.c_int(splits))
-        ws = torch.empty((max(1, ws_floats),), dtype=torch.float32, device=q.device)
-        hip().call("spy_attention_mfma", _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), ctypes.c_int(page_size),
-                   ctypes.c_int(num_pages), _ptr(meta.cu_q), _ptr(meta.pos0), _ptr(meta.kv_len), _ptr(meta.block_table),
-                   ctypes.c_int(meta.max_blocks), _ptr(tile_entry), _ptr(tile_row0), ctypes.c_int(meta.num_tiles),
-                   ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d),
-                   ctypes.c_float(scale), ctypes.c_int(win), ctypes.c_int(splits), _ptr(ws), _Hip.stream())
+        small_entry, small_row0, n_small = meta.tiles["small"]
+        big_entry, big_row0, n_big = meta.tiles["big"]
+        for name, t, n in (("small tile entries", small_entry, n_small), ("small tile rows", small_row0, n_small),
+                           ("big tile entries", big_entry, n_big), ("big tile rows", big_row0, n_big)):
+            _check(t.dtype == torch.int32 and tuple(t.shape) == (n,), "paged_attention: %s must be int32 [%d]" % (name, n))
+        common = (ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(meta.cu_q), _ptr(meta.pos0), _ptr(meta.kv_len),
+                  _ptr(meta.block_table), ctypes.c_int(meta.max_blocks))
+        sizes = (ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d), ctypes.c_float(scale),
+                 ctypes.c_int(win))
+        if n_big and d > PREFILL_ATTENTION_MAX_HEAD_DIM:
+            # the LDS-sharing kernel stops at this head size: its tiles are re-cut into 16-row tiles on the host side of
+            # the batch only if asked; here they simply run through the general kernel, 8 small tiles each
+            raise KernelError("paged_attention: big tiles were built for head_dim %d; the batch must build small tiles "
+                              "(StepBatch does, via ops.prefill_attention_ok)" % d)
+        if n_big:
+            hip().call("spy_attention_prefill", _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), *common, _ptr(big_entry),
+                       _ptr(big_row0), ctypes.c_int(n_big), *sizes, _Hip.stream())
+        if n_small:
+            splits = 1
+            if meta.max_q_len == 1:
+                # all single tokens: split the keys so that the chip is full; a block of 4 waves wants 128 keys at least
+                want = max(1, DECODE_SPLIT_TARGET // max(1, n_small * n_kv))
+                by_len = 16 if meta.fixed_shape else -(-meta.max_kv_len // 128)
+                splits = max(1, min(want, by_len, 16))
+            ws_floats = hip().lib.spy_attention_mfma_workspace(ctypes.c_int(n_small), ctypes.c_int(n_kv), ctypes.c_int(d),
+                                                               ctypes.c_int(splits))
+            ws = torch.empty((max(1, ws_floats),), dtype=torch.float32, device=q.device)
+            hip().call("spy_attention_mfma", _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), *common, _ptr(small_entry),
+                       _ptr(small_row0), ctypes.c_int(n_small), *sizes, ctypes.c_int(splits), _ptr(ws), _Hip.stream())
         return out
     hip().call("spy_attention_generic", _ptr(out), _ptr(q), _code(q, "q"), _ptr(k_cache), _ptr(v_cache),
                ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(meta.kv_len), _ptr(meta.block_table),

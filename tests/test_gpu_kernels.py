@@ -239,13 +239,18 @@ def make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed, window=None,
                     gk = h * n_kv // n_q
                     kc[bt[s][c // P], gk, c % P, :] = (q[t].view(n_q, d)[h].float() * 1.5).to(dtype)
     G = n_q // n_kv
-    tile_entry, tile_row0 = [], []
-    for s, (a, n) in enumerate(entries):
-        for r0 in range(0, n * G, 16):
-            tile_entry.append(s); tile_row0.append(r0)
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    tiles = {}
+    for kind, size in (("small", 16), ("big", 128)):
+        tile_entry, tile_row0 = [], []
+        for s, (a, n) in enumerate(entries):
+            is_big = n * G >= 64 and d <= 128
+            if is_big == (kind == "big"):
+                for r0 in range(0, n * G, size):
+                    tile_entry.append(s); tile_row0.append(r0)
+        tiles[kind] = (i32(tile_entry), i32(tile_row0), len(tile_entry))
     meta = AttentionMeta(i32(cu), i32(pos0), i32(kvl), i32(bt), i32(te), i32(ps), len(entries), T, maxb, max(kvl),
-                         max(n for _, n in entries), (i32(tile_entry), i32(tile_row0)), G, len(tile_entry))
+                         max(n for _, n in entries), tiles, G)
     return q, kc, vc, bt, te, ps, meta
 
 
@@ -262,6 +267,9 @@ ATT_CASES = [
     (3, 1, 112, 4, [(0, 19), (30, 1)], 8),
     (32, 8, 128, 16, [(1151, 1), (70, 1), (2000, 1), (0, 1)], None),      # single tokens only: keys split into parts
     (6, 2, 96, 8, [(700, 1), (333, 1)], 100),
+    (16, 2, 64, 16, [(200, 100), (0, 3)], None),                            # a long portion that starts late: 800 rows
+    (4, 4, 96, 32, [(50, 90), (0, 257)], None),
+    (8, 2, 128, 8, [(0, 300), (64, 64), (500, 1)], 130),
 ]
 
 
