@@ -79,40 +79,58 @@ __global__ __launch_bounds__(AW * 64) void attention_mfma_kernel(
     for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
+    // Pages are looked up one block ahead, both lookups together, and a block's K and V loads are
+    // all issued before its first product: a block costs one memory round trip, not four.
+    int kpage = -1, vpage = -1;
+    {
+        const int c0 = lo + 32 * (b_begin + wave);
+        const int key_a = c0 + 8 * (r16 >> 2) + (r16 & 3), key_v = c0 + 8 * g;
+        if (b_begin + wave < b_end) {
+            if (key_a < kvl) kpage = bt[key_a / P];
+            if (key_v < kvl) vpage = bt[key_v / P];
+        }
+    }
     for (int b = b_begin + wave; b < b_end; b += AW) {
         const int c0 = lo + 32 * b;
-        // ---- S^T = K . Q^T ------------------------------------------------------------------
         const int key_a = c0 + 8 * (r16 >> 2) + (r16 & 3);      // tile a; tile b is key_a + 4 (same page: P % 8 == 0)
-        int kpage = -1;
-        if (key_a < kvl) kpage = bt[key_a / P];
+        const int key_v = c0 + 8 * g;                             // this lane's 8 keys of V
         const bool k_ok = kpage >= 0 && kpage < num_pages;
+        const bool v_ok = vpage >= 0 && vpage < num_pages;
         const bf16_t* kp = kc + (((size_t)(k_ok ? kpage : 0) * n_kv + hk) * P + key_a % P) * d;
-        f32x4_t sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+        const bf16_t* vp = vc + (((size_t)(v_ok ? vpage : 0) * n_kv + hk) * d) * P + key_v % P;
+        bf16x8_t ka[KK], kb[KK], vt[DT];
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
             const int dofs = kk * 32 + 8 * g;
-            bf16x8_t ka = zero8(), kb = zero8();
+            ka[kk] = zero8();
+            kb[kk] = zero8();
             if (k_ok && dofs < d) {
-                ka = *reinterpret_cast<const bf16x8_t*>(kp + dofs);
-                if (key_a + 4 < kvl) kb = *reinterpret_cast<const bf16x8_t*>(kp + 4 * d + dofs);
-            }
-            if (kk * 32 < d) {
-                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, bq[kk], sa, 0, 0, 0);
-                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, bq[kk], sb, 0, 0, 0);
+                ka[kk] = *reinterpret_cast<const bf16x8_t*>(kp + dofs);
+                if (key_a + 4 < kvl) kb[kk] = *reinterpret_cast<const bf16x8_t*>(kp + 4 * d + dofs);
             }
         }
-        // ---- V^T fragments (issued early; used after the softmax) ----------------------------
-        const int key_v = c0 + 8 * g;                             // this lane's 8 keys
-        int vpage = -1;
-        if (key_v < kvl) vpage = bt[key_v / P];
-        const bool v_ok = vpage >= 0 && vpage < num_pages;
-        const int v_valid = min(8, kvl - key_v);                  // keys of the group that exist (slots beyond hold anything)
-        const bf16_t* vp = vc + (((size_t)(v_ok ? vpage : 0) * n_kv + hk) * d) * P + key_v % P;
-        bf16x8_t vt[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             const int dd = dt * 16 + r16;
             vt[dt] = (v_ok && dd < d) ? *reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P) : zero8();
+        }
+        const int v_valid = min(8, kvl - key_v);                  // keys of the group that exist (slots beyond hold anything)
+        // the next block's pages
+        kpage = -1;
+        vpage = -1;
+        if (b + AW < b_end) {
+            const int na = key_a + 32 * AW, nv = key_v + 32 * AW;
+            if (na < kvl) kpage = bt[na / P];
+            if (nv < kvl) vpage = bt[nv / P];
+        }
+        // ---- S^T = K . Q^T ------------------------------------------------------------------
+        f32x4_t sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            if (kk * 32 < d) {
+                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kk], bq[kk], sa, 0, 0, 0);
+                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[kk], bq[kk], sb, 0, 0, 0);
+            }
         }
         if (v_ok && v_valid < 8) {
 #pragma unroll

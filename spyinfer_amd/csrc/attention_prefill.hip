@@ -27,7 +27,7 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
-    int n_q, int n_kv, int d, float scale, int window) {
+    int n_q, int n_kv, int d, float scale, int window, int log2p) {
     constexpr int KK = DMAX / 32, DT = DMAX / 16;
     constexpr int KLD = DMAX + 8;            // bf16 per staged key row
     constexpr int VLD = PF_KEYS + 8;         // bf16 per staged value row (one head dim, 64 keys)
@@ -35,7 +35,8 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     __shared__ __attribute__((aligned(16))) bf16_t ks[PF_KEYS * KLD];
     __shared__ __attribute__((aligned(16))) bf16_t vs[DMAX * VLD];
 
-    const int tile = blockIdx.x, hk = blockIdx.y;
+    // tiles late in a request see the most keys: they are started first, the short ones fill in behind them
+    const int tile = gridDim.x - 1 - blockIdx.x, hk = blockIdx.y;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
@@ -78,6 +79,10 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     const int w_last_row = min(nrows, w_first_row + 32) - 1;
     const int w_hi = w_last_row >= w_first_row ? p0 + w_last_row / G : -1;               // last key any row of the wave reads
     const int w_lo = window > 0 ? max(0, p0 + w_first_row / G - window + 1) : 0;           // first key any row of the wave reads
+    const bool w_rows_full = w_first_row + 31 < nrows;                                     // all 32 rows of the wave exist
+    const int w_min_pos = p0 + w_first_row / G;                                            // keys up to here are before every row
+    const int w_max_lo = window > 0 ? max(0, w_hi - window + 1) : 0;                       // keys from here on are in every window
+    const float scale2 = scale * 1.4426950408889634f;                                      // scores times log2(e)
 
     f32x4_t acc[2][DT];
 #pragma unroll
@@ -87,54 +92,74 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
 
     bf16x8_t pk[NV], pv[NV];
-    // gather 64 keys' K and V into registers: vector v = tid + 256 i
-    //   K: key = v / d8, chunk = v % d8            (16 bytes of one key row)
-    //   V: kgrp = v % 8, dd = v / 8                (8 keys of one head dim)
+    int kpg[NV], vpg[NV];        // pages of this thread's vectors, looked up one round ahead of the data
+    // vector v = tid + 256 i of a round:  K: key = v / d8, chunk = v % d8 (16 bytes of one key row)
+    //                                     V: kgrp = v % 8, dd = v / 8     (8 keys of one head dim)
+    // What does not change from round to round is worked out once: the local key, the offsets inside a
+    // page and the places in LDS.  Pages are powers of two here, so a key's page is a shift away.
+    int k_local[NV], k_goff[NV], v_goff[NV], k_lds[NV], v_lds[NV];
+    bool v_on[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = tid + 256 * i;
+        v_on[i] = v < PF_KEYS * d8;
+        const int key = v_on[i] ? v / d8 : 0, ch = v_on[i] ? v % d8 : 0;
+        k_local[i] = key;
+        k_goff[i] = ch * 8;
+        const int k32 = key & 31;
+        // row order inside a 32-key half: tile a reads keys 8j + {0..3}, tile b keys 8j + {4..7}
+        const int rho = (key & 32) + (((k32 & 7) < 4) ? (4 * (k32 >> 3) + (k32 & 3)) : (16 + 4 * (k32 >> 3) + (k32 & 3)));
+        k_lds[i] = rho * KLD + ch * 8;
+        const int kg = v & 7, dd = v >> 3;
+        v_goff[i] = dd * P;
+        v_lds[i] = dd * VLD + 8 * kg;
+    }
+    const int pmask = P - 1;
+    // The page lookups of a round are issued together and a round early, so that a round costs one
+    // memory round trip (the data), not one per vector.
+#define PF_PAGES(C0)                                                                                          \
+    _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                          \
+        const int key = (C0) + k_local[i], key0 = (C0) + 8 * ((tid + 256 * i) & 7);                           \
+        kpg[i] = (v_on[i] && key < kvl) ? bt[key >> log2p] : -1;                                              \
+        vpg[i] = (v_on[i] && key0 < kvl) ? bt[key0 >> log2p] : -1;                                            \
+    }
 #define PF_PREFETCH(C0)                                                                                       \
     _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                          \
-        const int v = tid + 256 * i;                                                                          \
+        const int key = (C0) + k_local[i], key0 = (C0) + 8 * ((tid + 256 * i) & 7);                           \
         pk[i] = pf_zero8();                                                                                   \
         pv[i] = pf_zero8();                                                                                   \
-        if (v < PF_KEYS * d8) {                                                                               \
-            const int key = (C0) + v / d8, ch = v % d8;                                                       \
-            if (key < kvl) {                                                                                  \
-                const int page = bt[key / P];                                                                 \
-                if (page >= 0 && page < num_pages)                                                            \
-                    pk[i] = *reinterpret_cast<const bf16x8_t*>(kc + (((size_t)page * n_kv + hk) * P + key % P) * d + ch * 8); \
-            }                                                                                                 \
-            const int kg = v & 7, dd = v >> 3;                                                                \
-            const int key0 = (C0) + 8 * kg;                                                                   \
-            if (key0 < kvl) {                                                                                 \
-                const int page = bt[key0 / P];                                                                \
-                if (page >= 0 && page < num_pages) {                                                          \
-                    bf16x8_t x = *reinterpret_cast<const bf16x8_t*>(vc + (((size_t)page * n_kv + hk) * d + dd) * P + key0 % P); \
-                    const int valid = kvl - key0;      /* slots beyond the request's keys hold anything */     \
-                    if (valid < 8) { _Pragma("unroll") for (int j = 0; j < 8; ++j) if (j >= valid) x[j] = 0; } \
-                    pv[i] = x;                                                                                \
-                }                                                                                             \
-            }                                                                                                 \
+        if (kpg[i] >= 0 && kpg[i] < num_pages)                                                                \
+            pk[i] = *reinterpret_cast<const bf16x8_t*>(kc + (((size_t)kpg[i] * n_kv + hk) * P + (key & pmask)) * d + k_goff[i]); \
+        if (vpg[i] >= 0 && vpg[i] < num_pages)                                                                \
+            pv[i] = *reinterpret_cast<const bf16x8_t*>(vc + ((size_t)vpg[i] * n_kv + hk) * d * P + v_goff[i] + (key0 & pmask)); \
+    }                                                                                                         \
+    if ((C0) + PF_KEYS > kvl) {                        /* slots beyond the request's keys hold anything */     \
+        _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                      \
+            const int valid = kvl - ((C0) + 8 * ((tid + 256 * i) & 7));                                       \
+            if (valid < 8) { _Pragma("unroll") for (int j = 0; j < 8; ++j) if (j >= valid) pv[i][j] = 0; }     \
         }                                                                                                     \
     }
 
-    if (nblk > 0) PF_PREFETCH(lo)
+    if (nblk > 0) {
+        PF_PAGES(lo)
+        PF_PREFETCH(lo)
+        PF_PAGES(lo + PF_KEYS)
+    }
     for (int b = 0; b < nblk; ++b) {
         const int c0 = lo + PF_KEYS * b;
         __syncthreads();                               // the previous round's readers are done
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const int v = tid + 256 * i;
-            if (v < PF_KEYS * d8) {
-                const int key = v / d8, ch = v % d8;   // key local to the round, 0..63
-                const int k32 = key & 31;
-                // row order inside a 32-key half: tile a reads keys 8j + {0..3}, tile b keys 8j + {4..7}
-                const int rho = (key & 32) + (((k32 & 7) < 4) ? (4 * (k32 >> 3) + (k32 & 3)) : (16 + 4 * (k32 >> 3) + (k32 & 3)));
-                *reinterpret_cast<bf16x8_t*>(ks + rho * KLD + ch * 8) = pk[i];
-                const int kg = v & 7, dd = v >> 3;
-                *reinterpret_cast<bf16x8_t*>(vs + dd * VLD + 8 * kg) = pv[i];
+            if (v_on[i]) {
+                *reinterpret_cast<bf16x8_t*>(ks + k_lds[i]) = pk[i];
+                *reinterpret_cast<bf16x8_t*>(vs + v_lds[i]) = pv[i];
             }
         }
         __syncthreads();
-        if (b + 1 < nblk) PF_PREFETCH(c0 + PF_KEYS)
+        if (b + 1 < nblk) {
+            PF_PREFETCH(c0 + PF_KEYS)
+            PF_PAGES(c0 + 2 * PF_KEYS)
+        }
 
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
@@ -158,54 +183,62 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
                     }
                 }
             }
-            // ---- softmax: this lane has keys h0 + 8 g .. + 7 of its rows ----------------------------
+            // ---- softmax: this lane has keys h0 + 8 g .. + 7 of its rows.  Scores are kept times log2(e),
+            // so that the exponentials are single v_exp_f32; the result does not change. ---------------------
+            // Most key blocks lie wholly before every row of the wave and inside every window: no masks then.
+            const bool unmasked = w_rows_full && h0 + 31 <= w_min_pos && h0 >= w_max_lo && h0 + 31 < kvl;
             bf16x8_t pb[2];
             float alpha[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 float sc[8];
-                float bmax = -INFINITY;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int key = h0 + 8 * g + j;
-                    const float v = (j < 4 ? sa[t][j] : sb[t][j - 4]) * scale;
-                    const bool ok = row_ok[t] && key <= pos[t] && key >= lo_row[t] && key < kvl;
-                    sc[j] = ok ? v : -INFINITY;
-                    bmax = fmaxf(bmax, sc[j]);
+                for (int j = 0; j < 8; ++j) sc[j] = (j < 4 ? sa[t][j] : sb[t][j - 4]) * scale2;
+                if (!unmasked) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const int key = h0 + 8 * g + j;
+                        const bool ok = row_ok[t] && key <= pos[t] && key >= lo_row[t] && key < kvl;
+                        sc[j] = ok ? sc[j] : -INFINITY;
+                    }
                 }
+                float bmax = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
                 bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
                 bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
                 const float m_new = fmaxf(m[t], bmax);
-                alpha[t] = 1.f;
-                pb[t] = pf_zero8();
-                if (m_new != -INFINITY) {
-                    alpha[t] = (m[t] == -INFINITY) ? 0.f : __expf(m[t] - m_new);
-                    float psum = 0.f;
+                // a row that has seen no key yet keeps m = -inf: subtract 0 then, every p is exp2(-inf) = 0
+                const float base = (m_new == -INFINITY) ? 0.f : m_new;
+                alpha[t] = __builtin_amdgcn_exp2f(m[t] - base);
+                float pj[8];
+                float psum = 0.f;
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const float pj = (sc[j] == -INFINITY) ? 0.f : __expf(sc[j] - m_new);
-                        psum += pj;
-                        pb[t][j] = (short)f32_to_bf16(pj);
-                    }
-                    l[t] = l[t] * alpha[t] + psum;
-                    m[t] = m_new;
+                for (int j = 0; j < 8; ++j) { pj[j] = __builtin_amdgcn_exp2f(sc[j] - base); psum += pj[j]; }
+                typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+                const u32x4_t packed = {pack_bf16x2(pj[0], pj[1]), pack_bf16x2(pj[2], pj[3]), pack_bf16x2(pj[4], pj[5]), pack_bf16x2(pj[6], pj[7])};
+                pb[t] = __builtin_bit_cast(bf16x8_t, packed);
+                l[t] = l[t] * alpha[t] + psum;
+                m[t] = m_new;
+            }
+            // ---- O^T = O^T * alpha + V^T . P^T (the rescale is skipped while no row's maximum moves) -------
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (__any(alpha[t] != 1.f)) {
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) acc[t][dt] *= alpha[t];
                 }
             }
-            // ---- O^T = O^T * alpha + V^T . P^T ---------------------------------------------------------
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 if (dt * 16 < d) {
                     const bf16x8_t vt = *reinterpret_cast<const bf16x8_t*>(vs + (dt * 16 + r16) * VLD + 32 * half + 8 * g);
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        acc[t][dt] *= alpha[t];
-                        acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pb[t], acc[t][dt], 0, 0, 0);
-                    }
+                    for (int t = 0; t < 2; ++t) acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pb[t], acc[t][dt], 0, 0, 0);
                 }
             }
         }
     }
 #undef PF_PREFETCH
+#undef PF_PAGES
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         float lt = l[t];
@@ -219,8 +252,8 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
             const int dd = dt * 16 + 4 * g;
             if (dd < d) {
                 uint2 w;
-                w.x = (uint32_t)f32_to_bf16(acc[t][dt][0] * inv) | ((uint32_t)f32_to_bf16(acc[t][dt][1] * inv) << 16);
-                w.y = (uint32_t)f32_to_bf16(acc[t][dt][2] * inv) | ((uint32_t)f32_to_bf16(acc[t][dt][3] * inv) << 16);
+                w.x = pack_bf16x2(acc[t][dt][0] * inv, acc[t][dt][1] * inv);
+                w.y = pack_bf16x2(acc[t][dt][2] * inv, acc[t][dt][3] * inv);
                 *reinterpret_cast<uint2*>(op + dd) = w;
             }
         }
@@ -234,14 +267,16 @@ extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, c
     SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
                 "spy_attention_prefill: empty operand");
     SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "spy_attention_prefill: head_dim %d is not a multiple of 16 in 16..128", d);
-    SPY_REQUIRE(P % 8 == 0, "spy_attention_prefill: page size %d is not a multiple of 8", P);
+    SPY_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "spy_attention_prefill: page size %d is not a power of two >= 8", P);
+    int log2p = 0;
+    while ((1 << log2p) < P) ++log2p;
     SPY_REQUIRE(n_q % n_kv == 0, "spy_attention_prefill: n_q %d is not a multiple of n_kv %d", n_q, n_kv);
     SPY_REQUIRE(n_kv <= 65535, "spy_attention_prefill: too many kv heads");
     const dim3 grid(num_tiles, n_kv);
 #define PF_CASE(DM)                                                                                                              \
     attention_prefill_kernel<DM><<<grid, PF_WAVES * 64, 0, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, \
                                                                  P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,      \
-                                                                 tile_entry, tile_row0, n_q, n_kv, d, scale, window);
+                                                                 tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p);
     if (d <= 64) { PF_CASE(64) } else { PF_CASE(128) }
 #undef PF_CASE
     SPY_CHECK_LAUNCH("spy_attention_prefill");

@@ -28,12 +28,15 @@ int spy_fail(const char* fmt, ...);   // records the message, returns 1
 
 __device__ __forceinline__ float bf16_to_f32(bf16_t x) { return __uint_as_float(((uint32_t)x) << 16); }
 
-// round to nearest, ties to even; NaN stays NaN
-__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
+// round to nearest, ties to even; NaN stays NaN.  gfx950 converts in hardware (v_cvt_pk_bf16_f32).
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) { return __builtin_bit_cast(unsigned short, (__bf16)f); }
+
+// two values in one instruction: a in the low half, b in the high half
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    typedef float f32x2_ __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_ __attribute__((ext_vector_type(2)));
+    const f32x2_ v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_));
 }
 
 template <typename T> __device__ __forceinline__ float to_f32(T x);

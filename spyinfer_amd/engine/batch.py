@@ -119,6 +119,7 @@ class StepBatch:
             self._arrays["block_table_%d" % g.index] = table.reshape(-1)
             self._arrays["slot_mapping_%d" % g.index] = (pages * P + positions % P).astype(np.int32)
         self.num_groups = len(manager.page_groups)
+        self.page_size = manager.page_size
 
     # ---- additions by parts, before upload ---------------------------------
     def add_array(self, name: str, values) -> None:

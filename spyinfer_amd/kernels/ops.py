@@ -270,9 +270,10 @@ DECODE_SPLIT_TARGET = 768   # blocks (of 4 waves) wanted in flight when all entr
 PREFILL_ATTENTION_MAX_HEAD_DIM = 128
 
 
-def prefill_attention_ok(d: int) -> bool:
-    """Whether entries with many rows may be cut into 128-row tiles for this head size."""
-    return d <= PREFILL_ATTENTION_MAX_HEAD_DIM
+def prefill_attention_ok(d: int, page_size: int) -> bool:
+    """Whether entries with many rows may be cut into 128-row tiles: the LDS-sharing kernel takes head
+    sizes up to 128 and pages of a power of two; other shapes run wholly through the general kernel."""
+    return d <= PREFILL_ATTENTION_MAX_HEAD_DIM and page_size >= 8 and page_size & (page_size - 1) == 0
 
 
 def mfma_attention_ok(dtype, d: int, page_size: int) -> bool:
@@ -315,11 +316,9 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                   _ptr(meta.block_table), ctypes.c_int(meta.max_blocks))
         sizes = (ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d), ctypes.c_float(scale),
                  ctypes.c_int(win))
-        if n_big and d > PREFILL_ATTENTION_MAX_HEAD_DIM:
-            # the LDS-sharing kernel stops at this head size: its tiles are re-cut into 16-row tiles on the host side of
-            # the batch only if asked; here they simply run through the general kernel, 8 small tiles each
-            raise KernelError("paged_attention: big tiles were built for head_dim %d; the batch must build small tiles "
-                              "(StepBatch does, via ops.prefill_attention_ok)" % d)
+        if n_big and not prefill_attention_ok(d, page_size):
+            raise KernelError("paged_attention: 128-row tiles were built for head_dim %d and pages of %d, which the prefill "
+                              "kernel refuses; build 16-row tiles only (ops.prefill_attention_ok)" % (d, page_size))
         if n_big:
             hip().call("spy_attention_prefill", _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), *common, _ptr(big_entry),
                        _ptr(big_row0), ctypes.c_int(n_big), *sizes, _Hip.stream())

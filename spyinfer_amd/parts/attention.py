@@ -61,7 +61,7 @@ class PagedAttention(Mixer):
         return PagedKV(self.num_kv_heads, self.head_dim, self.window)
 
     def plan(self, batch) -> None:
-        batch.add_attention_tiles(self.num_heads // self.num_kv_heads, ops.prefill_attention_ok(self.head_dim))
+        batch.add_attention_tiles(self.num_heads // self.num_kv_heads, ops.prefill_attention_ok(self.head_dim, batch.page_size))
 
     # ---- step ------------------------------------------------------------
     def forward(self, x, batch, cache, store=True):

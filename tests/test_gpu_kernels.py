@@ -244,7 +244,7 @@ def make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed, window=None,
     for kind, size in (("small", 16), ("big", 128)):
         tile_entry, tile_row0 = [], []
         for s, (a, n) in enumerate(entries):
-            is_big = n * G >= 64 and d <= 128
+            is_big = n * G >= 64 and d <= 128 and P & (P - 1) == 0
             if is_big == (kind == "big"):
                 for r0 in range(0, n * G, size):
                     tile_entry.append(s); tile_row0.append(r0)
