@@ -171,30 +171,53 @@ __global__ void swiglu_kernel(const TA* __restrict__ in, TA* __restrict__ out, i
     }
 }
 
+// the same, 4 values per thread and step with vector loads (I % 4 == 0, 16-byte aligned rows)
+template <typename TA>
+__global__ void swiglu_vec_kernel(const TA* __restrict__ in, TA* __restrict__ out, int T, int I4) {
+    const size_t n = (size_t)T * I4;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = idx / I4, i = (idx - t * I4) * 4;
+        const size_t I = (size_t)I4 * 4;
+        float g[4], u[4], y[4];
+        Vec4<TA>::load(in + t * 2 * I + i, g);
+        Vec4<TA>::load(in + t * 2 * I + I + i, u);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = (g[e] / (1.0f + expf(-g[e]))) * u[e];
+        Vec4<TA>::store(out + t * I + i, y);
+    }
+}
+
 extern "C" int spy_swiglu(const void* in, void* out, int dtype, int T, int I, hipStream_t st) {
     SPY_REQUIRE(T > 0 && I > 0, "spy_swiglu: empty operand");
-    const size_t n = (size_t)T * I;
+    const bool vec = I % 8 == 0 && ((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 16) == 0;
+    const size_t n = (size_t)T * I / (vec ? 4 : 1);
     const unsigned blocks = (unsigned)((n + 255) / 256 > 65536 ? 65536 : (n + 255) / 256);
-    SPY_DISPATCH(dtype, TA, swiglu_kernel<TA><<<blocks, 256, 0, st>>>((const TA*)in, (TA*)out, T, I));
+    if (vec) {
+        SPY_DISPATCH(dtype, TA, swiglu_vec_kernel<TA><<<blocks, 256, 0, st>>>((const TA*)in, (TA*)out, T, I / 4));
+    } else {
+        SPY_DISPATCH(dtype, TA, swiglu_kernel<TA><<<blocks, 256, 0, st>>>((const TA*)in, (TA*)out, T, I));
+    }
     SPY_CHECK_LAUNCH("spy_swiglu");
     return 0;
 }
 
 // ---------------------------------------------------------------------------------------------
-// One block (one wave) per (token, head of q|k|v).  q, k: optional RMS norm over the head, then
-// half-split rotation of the first `rot` dims: y[j] = x[j] c - x[j+rot/2] s; y[j+rot/2] = x[j] s + x[j+rot/2] c.
+// One wave per (token, head of q|k|v), QK_WAVES heads per block.  q, k: optional RMS norm over the head,
+// then half-split rotation of the first `rot` dims: y[j] = x[j] c - x[j+rot/2] s; y[j+rot/2] = x[j] s + x[j+rot/2] c.
+// A lane holds both members of its pairs, so the rotation needs no exchange between lanes.
 // q -> q_out[t, h, :];  k -> K[page, h, off, :];  v -> V[page, h, :, off]  (values lie transposed in a page).
 #define QK_MAX_D 512
+#define QK_WAVES 4
 template <typename TA, typename TW>
-__global__ void qknorm_rope_store_kernel(const TA* __restrict__ qkv, TA* __restrict__ q_out, int n_q, int n_kv, int d,
-                                         const TW* __restrict__ qw, const TW* __restrict__ kw, float eps,
-                                         const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, int max_pos,
-                                         const int* __restrict__ positions, TA* __restrict__ kc, TA* __restrict__ vc,
-                                         int P, int num_pages, const int* __restrict__ slots) {
-    __shared__ float y[QK_MAX_D];
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int width = (n_q + 2 * n_kv) * d;
-    const TA* x = qkv + (size_t)t * width + (size_t)h * d;
+__global__ __launch_bounds__(QK_WAVES * 64) void qknorm_rope_store_kernel(
+    const TA* __restrict__ qkv, TA* __restrict__ q_out, int n_q, int n_kv, int d, const TW* __restrict__ qw,
+    const TW* __restrict__ kw, float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, int max_pos,
+    const int* __restrict__ positions, TA* __restrict__ kc, TA* __restrict__ vc, int P, int num_pages, const int* __restrict__ slots) {
+    const int t = blockIdx.x, lane = threadIdx.x & 63;
+    const int h = blockIdx.y * QK_WAVES + (threadIdx.x >> 6);
+    const int heads = n_q + 2 * n_kv;
+    if (h >= heads) return;
+    const TA* x = qkv + (size_t)t * heads * d + (size_t)h * d;
     const bool is_q = h < n_q, is_k = !is_q && h < n_q + n_kv;
     int page = -1, off = 0;
     if (!is_q) {
@@ -210,31 +233,47 @@ __global__ void qknorm_rope_store_kernel(const TA* __restrict__ qkv, TA* __restr
         for (int j = lane; j < d; j += 64) dst[(size_t)j * P] = x[j];
         return;
     }
+    const int half = rot >> 1;
+    constexpr int NP = QK_MAX_D / 2 / 64;     // pairs per lane at most
+    float a[NP], b[NP], tail[NP * 2];
     float ss = 0.f;
-    for (int j = lane; j < d; j += 64) { const float v = to_f32<TA>(x[j]); y[j] = v; ss += v * v; }
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        const int j = lane + 64 * i;
+        a[i] = b[i] = 0.f;
+        if (j < half) { a[i] = to_f32<TA>(x[j]); b[i] = to_f32<TA>(x[j + half]); }
+        ss += a[i] * a[i] + b[i] * b[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NP * 2; ++i) {        // dims at and beyond rot are not rotated
+        const int j = rot + lane + 64 * i;
+        tail[i] = j < d ? to_f32<TA>(x[j]) : 0.f;
+        ss += tail[i] * tail[i];
+    }
     const TW* w = is_q ? qw : kw;
+    float scale = 1.f;
     if (w) {
         ss = wave_sum(ss);
-        const float scale = 1.0f / sqrtf(ss / (float)d + eps);
-        for (int j = lane; j < d; j += 64) y[j] = (scale * y[j]) * to_f32<TW>(w[j]);
+        scale = 1.0f / sqrtf(ss / (float)d + eps);
     }
-    __syncthreads();
     int p = positions[t];
     p = p < 0 ? 0 : (p >= max_pos && max_pos > 0 ? max_pos - 1 : p);
-    const int half = rot >> 1;
     TA* dst = is_q ? q_out + ((size_t)t * n_q + h) * d : kc + (((size_t)page * n_kv + (h - n_q)) * P + off) * d;
-    for (int j = lane; j < d; j += 64) {
-        float v;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        const int j = lane + 64 * i;
         if (j < half) {
+            float ya = a[i], yb = b[i];
+            if (w) { ya = (scale * ya) * to_f32<TW>(w[j]); yb = (scale * yb) * to_f32<TW>(w[j + half]); }
             const float c = cos_t[(size_t)p * half + j], s = sin_t[(size_t)p * half + j];
-            v = y[j] * c - y[j + half] * s;
-        } else if (j < rot) {
-            const float c = cos_t[(size_t)p * half + j - half], s = sin_t[(size_t)p * half + j - half];
-            v = y[j - half] * s + y[j] * c;
-        } else {
-            v = y[j];
+            dst[j] = from_f32<TA>(ya * c - yb * s);
+            dst[j + half] = from_f32<TA>(ya * s + yb * c);
         }
-        dst[j] = from_f32<TA>(v);
+    }
+#pragma unroll
+    for (int i = 0; i < NP * 2; ++i) {
+        const int j = rot + lane + 64 * i;
+        if (j < d) dst[j] = from_f32<TA>(w ? (scale * tail[i]) * to_f32<TW>(w[j]) : tail[i]);
     }
 }
 
@@ -247,10 +286,10 @@ extern "C" int spy_qknorm_rope_store(const void* qkv, int dtype, void* q_out, in
     SPY_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "spy_qknorm_rope_store: rotary_dim %d does not fit head_dim %d", rot, d);
     SPY_REQUIRE(rot == 0 || (cos_t && sin_t && max_pos > 0), "spy_qknorm_rope_store: rotation without tables");
     SPY_REQUIRE(!slots || (kc && vc && P > 0 && num_pages > 0), "spy_qknorm_rope_store: slots without a cache");
-    SPY_REQUIRE(n_q + 2 * n_kv <= 65535, "spy_qknorm_rope_store: too many heads");
-    const dim3 grid(T, n_q + 2 * n_kv);
+    SPY_REQUIRE(n_q + 2 * n_kv <= 65535 * QK_WAVES, "spy_qknorm_rope_store: too many heads");
+    const dim3 grid(T, (n_q + 2 * n_kv + QK_WAVES - 1) / QK_WAVES);
     const int wd = w_dtype < 0 ? SPY_F32 : w_dtype;
-    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(wd, TW, (qknorm_rope_store_kernel<TA, TW><<<grid, 64, 0, st>>>(
+    SPY_DISPATCH(dtype, TA, SPY_DISPATCH(wd, TW, (qknorm_rope_store_kernel<TA, TW><<<grid, QK_WAVES * 64, 0, st>>>(
         (const TA*)qkv, (TA*)q_out, n_q, n_kv, d, (const TW*)qw, (const TW*)kw, eps, cos_t, sin_t, rot, max_pos, positions,
         (TA*)kc, (TA*)vc, P, num_pages, slots))));
     SPY_CHECK_LAUNCH("spy_qknorm_rope_store");

@@ -21,14 +21,17 @@ __device__ __forceinline__ bf16x8_t load8(const bf16_t* p, bool ok) {
     return v;
 }
 
-template <int MT, int NT, int WAVES, typename TC>
+// GATED (with NT = 2): W holds [gate rows | up rows], N is the number of gate rows; tile 0 of a block is
+// 16 gate rows, tile 1 the 16 up rows of the same columns, and the block stores silu(gate) * up [M, N]:
+// the SwiGLU of a gated feed-forward without a pass of its own.
+template <int MT, int NT, int WAVES, typename TC, bool GATED = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                                  TC* __restrict__ C, int M, int N, int K) {
     __shared__ float red[(WAVES - 1) * NT * MT * 64 * 4];
     // the wave index is the same in all lanes: keep it in a scalar register so that loops over it are scalar too
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int r = lane & 15, g = lane >> 4;
-    const int n_base = blockIdx.x * (16 * NT);
+    const int n_base = GATED ? blockIdx.x * 16 : blockIdx.x * (16 * NT);
     f32x4_t acc[NT][MT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
@@ -43,7 +46,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
     const char* xbase = reinterpret_cast<const char*>(X);
     unsigned woff[NT], xoff[MT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) woff[nt] = (unsigned)(min(n_base + nt * 16 + r, N - 1) - n_base) * (unsigned)K * 2u + 16u * g;
+    for (int nt = 0; nt < NT; ++nt) {
+        const int row = GATED ? nt * N + min(n_base + r, N - 1) : min(n_base + nt * 16 + r, N - 1);
+        woff[nt] = (unsigned)(row - n_base) * (unsigned)K * 2u + 16u * g;
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) xoff[mt] = (unsigned)min(mt * 16 + r, M - 1) * (unsigned)K * 2u + 16u * g;
     // lanes whose row of X does not exist load nothing (their columns of the result are not stored):
@@ -142,6 +148,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 #pragma unroll
                     for (int i = 0; i < 4; ++i) acc[nt][mt][i] += red[((((w - 1) * NT + nt) * MT + mt) * 4 + i) * 64 + lane];
     }
+    if (GATED) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + r;
+            const int n = n_base + 4 * g;
+            if (m >= M) continue;
+            TC* out = C + (size_t)m * N + n;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float gt = acc[0][mt][i], up = acc[NT - 1][mt][i];
+                if (n + i < N) out[i] = from_f32<TC>((gt / (1.0f + expf(-gt))) * up);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -178,6 +199,22 @@ extern "C" int spy_gemm_skinny_cfg(const void* X, const void* W, void* C, int M,
     CFG(1, 2) CFG(1, 4) CFG(1, 8) CFG(1, 16) CFG(2, 2) CFG(2, 4) CFG(2, 8) CFG(2, 16) CFG(4, 2) CFG(4, 4) CFG(4, 8)
 #undef CFG
     return spy_fail("spy_gemm_skinny_cfg: no such configuration");
+}
+
+// out[M, I] = silu(X . Wgate^T) * (X . Wup^T) with W = [Wgate | Wup] stored [2 I, K]
+extern "C" int spy_gemm_skinny_swiglu(const void* X, const void* W, void* C, int c_dtype, int M, int I, int K, hipStream_t st) {
+    SPY_REQUIRE(M > 0 && I > 0 && K > 0, "spy_gemm_skinny_swiglu: empty operand");
+    SPY_REQUIRE(M <= 16, "spy_gemm_skinny_swiglu: M = %d exceeds 16 rows", M);
+    SPY_REQUIRE(K % 8 == 0, "spy_gemm_skinny_swiglu: K = %d is not a multiple of 8", K);
+    SPY_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0, "spy_gemm_skinny_swiglu: operands must be 16-byte aligned");
+    SPY_REQUIRE((long long)(I + 16) * K * 2 < (1ll << 32), "spy_gemm_skinny_swiglu: the gate and up rows lie too far apart");
+    const int blocks = (I + 15) / 16;
+    if (c_dtype == SPY_F32)
+        gemm_skinny_kernel<1, 2, 8, float, true><<<blocks, 8 * 64, 0, st>>>((const bf16_t*)X, (const bf16_t*)W, (float*)C, M, I, K);
+    else
+        gemm_skinny_kernel<1, 2, 8, bf16_t, true><<<blocks, 8 * 64, 0, st>>>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, I, K);
+    SPY_CHECK_LAUNCH("spy_gemm_skinny_swiglu");
+    return 0;
 }
 
 extern "C" int spy_gemm_skinny(const void* X, const void* W, void* C, int c_dtype, int M, int N, int K, hipStream_t st) {

@@ -74,7 +74,7 @@ class _Hip:
         for name in ("spy_embedding", "spy_add_rmsnorm", "spy_rmsnorm", "spy_gemm", "spy_qknorm_rope_store",
                      "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_prefill",
                      "spy_swiglu",
-                     "spy_sample", "spy_sample_workspace", "spy_gemm_skinny"):
+                     "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: rebuild it (python -c 'import __graft_entry__ as g; g.build()')"
                                   % (self.lib._name, name))
@@ -193,6 +193,25 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     hip().call("spy_gemm", _ptr(x), _code(x, "x"), _ptr(w), _code(w, "w"), _ptr(out), _code(out, "out"),
                ctypes.c_int(M), ctypes.c_int(N), ctypes.c_int(K), _Hip.stream())
     return out
+
+
+def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(x . Wgate^T) * (x . Wup^T) with ``w_gate_up [2 I, K]`` = [Wgate | Wup] -> [M, I].  For few bfloat16 rows
+    (decode) one kernel does both products and the SwiGLU; otherwise it is linear() followed by swiglu()."""
+    if _impl is not None:
+        return _impl.swiglu(_impl.linear(x, w_gate_up, None))
+    _dev(x, w_gate_up)
+    _check(x.dim() == 2 and w_gate_up.dim() == 2 and x.shape[1] == w_gate_up.shape[1] and w_gate_up.shape[0] % 2 == 0,
+           "linear_swiglu: x [M, K] and w [2 I, K] expected")
+    M, K = x.shape
+    I = w_gate_up.shape[0] // 2
+    if x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 \
+            and (I + 16) * K * 2 < (1 << 32):
+        out = torch.empty((M, I), dtype=x.dtype, device=x.device)
+        hip().call("spy_gemm_skinny_swiglu", _ptr(x), _ptr(w_gate_up), _ptr(out), _code(out, "out"), ctypes.c_int(M),
+                   ctypes.c_int(I), ctypes.c_int(K), _Hip.stream())
+        return out
+    return swiglu(linear(x, w_gate_up))
 
 
 def qk_norm_rope_store(qkv: torch.Tensor, n_q: int, n_kv: int, d: int, q_norm_w, k_norm_w, eps: float,

@@ -30,4 +30,4 @@ class GatedMLP(FeedForward):
         self.w_down = weights[prefix + ".down_proj.weight"]
 
     def forward(self, x, batch):
-        return ops.linear(ops.swiglu(ops.linear(x, self.w_gate_up)), self.w_down)
+        return ops.linear(ops.linear_swiglu(x, self.w_gate_up), self.w_down)

@@ -136,6 +136,21 @@ def test_swiglu(dtype):
     assert o[0] == 0 and abs(o[1] - 90) < 0.5 and abs(o[2]) < 1e-6
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,I,K", [(1, 160, 96), (7, 200, 88), (16, 1000, 1024), (8, 12288, 4096), (40, 128, 64), (3, 24, 20)])
+def test_linear_swiglu(dtype, M, I, K):
+    """Gate and up products with the SwiGLU in one call (one kernel for few bfloat16 rows)."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    x = rnd((M, K), dtype, dev, 15)
+    w = rnd((2 * I, K), dtype, dev, 16, 0.05)
+    y = x.double() @ w.double().t()
+    g, u = y[:, :I], y[:, I:]
+    out = ops.linear_swiglu(x, w)
+    assert out.shape == (M, I) and out.dtype == dtype
+    close(out, g / (1 + torch.exp(-g)) * u, dtype, scale=2.0, what="linear_swiglu")
+
+
 def plain_qk(qkv, n_q, n_kv, d, qw, kw, eps, theta, rot, pos):
     T = qkv.shape[0]
     x = qkv.double()
