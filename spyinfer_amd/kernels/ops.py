@@ -74,7 +74,8 @@ class _Hip:
         for name in ("spy_embedding", "spy_add_rmsnorm", "spy_rmsnorm", "spy_gemm", "spy_qknorm_rope_store",
                      "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_prefill",
                      "spy_swiglu",
-                     "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu"):
+                     "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
+                     "spy_gemm_skinny_tiled"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: rebuild it (python -c 'import __graft_entry__ as g; g.build()')"
                                   % (self.lib._name, name))
@@ -165,8 +166,28 @@ SKINNY_MAX_ROWS = 16
 SKINNY_MAX_ROWS_F32_OUT = 64
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+#: Keep a second copy of every bfloat16 weight matrix in MFMA tile order for the decode kernel (its loads are
+#: then whole cache lines).  Costs the weights' size again in device memory; the row-major copy stays for the
+#: library product of prefill.
+TILED_WEIGHTS = True
+
+
+def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
+    """``w [N, K]`` in the order the streaming MFMA kernel reads it: [N/16][K/32][g = 4][r = 16][8], the values
+    of lane 16 g + r being w[16 tile + r][32 step + 8 g ..].  None if the copy is switched off or the shape or
+    dtype does not allow it (then the kernel reads the row-major matrix)."""
+    if not TILED_WEIGHTS or _impl is not None or not w.is_cuda or w.dtype != torch.bfloat16 or w.dim() != 2:
+        return None
+    N, K = w.shape
+    if N % 16 or K % 128:
+        return None
+    return w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(N, K)
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y = x . w^T with w stored [N, K] (out_features, in_features), float32 accumulation.
+    ``tiled``: the same matrix from ``tile_weight``, used when few bfloat16 rows stream it.
 
     float32 anywhere among x and w -> the hand-written true-fp32 kernel.  All bfloat16: the streaming
     MFMA kernel for few rows, the library product for many."""
@@ -182,6 +203,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     if M == 0:
         return torch.empty((0, N), dtype=out_dtype, device=x.device)
     all_bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    if all_bf16 and tiled is not None and M <= 16:
+        _dev(tiled)
+        _check(tiled.shape == w.shape and tiled.dtype == w.dtype and N % 16 == 0 and K % 128 == 0,
+               "linear: the tiled copy does not fit the matrix")
+        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        hip().call("spy_gemm_skinny_tiled", _ptr(x), _ptr(tiled), _ptr(out), _code(out, "out"), ctypes.c_int(M), ctypes.c_int(N),
+                   ctypes.c_int(K), ctypes.c_int(0), _Hip.stream())
+        return out
     if all_bf16 and K % 8 == 0 and M <= (SKINNY_MAX_ROWS_F32_OUT if out_dtype == torch.float32 else SKINNY_MAX_ROWS):
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         hip().call("spy_gemm_skinny", _ptr(x), _ptr(w), _ptr(out), _code(out, "out"), ctypes.c_int(M), ctypes.c_int(N),
@@ -195,7 +224,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     return out
 
 
-def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """silu(x . Wgate^T) * (x . Wup^T) with ``w_gate_up [2 I, K]`` = [Wgate | Wup] -> [M, I].  For few bfloat16 rows
     (decode) one kernel does both products and the SwiGLU; otherwise it is linear() followed by swiglu()."""
     if _impl is not None:
@@ -205,6 +234,14 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
            "linear_swiglu: x [M, K] and w [2 I, K] expected")
     M, K = x.shape
     I = w_gate_up.shape[0] // 2
+    if x.dtype == torch.bfloat16 and tiled is not None and 0 < M <= 16 and I % 16 == 0 and K % 128 == 0 \
+            and (I + 16) * K * 2 < (1 << 32):
+        _dev(tiled)
+        _check(tiled.shape == w_gate_up.shape and tiled.dtype == torch.bfloat16, "linear_swiglu: the tiled copy does not fit")
+        out = torch.empty((M, I), dtype=x.dtype, device=x.device)
+        hip().call("spy_gemm_skinny_tiled", _ptr(x), _ptr(tiled), _ptr(out), _code(out, "out"), ctypes.c_int(M), ctypes.c_int(I),
+                   ctypes.c_int(K), ctypes.c_int(1), _Hip.stream())
+        return out
     if x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 \
             and (I + 16) * K * 2 < (1 << 32):
         out = torch.empty((M, I), dtype=x.dtype, device=x.device)
@@ -283,7 +320,7 @@ class AttentionMeta:
 
 
 MFMA_ATTENTION = True      # False forces the plain kernel for bfloat16 too (used by tests)
-DECODE_SPLIT_TARGET = 768   # blocks (of 4 waves) wanted in flight when all entries are single tokens
+DECODE_SPLIT_TARGET = 256   # blocks (of 4 waves) wanted in flight when all entries are single tokens (measured: B=8 best at 4 parts)
 
 
 PREFILL_ATTENTION_MAX_HEAD_DIM = 128

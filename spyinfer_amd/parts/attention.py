@@ -33,7 +33,7 @@ class PagedAttention(Mixer):
         self.qk_norm_eps = qk_norm_eps
         self.window = window
         self.scale = 1.0 / math.sqrt(head_dim) if scale is None else float(scale)
-        self.w_qkv = self.w_o = self.q_norm = self.k_norm = None
+        self.w_qkv = self.w_o = self.q_norm = self.k_norm = self.w_qkv_tiled = self.w_o_tiled = None
 
     # ---- weights ---------------------------------------------------------
     def weight_specs(self, prefix):
@@ -51,6 +51,7 @@ class PagedAttention(Mixer):
         # one product for q, k and v: rows [q heads | k heads | v heads]
         self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
         self.w_o = weights[prefix + ".o_proj.weight"]
+        self.w_qkv_tiled, self.w_o_tiled = ops.tile_weight(self.w_qkv), ops.tile_weight(self.w_o)
         if self.qk_norm_eps is not None:
             self.q_norm, self.k_norm = weights[prefix + ".q_norm.weight"], weights[prefix + ".k_norm.weight"]
             if self.q_norm.dtype != self.k_norm.dtype:
@@ -66,7 +67,7 @@ class PagedAttention(Mixer):
     # ---- step ------------------------------------------------------------
     def forward(self, x, batch, cache, store=True):
         nq, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
-        qkv = ops.linear(x, self.w_qkv)
+        qkv = ops.linear(x, self.w_qkv, tiled=self.w_qkv_tiled)
         rot = self.position.rotary() if self.position is not None else None
         cos, sin, rdim = rot if rot is not None else (None, None, 0)
         slots = batch.slot_mapping(cache.group) if store else None
@@ -75,4 +76,4 @@ class PagedAttention(Mixer):
                                    cos, sin, rdim, batch.positions, cache.k, cache.v, cache.page_size, slots)
         meta = batch.attention_meta(cache.group, nq // nkv)
         a = ops.paged_attention(q, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window)
-        return ops.linear(a, self.w_o)
+        return ops.linear(a, self.w_o, tiled=self.w_o_tiled)

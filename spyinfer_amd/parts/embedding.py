@@ -38,6 +38,7 @@ class LMHead(Part):
 
     def bind(self, prefix, weights):
         self.weight = self.tied_to.weight if self.tied_to is not None else weights[prefix + ".weight"]
+        self.weight_tiled = ops.tile_weight(self.weight)
 
     def forward(self, normed):
-        return ops.linear(normed, self.weight, torch.float32)
+        return ops.linear(normed, self.weight, torch.float32, tiled=self.weight_tiled)

@@ -15,7 +15,7 @@ class GatedMLP(FeedForward):
         if activation != "silu":
             raise ValueError("GatedMLP: activation %r is not implemented" % activation)
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
-        self.w_gate_up = self.w_down = None
+        self.w_gate_up = self.w_down = self.w_gate_up_tiled = self.w_down_tiled = None
 
     def weight_specs(self, prefix):
         H, I = self.hidden_size, self.intermediate_size
@@ -28,6 +28,9 @@ class GatedMLP(FeedForward):
             g, u = g.float(), u.float()
         self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
         self.w_down = weights[prefix + ".down_proj.weight"]
+        # tiles 0 .. I/16 - 1 of the tiled copy are gate rows, the rest up rows: what the fused SwiGLU kernel expects
+        self.w_gate_up_tiled = ops.tile_weight(self.w_gate_up) if self.intermediate_size % 16 == 0 else None
+        self.w_down_tiled = ops.tile_weight(self.w_down)
 
     def forward(self, x, batch):
-        return ops.linear(ops.linear_swiglu(x, self.w_gate_up), self.w_down)
+        return ops.linear(ops.linear_swiglu(x, self.w_gate_up, self.w_gate_up_tiled), self.w_down, tiled=self.w_down_tiled)

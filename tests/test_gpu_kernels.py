@@ -89,6 +89,28 @@ def test_linear(dtype, M, N, K):
               scale=math.sqrt(K) * 0.05, what="linear %s->%s" % (dtype, od))
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 16, 128), (8, 4096, 4096), (16, 160, 256), (5, 1024, 12288), (3, 151936, 512)])
+def test_linear_with_tiled_weights(M, N, K):
+    """The decode kernel reading the copy of W in MFMA tile order gives what it gives on the row-major matrix."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    x = rnd((M, K), torch.bfloat16, dev, 17)
+    w = rnd((N, K), torch.bfloat16, dev, 18, 0.05)
+    wt = ops.tile_weight(w)
+    assert wt is not None and wt.shape == w.shape
+    for od in (torch.bfloat16, torch.float32):
+        a, b = ops.linear(x, w, od, tiled=wt), ops.linear(x, w, od)
+        close(a, x.double() @ w.double().t(), torch.bfloat16, scale=1.0, what="tiled linear")
+        assert torch.allclose(a.float(), b.float(), atol=2e-2, rtol=2e-2)
+    if N % 32 == 0:
+        I = N // 2
+        y = x.double() @ w.double().t()
+        ref = y[:, :I] / (1 + torch.exp(-y[:, :I])) * y[:, I:]
+        if I % 16 == 0:
+            close(ops.linear_swiglu(x, w, wt), ref, torch.bfloat16, scale=2.0, what="tiled linear_swiglu")
+    assert ops.tile_weight(rnd((24, 128), torch.bfloat16, dev, 1)) is None and ops.tile_weight(rnd((32, 96), torch.bfloat16, dev, 1)) is None
+
+
 def test_linear_reference_vector():
     """test/test_linear.cpp:53-60 of the reference: x . W^T before the bias."""
     from spyinfer_amd.kernels import ops
