@@ -19,6 +19,8 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 #define PF_WAVES 4
 #define PF_ROWS 128      // rows per block
 #define PF_KEYS 64       // keys staged per round
+#define PF_SLACK 8.0f    // a score may exceed the running maximum by 2^8 before the maximum is raised
+#define PF_KG (PF_KEYS / 8)   // groups of 8 keys per round
 
 __device__ __forceinline__ bf16x8_t pf_zero8() { return bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
 
@@ -27,19 +29,25 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
-    int n_q, int n_kv, int d, float scale, int window, int log2p) {
+    int n_q, int n_kv, int d, float scale, int window, int log2p, int num_tiles) {
     constexpr int KK = DMAX / 32, DT = DMAX / 16;
     constexpr int KLD = DMAX + 8;            // bf16 per staged key row
     constexpr int VLD = PF_KEYS + 8;         // bf16 per staged value row (one head dim, 64 keys)
-    constexpr int NV = DMAX / 32;            // 16-byte vectors per thread and operand per round (64 keys * DMAX / 8 / 256)
+    constexpr int NV = PF_KEYS * DMAX / 8 / 256;   // 16-byte vectors per thread and operand per round
     __shared__ __attribute__((aligned(16))) bf16_t ks[PF_KEYS * KLD];
     __shared__ __attribute__((aligned(16))) bf16_t vs[DMAX * VLD];
 
-    // tiles late in a request see the most keys: they are started first, the short ones fill in behind them
-    const int tile = gridDim.x - 1 - blockIdx.x, hk = blockIdx.y;
+    // A block works on two tiles, one after the other: tile b and tile n - 1 - b of a list that the host
+    // has sorted by the number of keys a tile reads.  So every block has about the same work, which a
+    // causal prompt's tiles alone (few keys early, many late) do not give.
+    const int hk = blockIdx.y;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    for (int which = 0; which < 2; ++which) {
+    const int tile = which == 0 ? (int)blockIdx.x : num_tiles - 1 - (int)blockIdx.x;
+    if (which == 1 && tile <= (int)blockIdx.x) break;
+    __syncthreads();                                   // the first tile's last readers of LDS are done
     const int s = tile_entry[tile];
     const int row0 = tile_row0[tile];
     const int G = n_q / n_kv;
@@ -108,9 +116,9 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
         k_goff[i] = ch * 8;
         const int k32 = key & 31;
         // row order inside a 32-key half: tile a reads keys 8j + {0..3}, tile b keys 8j + {4..7}
-        const int rho = (key & 32) + (((k32 & 7) < 4) ? (4 * (k32 >> 3) + (k32 & 3)) : (16 + 4 * (k32 >> 3) + (k32 & 3)));
+        const int rho = (key & ~31) + (((k32 & 7) < 4) ? (4 * (k32 >> 3) + (k32 & 3)) : (16 + 4 * (k32 >> 3) + (k32 & 3)));
         k_lds[i] = rho * KLD + ch * 8;
-        const int kg = v & 7, dd = v >> 3;
+        const int kg = v % PF_KG, dd = v / PF_KG;
         v_goff[i] = dd * P;
         v_lds[i] = dd * VLD + 8 * kg;
     }
@@ -119,13 +127,13 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     // memory round trip (the data), not one per vector.
 #define PF_PAGES(C0)                                                                                          \
     _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                          \
-        const int key = (C0) + k_local[i], key0 = (C0) + 8 * ((tid + 256 * i) & 7);                           \
+        const int key = (C0) + k_local[i], key0 = (C0) + 8 * ((tid + 256 * i) % PF_KG);                       \
         kpg[i] = (v_on[i] && key < kvl) ? bt[key >> log2p] : -1;                                              \
         vpg[i] = (v_on[i] && key0 < kvl) ? bt[key0 >> log2p] : -1;                                            \
     }
 #define PF_PREFETCH(C0)                                                                                       \
     _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                          \
-        const int key = (C0) + k_local[i], key0 = (C0) + 8 * ((tid + 256 * i) & 7);                           \
+        const int key = (C0) + k_local[i], key0 = (C0) + 8 * ((tid + 256 * i) % PF_KG);                       \
         pk[i] = pf_zero8();                                                                                   \
         pv[i] = pf_zero8();                                                                                   \
         if (kpg[i] >= 0 && kpg[i] < num_pages)                                                                \
@@ -135,7 +143,7 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     }                                                                                                         \
     if ((C0) + PF_KEYS > kvl) {                        /* slots beyond the request's keys hold anything */     \
         _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                      \
-            const int valid = kvl - ((C0) + 8 * ((tid + 256 * i) & 7));                                       \
+            const int valid = kvl - ((C0) + 8 * ((tid + 256 * i) % PF_KG));                                   \
             if (valid < 8) { _Pragma("unroll") for (int j = 0; j < 8; ++j) if (j >= valid) pv[i][j] = 0; }     \
         }                                                                                                     \
     }
@@ -162,7 +170,7 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
         }
 
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
+        for (int half = 0; half < PF_KEYS / 32; ++half) {          // 32 keys at a time
             const int h0 = c0 + 32 * half;
             if (h0 > w_hi || h0 + 31 < w_lo) continue;             // no row of this wave reads these keys (wave-uniform)
             // ---- S^T = K . Q^T for both row tiles ------------------------------------------------
@@ -191,9 +199,9 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
             float alpha[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                float sc[8];
+                float sc[8];                          // raw scores; the scale goes into the exponent's fma
 #pragma unroll
-                for (int j = 0; j < 8; ++j) sc[j] = (j < 4 ? sa[t][j] : sb[t][j - 4]) * scale2;
+                for (int j = 0; j < 8; ++j) sc[j] = j < 4 ? sa[t][j] : sb[t][j - 4];
                 if (!unmasked) {
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
@@ -202,22 +210,29 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
                         sc[j] = ok ? sc[j] : -INFINITY;
                     }
                 }
-                float bmax = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-                bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
-                bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
-                const float m_new = fmaxf(m[t], bmax);
-                // a row that has seen no key yet keeps m = -inf: subtract 0 then, every p is exp2(-inf) = 0
-                const float base = (m_new == -INFINITY) ? 0.f : m_new;
-                alpha[t] = __builtin_amdgcn_exp2f(m[t] - base);
+                const float bmax = scale2 * fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+                // The running maximum m[t] (times log2 e) only has to bound the scores loosely: it is raised,
+                // for the whole wave at once, only when some score exceeds it by more than 2^PF_SLACK.  Most
+                // rounds then need neither the exchange between the four lanes of a row nor a rescale of O.
+                alpha[t] = 1.f;
+                if (__any(bmax > m[t] + PF_SLACK)) {
+                    float rmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
+                    rmax = fmaxf(rmax, __shfl_xor(rmax, 32, 64));
+                    const float m_new = fmaxf(m[t], rmax);
+                    // a row that has seen no key yet keeps m = -inf; its exponent base is 0 then (all its p are 0)
+                    alpha[t] = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m[t] - m_new);
+                    l[t] *= alpha[t];
+                    m[t] = m_new;
+                }
+                const float nbase = (m[t] == -INFINITY) ? 0.f : -m[t];
                 float pj[8];
                 float psum = 0.f;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) { pj[j] = __builtin_amdgcn_exp2f(sc[j] - base); psum += pj[j]; }
+                for (int j = 0; j < 8; ++j) { pj[j] = __builtin_amdgcn_exp2f(fmaf(sc[j], scale2, nbase)); psum += pj[j]; }
                 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
                 const u32x4_t packed = {pack_bf16x2(pj[0], pj[1]), pack_bf16x2(pj[2], pj[3]), pack_bf16x2(pj[4], pj[5]), pack_bf16x2(pj[6], pj[7])};
                 pb[t] = __builtin_bit_cast(bf16x8_t, packed);
-                l[t] = l[t] * alpha[t] + psum;
-                m[t] = m_new;
+                l[t] += psum;
             }
             // ---- O^T = O^T * alpha + V^T . P^T (the rescale is skipped while no row's maximum moves) -------
 #pragma unroll
@@ -258,6 +273,7 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
             }
         }
     }
+    }   // which
 }
 
 extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, const void* vc, int P, int num_pages, const int* cu_q,
@@ -272,11 +288,11 @@ extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, c
     while ((1 << log2p) < P) ++log2p;
     SPY_REQUIRE(n_q % n_kv == 0, "spy_attention_prefill: n_q %d is not a multiple of n_kv %d", n_q, n_kv);
     SPY_REQUIRE(n_kv <= 65535, "spy_attention_prefill: too many kv heads");
-    const dim3 grid(num_tiles, n_kv);
+    const dim3 grid((num_tiles + 1) / 2, n_kv);
 #define PF_CASE(DM)                                                                                                              \
     attention_prefill_kernel<DM><<<grid, PF_WAVES * 64, 0, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, \
                                                                  P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,      \
-                                                                 tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p);
+                                                                 tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p, num_tiles);
     if (d <= 64) { PF_CASE(64) } else { PF_CASE(128) }
 #undef PF_CASE
     SPY_CHECK_LAUNCH("spy_attention_prefill");

@@ -142,6 +142,12 @@ class StepBatch:
             first = np.zeros(self.S + 1, dtype=np.int64)
             np.cumsum(ntiles, out=first[1:])
             tile_row0 = ((np.arange(int(first[-1]), dtype=np.int64) - first[:-1][tile_entry]) * size).astype(np.int32)
+            if kind == "big" and tile_entry.shape[0] > 2:
+                # the prefill kernel gives a block the tiles b and n - 1 - b: sorted by the keys they read, blocks are even
+                pos0 = self._arrays["pos0"][tile_entry].astype(np.int64)
+                last_tok = np.minimum(self.lens[tile_entry].astype(np.int64), (tile_row0.astype(np.int64) + size + group_size - 1) // group_size)
+                order = np.argsort(-(pos0 + last_tok), kind="stable")
+                tile_entry, tile_row0 = tile_entry[order], tile_row0[order]
             counts[kind] = int(first[-1])
             self.add_array("tile_entry_%s_%d" % (kind, group_size), tile_entry)
             self.add_array("tile_row0_%s_%d" % (kind, group_size), tile_row0)

@@ -164,6 +164,7 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
 #: (logits) always come from the hand-written kernels, which keep the float32 sums.
 SKINNY_MAX_ROWS = 16
 SKINNY_MAX_ROWS_F32_OUT = 64
+_LIBRARY_F32_OUT = True      # torch.mm(..., out_dtype=float32) exists in this torch (float32 sums kept in the result)
 
 
 #: Keep a second copy of every bfloat16 weight matrix in MFMA tile order for the decode kernel (its loads are
@@ -211,6 +212,12 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         hip().call("spy_gemm_skinny_tiled", _ptr(x), _ptr(tiled), _ptr(out), _code(out, "out"), ctypes.c_int(M), ctypes.c_int(N),
                    ctypes.c_int(K), ctypes.c_int(0), _Hip.stream())
         return out
+    global _LIBRARY_F32_OUT
+    if all_bf16 and out_dtype == torch.float32 and M > SKINNY_MAX_ROWS and _LIBRARY_F32_OUT:
+        try:
+            return torch.mm(x, w.t(), out_dtype=torch.float32)      # logits of many rows: the library, float32 result
+        except TypeError:
+            _LIBRARY_F32_OUT = False
     if all_bf16 and K % 8 == 0 and M <= (SKINNY_MAX_ROWS_F32_OUT if out_dtype == torch.float32 else SKINNY_MAX_ROWS):
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         hip().call("spy_gemm_skinny", _ptr(x), _ptr(w), _ptr(out), _code(out, "out"), ctypes.c_int(M), ctypes.c_int(N),
