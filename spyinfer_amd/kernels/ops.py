@@ -386,12 +386,11 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             hip().call("spy_attention_prefill", _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), *common, _ptr(big_entry),
                        _ptr(big_row0), ctypes.c_int(n_big), *sizes, _Hip.stream())
         if n_small:
-            splits = 1
-            if meta.max_q_len == 1:
-                # all single tokens: split the keys so that the chip is full; a block of 4 waves wants 128 keys at least
-                want = max(1, DECODE_SPLIT_TARGET // max(1, n_small * n_kv))
-                by_len = 16 if meta.fixed_shape else -(-meta.max_kv_len // 128)
-                splits = max(1, min(want, by_len, 16))
+            # Few 16-row tiles cannot fill the chip by themselves (decoding requests, short portions): their keys are
+            # split into parts, each part a block of 4 waves that wants 128 keys at least, and a second kernel merges.
+            want = max(1, DECODE_SPLIT_TARGET // max(1, n_small * n_kv))
+            by_len = 16 if meta.fixed_shape else -(-meta.max_kv_len // 128)
+            splits = max(1, min(want, by_len, 16))
             ws_floats = hip().lib.spy_attention_mfma_workspace(ctypes.c_int(n_small), ctypes.c_int(n_kv), ctypes.c_int(d),
                                                                ctypes.c_int(splits))
             ws = torch.empty((max(1, ws_floats),), dtype=torch.float32, device=q.device)

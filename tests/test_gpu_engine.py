@@ -137,6 +137,30 @@ def test_temperature_through_entry_point(folder_a):
     assert greedy != a
 
 
+def test_command_line(folder_a, tmp_path):
+    """python -m spyinfer_amd -m MODEL --prompt-ids ...: the generated ids of each prompt on a line; and the
+    conversation loop with /new and /exit on standard input."""
+    import subprocess
+    import sys
+    require_gpu()
+    ps = prompts(256, [7, 21], 9)
+    plain = PlainQwen3(folder_a)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    base = [sys.executable, "-m", "spyinfer_amd", "-m", folder_a, "--dtype", "float32", "--max-model-len", "128",
+            "--num-kvcache-blocks", "32", "--max-new-tokens", "5", "--ignore-eos"]
+    cmd = base + sum((["--prompt-ids", " ".join(map(str, p))] for p in ps), [])
+    r = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.strip().splitlines() if l and l[0].isdigit()]
+    assert [[int(x) for x in l.split()] for l in lines] == [plain.greedy(p, 5) for p in ps]
+    talk = "%s\n/new\n%s\n/exit\n" % (",".join(map(str, ps[0])), " ".join(map(str, ps[1])))
+    r = subprocess.run(base, cwd=root, input=talk, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    answers = [l.split("Assistant:")[1].split() for l in r.stdout.splitlines() if "Assistant:" in l]
+    assert [[int(x) for x in a] for a in answers] == [plain.greedy(p, 5) for p in ps]
+    assert "Starting new conversation." in r.stdout
+
+
 # ---------------------------------------------------------------------------------------------
 # A toy architecture defined here: blocks whose mixer keeps a running mean of its inputs per
 # request (state of fixed size in a slot) beside ordinary attention blocks.
