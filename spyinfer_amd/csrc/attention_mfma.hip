@@ -19,6 +19,7 @@
 // (Letting the block that finishes last merge, found with a counter and device-scope fences, was
 // measured slower: 26 us against 17 us at 8 requests, because each fence writes back and invalidates L2.)
 #include "common.h"
+#include "attention_merge.h"
 #include <math.h>
 
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
@@ -243,44 +244,6 @@ __global__ __launch_bounds__(AW * 64) void attention_mfma_kernel(
     }
 }
 
-// Merge the parts of each (tile, kv head): O = sum_i O_i e^(m_i - M) / sum_i l_i e^(m_i - M).
-template <int DMAX>
-__global__ __launch_bounds__(256) void attention_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws,
-                                                              const int* __restrict__ cu_q, const int* __restrict__ tile_entry,
-                                                              const int* __restrict__ tile_row0, int n_q, int n_kv, int d, int splits) {
-    __shared__ float wgt[64 * 16];     // weight of part i for row r: [i][r], up to 64 parts
-    __shared__ float inv_l[16];
-    const int tile = blockIdx.x, hk = blockIdx.y, tid = threadIdx.x;
-    const int s = tile_entry[tile], row0 = tile_row0[tile];
-    const int G = n_q / n_kv;
-    const int q0 = cu_q[s];
-    const int nrows = (cu_q[s + 1] - q0) * G;
-    const float* base = ws + ((size_t)tile * n_kv + hk) * splits * (16 * (DMAX + 2));
-    if (tid < 16) {
-        float M = -INFINITY;
-        for (int i = 0; i < splits; ++i) M = fmaxf(M, base[(size_t)i * (16 * (DMAX + 2)) + 16 * DMAX + tid]);
-        float L = 0.f;
-        for (int i = 0; i < splits; ++i) {
-            const float* w = base + (size_t)i * (16 * (DMAX + 2));
-            const float mi = w[16 * DMAX + tid];
-            const float e = (mi == -INFINITY) ? 0.f : __expf(mi - M);
-            wgt[i * 16 + tid] = e;
-            L += w[16 * DMAX + 16 + tid] * e;
-        }
-        inv_l[tid] = L > 0.f ? 1.0f / L : 0.f;
-    }
-    __syncthreads();
-    const int valid = min(16, nrows - row0);
-    for (int e = tid; e < valid * d; e += 256) {
-        const int r = e / d, dd = e - r * d;
-        const int row = row0 + r;
-        float o = 0.f;
-        for (int i = 0; i < splits; ++i) o += base[(size_t)i * (16 * (DMAX + 2)) + r * DMAX + dd] * wgt[i * 16 + r];
-        const int tq = row / G, head = hk * G + row % G;
-        out[((size_t)(q0 + tq) * n_q + head) * d + dd] = f32_to_bf16(o * inv_l[r]);
-    }
-}
-
 static int dmax_of(int d) { return d <= 64 ? 64 : (d <= 128 ? 128 : 256); }
 
 extern "C" int64_t spy_attention_mfma_workspace(int num_tiles, int n_kv, int d, int splits) {
@@ -307,7 +270,7 @@ extern "C" int spy_attention_mfma(void* out, const void* q, const void* kc, cons
                                                    num_pages, cu_q, pos0, kv_len, block_table, max_blocks, tile_entry,        \
                                                    tile_row0, n_q, n_kv, d, scale, window, splits, ws);                       \
     if (splits > 1)                                                                                                           \
-        attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits);
+        attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits, 1);
     switch (dmax_of(d)) {
         case 64: ATT_CASE(64) break;
         case 128: ATT_CASE(128) break;

@@ -11,6 +11,7 @@
 // order the two S^T tiles read them (rows 0..15 tile a, 16..31 tile b), which makes the 16-byte
 // reads of 16 lanes hit 16 different bank groups.
 #include "common.h"
+#include "attention_merge.h"
 #include <math.h>
 
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
@@ -29,7 +30,7 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
-    int n_q, int n_kv, int d, float scale, int window, int log2p, int num_tiles) {
+    int n_q, int n_kv, int d, float scale, int window, int log2p, int num_tiles, int splits, float* __restrict__ ws) {
     constexpr int KK = DMAX / 32, DT = DMAX / 16;
     constexpr int KLD = DMAX + 8;            // bf16 per staged key row
     constexpr int VLD = PF_KEYS + 8;         // bf16 per staged value row (one head dim, 64 keys)
@@ -44,9 +45,12 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    // With key parts (splits > 1: few tiles, many keys, e.g. a late portion of a long prompt) a block has one
+    // tile and the rounds of one part; the parts are merged by attention_merge_kernel.
+    const int part = blockIdx.z;
     for (int which = 0; which < 2; ++which) {
     const int tile = which == 0 ? (int)blockIdx.x : num_tiles - 1 - (int)blockIdx.x;
-    if (which == 1 && tile <= (int)blockIdx.x) break;
+    if (which == 1 && (splits > 1 || tile <= (int)blockIdx.x)) break;
     __syncthreads();                                   // the first tile's last readers of LDS are done
     const int s = tile_entry[tile];
     const int row0 = tile_row0[tile];
@@ -148,12 +152,14 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
         }                                                                                                     \
     }
 
-    if (nblk > 0) {
-        PF_PAGES(lo)
-        PF_PREFETCH(lo)
-        PF_PAGES(lo + PF_KEYS)
+    const int per_part = (nblk + splits - 1) / splits;
+    const int b_first = part * per_part, b_last = min(nblk, b_first + per_part);
+    if (b_first < b_last) {
+        PF_PAGES(lo + PF_KEYS * b_first)
+        PF_PREFETCH(lo + PF_KEYS * b_first)
+        PF_PAGES(lo + PF_KEYS * (b_first + 1))
     }
-    for (int b = 0; b < nblk; ++b) {
+    for (int b = b_first; b < b_last; ++b) {
         const int c0 = lo + PF_KEYS * b;
         __syncthreads();                               // the previous round's readers are done
 #pragma unroll
@@ -164,7 +170,7 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
             }
         }
         __syncthreads();
-        if (b + 1 < nblk) {
+        if (b + 1 < b_last) {
             PF_PREFETCH(c0 + PF_KEYS)
             PF_PAGES(c0 + 2 * PF_KEYS)
         }
@@ -259,6 +265,18 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
         float lt = l[t];
         lt += __shfl_xor(lt, 16, 64);
         lt += __shfl_xor(lt, 32, 64);
+        if (splits > 1) {
+            // this part's share of the 16-row unit: O unnormalised, m back in the natural-log domain, l
+            const int unit = tile * (PF_ROWS / 16) + wave * 2 + t;
+            float* w = ws + (((size_t)unit * n_kv + hk) * splits + part) * (16 * (DMAX + 2));
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4_t*>(w + r16 * DMAX + dt * 16 + 4 * g) = acc[t][dt];
+            if (g == 0) {
+                w[16 * DMAX + r16] = m[t] * 0.6931471805599453f;
+                w[16 * DMAX + 16 + r16] = lt;
+            }
+            continue;
+        }
         if (!row_ok[t]) continue;
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
         bf16_t* op = out + ((size_t)(q0 + tq[t]) * n_q + head[t]) * d;
@@ -276,10 +294,15 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     }   // which
 }
 
+extern "C" int64_t spy_attention_prefill_workspace(int num_tiles, int n_kv, int d, int splits) {
+    if (splits <= 1) return 0;
+    return (int64_t)num_tiles * (PF_ROWS / 16) * n_kv * splits * 16 * ((d <= 64 ? 64 : 128) + 2);
+}
+
 extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, const void* vc, int P, int num_pages, const int* cu_q,
                                      const int* pos0, const int* kv_len, const int* block_table, int max_blocks,
                                      const int* tile_entry, const int* tile_row0, int num_tiles, int S, int T, int n_q, int n_kv,
-                                     int d, float scale, int window, hipStream_t st) {
+                                     int d, float scale, int window, int splits, float* ws, hipStream_t st) {
     SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
                 "spy_attention_prefill: empty operand");
     SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "spy_attention_prefill: head_dim %d is not a multiple of 16 in 16..128", d);
@@ -288,11 +311,18 @@ extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, c
     while ((1 << log2p) < P) ++log2p;
     SPY_REQUIRE(n_q % n_kv == 0, "spy_attention_prefill: n_q %d is not a multiple of n_kv %d", n_q, n_kv);
     SPY_REQUIRE(n_kv <= 65535, "spy_attention_prefill: too many kv heads");
-    const dim3 grid((num_tiles + 1) / 2, n_kv);
+    SPY_REQUIRE(splits >= 1 && splits <= 16, "spy_attention_prefill: %d key parts (1..16 allowed)", splits);
+    SPY_REQUIRE(splits == 1 || ws, "spy_attention_prefill: key parts without a workspace");
+    const dim3 grid(splits > 1 ? num_tiles : (num_tiles + 1) / 2, n_kv, splits);
+    const dim3 mgrid(num_tiles * (PF_ROWS / 16), n_kv);
 #define PF_CASE(DM)                                                                                                              \
     attention_prefill_kernel<DM><<<grid, PF_WAVES * 64, 0, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, \
                                                                  P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,      \
-                                                                 tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p, num_tiles);
+                                                                 tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p,      \
+                                                                 num_tiles, splits, ws);                                         \
+    if (splits > 1)                                                                                                              \
+        attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits,    \
+                                                          PF_ROWS / 16);
     if (d <= 64) { PF_CASE(64) } else { PF_CASE(128) }
 #undef PF_CASE
     SPY_CHECK_LAUNCH("spy_attention_prefill");

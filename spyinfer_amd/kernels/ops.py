@@ -73,7 +73,7 @@ class _Hip:
         self.lib.spy_last_error.restype = ctypes.c_char_p
         for name in ("spy_embedding", "spy_add_rmsnorm", "spy_rmsnorm", "spy_gemm", "spy_qknorm_rope_store",
                      "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_prefill",
-                     "spy_swiglu",
+                     "spy_attention_prefill_workspace", "spy_swiglu",
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
                      "spy_gemm_skinny_tiled"):
             if not hasattr(self.lib, name):
@@ -331,6 +331,7 @@ DECODE_SPLIT_TARGET = 256   # blocks (of 4 waves) wanted in flight when all entr
 
 
 PREFILL_ATTENTION_MAX_HEAD_DIM = 128
+PREFILL_SPLIT_BELOW = 256   # fewer (128-row tile, kv head) pairs than this: split the keys to fill the chip
 
 
 def prefill_attention_ok(d: int, page_size: int) -> bool:
@@ -383,8 +384,15 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             raise KernelError("paged_attention: 128-row tiles were built for head_dim %d and pages of %d, which the prefill "
                               "kernel refuses; build 16-row tiles only (ops.prefill_attention_ok)" % (d, page_size))
         if n_big:
+            # few tiles with many keys (a late portion of a long prompt): their keys are split into parts as well
+            bsplits = 1
+            if n_big * n_kv < PREFILL_SPLIT_BELOW:
+                bsplits = max(1, min(PREFILL_SPLIT_BELOW * 2 // (n_big * n_kv), meta.max_kv_len // 256, 16))
+            bws_floats = hip().lib.spy_attention_prefill_workspace(ctypes.c_int(n_big), ctypes.c_int(n_kv), ctypes.c_int(d),
+                                                                   ctypes.c_int(bsplits))
+            bws = torch.empty((max(1, bws_floats),), dtype=torch.float32, device=q.device)
             hip().call("spy_attention_prefill", _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), *common, _ptr(big_entry),
-                       _ptr(big_row0), ctypes.c_int(n_big), *sizes, _Hip.stream())
+                       _ptr(big_row0), ctypes.c_int(n_big), *sizes, ctypes.c_int(bsplits), _ptr(bws), _Hip.stream())
         if n_small:
             # Few 16-row tiles cannot fill the chip by themselves (decoding requests, short portions): their keys are
             # split into parts, each part a block of 4 waves that wants 128 keys at least, and a second kernel merges.

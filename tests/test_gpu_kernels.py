@@ -307,6 +307,8 @@ ATT_CASES = [
     (16, 2, 64, 16, [(200, 100), (0, 3)], None),                            # a long portion that starts late: 800 rows
     (4, 4, 96, 32, [(50, 90), (0, 257)], None),
     (8, 2, 128, 8, [(0, 300), (64, 64), (500, 1)], 130),
+    (4, 2, 64, 16, [(900, 70), (1300, 40)], None),                          # few big tiles, many keys: key parts + merge
+    (8, 2, 128, 16, [(1500, 33)], 700),
 ]
 
 
