@@ -25,6 +25,40 @@ extern "C" int spy_embedding(float* out, const void* table, int table_dtype, con
     return 0;
 }
 
+// The same for at most 16 tokens, prepared for a product that applies the first RMS norm's scale after its sum:
+// xw[t] = bf16(h[t] * w_norm) and ss[t] = sum(h[t]^2) (ss[T..15] = 0).
+template <typename TW>
+__global__ __launch_bounds__(256) void embedding_sumsq_kernel(float* __restrict__ out, bf16_t* __restrict__ xw, float* __restrict__ ss,
+                                                              const TW* __restrict__ table, const bf16_t* __restrict__ w_norm,
+                                                              const int* __restrict__ ids, int T, int H, int V) {
+    __shared__ float red[8];
+    const int t = blockIdx.x;
+    if (t >= T) { if (threadIdx.x == 0) ss[t] = 0.f; return; }
+    const int id = ids[t];
+    float* o = out + (size_t)t * H;
+    bf16_t* x = xw + (size_t)t * H;
+    const TW* row = table + (size_t)(id < 0 || id >= V ? 0 : id) * H;
+    const bool known = id >= 0 && id < V;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float v = known ? to_f32<TW>(row[i]) : 0.f;
+        o[i] = v;
+        x[i] = f32_to_bf16(v * bf16_to_f32(w_norm[i]));
+        s += v * v;
+    }
+    s = block_sum(s, red);
+    if (threadIdx.x == 0) ss[t] = s;
+}
+
+extern "C" int spy_embedding_sumsq(float* out, void* xw, float* ss, const void* table, int table_dtype, const void* w_norm,
+                                   const int* ids, int T, int H, int V, hipStream_t st) {
+    SPY_REQUIRE(T > 0 && T <= 16 && H > 0 && V > 0, "spy_embedding_sumsq: T = %d tokens (1..16 allowed)", T);
+    SPY_DISPATCH(table_dtype, TW, embedding_sumsq_kernel<TW><<<16, 256, 0, st>>>(out, (bf16_t*)xw, ss, (const TW*)table,
+                                                                                 (const bf16_t*)w_norm, ids, T, H, V));
+    SPY_CHECK_LAUNCH("spy_embedding_sumsq");
+    return 0;
+}
+
 // ---------------------------------------------------------------------------------------------
 // x = resid[t] (+ delta[t]);  rows == null: resid[t] = x.  out[r] = (x / sqrt(mean(x^2) + eps)) * w
 // One block per row.  The row is read once and kept in registers (4 values per thread and pass,

@@ -1,0 +1,197 @@
+// Decode-time products (at most 16 rows) with the neighbouring small kernels folded in, so that a decode
+// step launches fewer kernels (each costs 5-7 us here however little it does):
+//
+//   EPI_RESID the result is added to the residual stream h in place (float32); the block also writes
+//             bf16(h_new * w_next), the next RMS norm's input already multiplied by that norm's weight, and
+//             its part of every row's sum(h_new^2).
+//   SCALED    the input is such a bf16(h * w) with the parts of sum(h^2); they are summed in a fixed order
+//             and the result of the product is multiplied by rsqrt(sum / K + eps) in float32.  Together:
+//             x . W^T with x = norm(h), the scale applied after the sum instead of before it.  The one
+//             rounding of the operand to bfloat16 happens before the scale, which changes nothing in its
+//             relative size.
+//   EPI_GATED W = [gate | up] tiles, the block stores silu(gate) * up.
+//   EPI_STORE the block stores the result (bfloat16 or float32).
+//
+// W is in MFMA tile order (see gemm_skinny.hip, TILED): [N/16][K/32][64 lanes][8].  One 16-row tile (two for
+// EPI_GATED) per block, 8 waves split K in interleaved chunks of 128 and add through LDS in a fixed order.
+#include "common.h"
+#include <math.h>
+
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+
+#define GD_WAVES 8
+#define GD_CHUNK 128
+#define EPI_STORE 0
+#define EPI_GATED 1
+#define EPI_RESID 2
+
+template <int EPI, bool SCALED, typename TC>
+__global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, float* __restrict__ resid_out,
+    bf16_t* __restrict__ xw_out, const bf16_t* __restrict__ w_next, float* __restrict__ ss_out, const float* __restrict__ ss_in,
+    int n_parts, float eps, int M, int N, int K) {
+    constexpr int NT = EPI == EPI_GATED ? 2 : 1;
+    __shared__ float red[(GD_WAVES - 1) * NT * 64 * 4];
+    __shared__ float ss_red[GD_WAVES * 4 * 16];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int n_base = blockIdx.x * 16;
+    const bool x_ok = r < M;                       // lanes whose row of X does not exist load nothing
+
+    // Loads whose values are needed only after the product are issued now, so that they are on their way while
+    // the matrix streams: every thread's share of the parts of sum(h^2) of row r (the first 256 parts; more are
+    // summed here), and for the residual epilogue wave 0's piece of the stream and of the next norm's weight.
+    float pv[8], part = 0.f;
+    if (SCALED) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int p = wave * 4 + g + GD_WAVES * 4 * i;
+            pv[i] = p < n_parts ? ss_in[p * 16 + r] : 0.f;
+        }
+        for (int p = 256 + wave * 4 + g; p < n_parts; p += GD_WAVES * 4) part += ss_in[p * 16 + r];
+    }
+    f32x4_t h_old = {0.f, 0.f, 0.f, 0.f};
+    uint2 wn = {0u, 0u};
+    if (EPI == EPI_RESID && wave == 0 && x_ok) {
+        h_old = *reinterpret_cast<const f32x4_t*>(resid_out + (size_t)r * N + n_base + 4 * g);
+        wn = *reinterpret_cast<const uint2*>(w_next + n_base + 4 * g);
+    }
+
+    f32x4_t acc[NT], acc2[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) { acc[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f}; acc2[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f}; }
+    const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)n_base * K * 2;
+    unsigned woff[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) woff[nt] = (unsigned)(nt * N / 16) * (unsigned)K * 32u + 16u * lane;
+    const char* xbase = reinterpret_cast<const char*>(X);
+    const unsigned xoff = (unsigned)min(r, M - 1) * (unsigned)K * 2u + 16u * g;
+
+    bf16x8_t a0[NT][4], a1[NT][4], b0[4], b1[4];
+#define GD_LOAD(A, B, CHUNK)                                                                             \
+    {                                                                                                    \
+        const char* wb_ = wbase + (size_t)(CHUNK) * 4096;                                                \
+        const char* xb_ = xbase + (size_t)(CHUNK) * (GD_CHUNK * 2) + xoff;                               \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                  \
+            _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                            \
+                A[nt][j] = *reinterpret_cast<const bf16x8_t*>(wb_ + woff[nt] + 1024 * j);                \
+            B[j] = x_ok ? *reinterpret_cast<const bf16x8_t*>(xb_ + 64 * j) : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; \
+        }                                                                                                \
+    }
+#define GD_MFMA(A, B, ACC)                                                                               \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                        \
+        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                \
+            ACC[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[nt][j], B[j], ACC[nt], 0, 0, 0);
+
+    const int nfull = K / GD_CHUNK;                 // K is a multiple of 128
+    int c = wave;
+    for (; c + GD_WAVES < nfull; c += 2 * GD_WAVES) {
+        GD_LOAD(a0, b0, c)
+        GD_LOAD(a1, b1, c + GD_WAVES)
+        GD_MFMA(a0, b0, acc)
+        GD_MFMA(a1, b1, acc2)
+    }
+    if (c < nfull) {
+        GD_LOAD(a0, b0, c)
+        GD_MFMA(a0, b0, acc)
+    }
+#undef GD_LOAD
+#undef GD_MFMA
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[nt] += acc2[nt];
+
+    if (SCALED) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) part += pv[i];
+        ss_red[(wave * 4 + g) * 16 + r] = part;
+    }
+    // ---- add the waves' tiles, in a fixed order ---------------------------------------------------------------
+    if (wave > 0) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[(((wave - 1) * NT + nt) * 4 + i) * 64 + lane] = acc[nt][i];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 1; w < GD_WAVES; ++w)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[nt][i] += red[(((w - 1) * NT + nt) * 4 + i) * 64 + lane];
+    if (SCALED) {
+        float s = 0.f;
+        for (int i = 0; i < GD_WAVES * 4; ++i) s += ss_red[i * 16 + r];
+        const float scale = 1.0f / sqrtf(s / (float)K + eps);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[nt][i] *= scale;
+    }
+
+    // lane (m = r, g) holds C[m][n_base + 4 g + i]
+    const int m = r, n = n_base + 4 * g;
+    if (EPI == EPI_RESID) {
+        float s = 0.f;
+        if (m < M) {
+            float* hp = resid_out + (size_t)m * N + n;
+            f32x4_t h = h_old;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { h[i] += acc[0][i]; s += h[i] * h[i]; }
+            *reinterpret_cast<f32x4_t*>(hp) = h;
+            uint2 o;
+            o.x = pack_bf16x2(h[0] * __uint_as_float(wn.x << 16), h[1] * __uint_as_float(wn.x & 0xffff0000u));
+            o.y = pack_bf16x2(h[2] * __uint_as_float(wn.y << 16), h[3] * __uint_as_float(wn.y & 0xffff0000u));
+            *reinterpret_cast<uint2*>(xw_out + (size_t)m * N + n) = o;
+        }
+        s += __shfl_xor(s, 16, 64);
+        s += __shfl_xor(s, 32, 64);
+        if (g == 0) ss_out[blockIdx.x * 16 + r] = s;     // rows beyond M: 0
+        return;
+    }
+    if (m >= M) return;
+    TC* out = C + (size_t)m * N + n;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float v = acc[0][i];
+        if (EPI == EPI_GATED) { const float up = acc[NT - 1][i]; v = (v / (1.0f + expf(-v))) * up; }
+        out[i] = from_f32<TC>(v);
+    }
+}
+
+// x: bfloat16 [M, K].  scaled != 0: x = bf16(h * w_norm) and ss_in [n_parts, 16] holds the parts of sum(h^2); the
+// result is multiplied by rsqrt(sum / K + eps).
+// epi 0: C [M, N] (c_dtype);  epi 1: W = [gate | up], C [M, N] = silu(gate) * up;  epi 2: resid [M, N] += result,
+// xw_out [M, N] = bf16(resid * w_next), ss_out [N / 16, 16] = every block's part of the rows' sums of squares.
+extern "C" int spy_gemm_decode(const void* X, int scaled, const float* ss_in, int n_parts, float eps, const void* Wt, int epi,
+                               void* C, int c_dtype, float* resid, void* xw_out, const void* w_next, float* ss_out, int M, int N,
+                               int K, hipStream_t st) {
+    SPY_REQUIRE(M > 0 && M <= 16, "spy_gemm_decode: M = %d rows (1..16 allowed)", M);
+    SPY_REQUIRE(N > 0 && N % 16 == 0 && K > 0 && K % 128 == 0, "spy_gemm_decode: N = %d must be a multiple of 16 and K = %d of 128", N, K);
+    SPY_REQUIRE(epi >= 0 && epi <= 2, "spy_gemm_decode: unknown epilogue %d", epi);
+    SPY_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)Wt % 16) == 0, "spy_gemm_decode: operands must be 16-byte aligned");
+    SPY_REQUIRE(!scaled || (ss_in && n_parts > 0), "spy_gemm_decode: the scale needs the parts of the sums of squares");
+    SPY_REQUIRE(epi != EPI_RESID || (resid && ss_out && xw_out && w_next && ((uintptr_t)resid % 16) == 0 &&
+                                     ((uintptr_t)xw_out % 8) == 0 && ((uintptr_t)w_next % 8) == 0),
+                "spy_gemm_decode: the residual epilogue needs the stream, the next norm's weight and its outputs");
+    SPY_REQUIRE(epi == EPI_RESID || (C && ((uintptr_t)C % 16) == 0), "spy_gemm_decode: no output");
+    SPY_REQUIRE((long long)(N + 16) * K * 2 < (1ll << 32), "spy_gemm_decode: the matrix is too large for 32-bit offsets inside a block");
+    const bf16_t* x = (const bf16_t*)X;
+    const bf16_t* w = (const bf16_t*)Wt;
+    const int blocks = N / 16;
+#define GD_LAUNCH(EPI_, SCALED_, TC_)                                                                             \
+    gemm_decode_kernel<EPI_, SCALED_, TC_><<<blocks, GD_WAVES * 64, 0, st>>>(x, w, (TC_*)C, resid, (bf16_t*)xw_out, (const bf16_t*)w_next, \
+                                                                             ss_out, ss_in, n_parts, eps, M, N, K)
+#define GD_TYPES(EPI_, SCALED_)                                                  \
+    if (c_dtype == SPY_F32) GD_LAUNCH(EPI_, SCALED_, float); else GD_LAUNCH(EPI_, SCALED_, bf16_t)
+    if (epi == EPI_RESID) { if (scaled) GD_LAUNCH(EPI_RESID, true, bf16_t); else GD_LAUNCH(EPI_RESID, false, bf16_t); }
+    else if (epi == EPI_GATED) { if (scaled) { GD_TYPES(EPI_GATED, true); } else { GD_TYPES(EPI_GATED, false); } }
+    else { if (scaled) { GD_TYPES(EPI_STORE, true); } else { GD_TYPES(EPI_STORE, false); } }
+#undef GD_TYPES
+#undef GD_LAUNCH
+    SPY_CHECK_LAUNCH("spy_gemm_decode");
+    return 0;
+}

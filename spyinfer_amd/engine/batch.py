@@ -89,6 +89,8 @@ class StepBatch:
         positions = (np.arange(T, dtype=np.int32) - cu_q[:-1][token_entry] + pos0[token_entry]).astype(np.int32)
         rows = np.fromiter((int(cu_q[s]) + w for s, e in enumerate(self.entries) for w in e.want), dtype=np.int32)
         self.R = int(rows.shape[0])
+        #: every token's logits are wanted, in order: the output head may take the step's rows as they are
+        self.all_rows_wanted = self.R == T and bool((rows == np.arange(T, dtype=np.int32)).all())
         kv_len = pos0 + lens
         self.max_q_len = int(lens.max()) if S else 0
         self.max_kv_len = int(kv_len.max()) if S else 0

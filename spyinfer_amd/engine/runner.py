@@ -121,7 +121,7 @@ class ModelRunner:
 
     # ---- graphs -----------------------------------------------------------------
     def _step_graph(self, batch: StepBatch) -> torch.Tensor:
-        key = batch.layout_key()
+        key = (batch.layout_key(), batch.all_rows_wanted)
         held = self._graphs.get(key)
         if held is not None:
             graph, dev_buf, logits = held

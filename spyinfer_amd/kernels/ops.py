@@ -75,7 +75,7 @@ class _Hip:
                      "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_prefill",
                      "spy_attention_prefill_workspace", "spy_swiglu",
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
-                     "spy_gemm_skinny_tiled"):
+                     "spy_gemm_skinny_tiled", "spy_gemm_decode", "spy_embedding_sumsq"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: rebuild it (python -c 'import __graft_entry__ as g; g.build()')"
                                   % (self.lib._name, name))
@@ -256,6 +256,104 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, tiled: Optional[torc
                    ctypes.c_int(I), ctypes.c_int(K), _Hip.stream())
         return out
     return swiglu(linear(x, w_gate_up))
+
+
+# --------------------------------------------------------------------------
+# Decode-time products with the norm and the residual sum folded in
+class ScaledInput:
+    """The input of a product as 'the RMS norm of the residual stream' with the scale still to come:
+    ``xw [M, K]`` = bfloat16(h * w_norm), and the parts ``ss_parts [n, 16]`` of every row's sum of squares
+    (row r of the stream in column r; their sum over n is sum(h[r]^2)).  ``decode_linear`` and
+    ``decode_linear_swiglu`` multiply their result by rsqrt(sum / K + eps), which equals the product with the
+    normed rows.  ``norm`` is the norm part this was prepared for."""
+    __slots__ = ("xw", "ss_parts", "eps", "norm")
+
+    def __init__(self, xw: torch.Tensor, ss_parts: torch.Tensor, eps: float, norm=None):
+        self.xw, self.ss_parts, self.eps, self.norm = xw, ss_parts, float(eps), norm
+
+
+#: False switches the folded decode products off (every norm then runs as a kernel of its own).
+FUSED_DECODE = True
+FUSED_DECODE_MAX_ROWS = 16
+
+
+def fused_decode_ok(rows: int, act_dtype, *tiled_weights) -> bool:
+    """True if products of ``rows`` rows with these tiled matrices can run with the norm's scale and the residual
+    sum folded in: bfloat16 activations, at most 16 rows, tiled bfloat16 weights."""
+    if not FUSED_DECODE or _impl is not None or act_dtype != torch.bfloat16 or not 0 < rows <= FUSED_DECODE_MAX_ROWS:
+        return False
+    return all(t is not None and t.dtype == torch.bfloat16 and t.shape[0] % 16 == 0 and t.shape[1] % 128 == 0
+               and (t.shape[0] + 16) * t.shape[1] * 2 < (1 << 32) for t in tiled_weights)
+
+
+def _gemm_decode(x, tiled: torch.Tensor, epi: int, n_out: int, out, resid, xw_out, w_next, ss_out) -> None:
+    _check(tiled.dtype == torch.bfloat16 and tiled.dim() == 2, "decode product: the tiled matrix must be bfloat16 [N, K]")
+    K = tiled.shape[1]
+    if isinstance(x, ScaledInput):
+        xs, ss, eps = x.xw, x.ss_parts, x.eps
+        _check(ss.dtype == torch.float32 and ss.dim() == 2 and ss.shape[1] == 16 and ss.shape[0] > 0,
+               "decode product: the parts of the sums of squares must be float32 [n, 16]")
+    else:
+        xs, ss, eps = x, None, 0.0
+    _dev(xs, ss, tiled, out, resid, xw_out, w_next, ss_out)
+    _check(xs.dtype == torch.bfloat16 and xs.dim() == 2 and xs.shape[1] == K, "decode product: x must be bfloat16 [M, %d]" % K)
+    M = xs.shape[0]
+    _check(0 < M <= FUSED_DECODE_MAX_ROWS, "decode product: %d rows (1..%d allowed)" % (M, FUSED_DECODE_MAX_ROWS))
+    hip().call("spy_gemm_decode", _ptr(xs), ctypes.c_int(0 if ss is None else 1), _ptr(ss), ctypes.c_int(0 if ss is None else ss.shape[0]),
+               ctypes.c_float(eps), _ptr(tiled), ctypes.c_int(epi), _ptr(out), ctypes.c_int(0 if out is None else _code(out, "out")),
+               _ptr(resid), _ptr(xw_out), _ptr(w_next), _ptr(ss_out), ctypes.c_int(M), ctypes.c_int(n_out), ctypes.c_int(K),
+               _Hip.stream())
+
+
+def _rows_of(x) -> int:
+    return (x.xw if isinstance(x, ScaledInput) else x).shape[0]
+
+
+def decode_linear(x, tiled: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """y = x . w^T for at most 16 rows; ``x`` bfloat16 [M, K] or a ScaledInput, ``tiled`` from tile_weight."""
+    N = tiled.shape[0]
+    out = torch.empty((_rows_of(x), N), dtype=out_dtype, device=tiled.device)
+    _gemm_decode(x, tiled, 0, N, out, None, None, None, None)
+    return out
+
+
+def decode_linear_swiglu(x, tiled_gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(x . Wgate^T) * (x . Wup^T) for at most 16 rows; ``tiled_gate_up [2 I, K]`` = tiles of [Wgate | Wup]."""
+    _check(tiled_gate_up.shape[0] % 32 == 0, "decode_linear_swiglu: [2 I, K] with I a multiple of 16 expected")
+    I = tiled_gate_up.shape[0] // 2
+    out = torch.empty((_rows_of(x), I), dtype=torch.bfloat16, device=tiled_gate_up.device)
+    _gemm_decode(x, tiled_gate_up, 1, I, out, None, None, None, None)
+    return out
+
+
+def decode_linear_residual(x: torch.Tensor, tiled: torch.Tensor, resid: torch.Tensor, next_norm_weight: torch.Tensor,
+                           eps: float, norm=None) -> ScaledInput:
+    """resid += x . w^T (float32, in place) for at most 16 rows -> the ScaledInput of the norm that reads the
+    stream next: bfloat16(resid * next_norm_weight) and the parts [N / 16, 16] of the new rows' sums of squares."""
+    N = tiled.shape[0]
+    _check(resid.dtype == torch.float32 and resid.dim() == 2 and resid.shape == (_rows_of(x), N),
+           "decode_linear_residual: the stream must be float32 [M, %d]" % N)
+    _check(next_norm_weight.dtype == torch.bfloat16 and next_norm_weight.shape == (N,),
+           "decode_linear_residual: the next norm's weight must be bfloat16 [%d]" % N)
+    ss = torch.empty((N // 16, 16), dtype=torch.float32, device=resid.device)
+    xw = torch.empty((resid.shape[0], N), dtype=torch.bfloat16, device=resid.device)
+    _gemm_decode(x, tiled, 2, N, None, resid, xw, next_norm_weight, ss)
+    return ScaledInput(xw, ss, eps, norm)
+
+
+def embedding_scaled(ids: torch.Tensor, table: torch.Tensor, norm_weight: torch.Tensor, eps: float, norm=None):
+    """embedding() for at most 16 tokens -> (stream, ScaledInput of the first norm)."""
+    _dev(ids, table, norm_weight)
+    _check(ids.dtype == torch.int32 and ids.dim() == 1 and 0 < ids.shape[0] <= 16, "embedding_scaled: ids must be int32 [1..16]")
+    _check(table.dim() == 2, "embedding: table must be [V, H]")
+    T, (V, H) = ids.shape[0], table.shape
+    _check(norm_weight.dtype == torch.bfloat16 and norm_weight.shape == (H,), "embedding_scaled: the norm weight must be bfloat16 [H]")
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    xw = torch.empty((T, H), dtype=torch.bfloat16, device=table.device)
+    ss = torch.empty((1, 16), dtype=torch.float32, device=table.device)
+    hip().call("spy_embedding_sumsq", _ptr(out), _ptr(xw), _ptr(ss), _ptr(table), _code(table, "embedding table"), _ptr(norm_weight),
+               _ptr(ids), ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(V), _Hip.stream())
+    return out, ScaledInput(xw, ss, eps, norm)
 
 
 def qk_norm_rope_store(qkv: torch.Tensor, n_q: int, n_kv: int, d: int, q_norm_w, k_norm_w, eps: float,

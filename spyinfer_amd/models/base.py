@@ -13,6 +13,7 @@ from typing import Dict, List, NamedTuple, Optional, Sequence
 
 import torch
 
+from ..kernels.ops import ScaledInput
 from ..parts.base import Block, Norm, PositionEncoding
 from ..parts.embedding import LMHead, TokenEmbedding
 from ..weights.loader import WeightSpec
@@ -92,14 +93,20 @@ class DecoderModel:
     def forward(self, batch, storage) -> torch.Tensor:
         """Runs the batch's tokens through all calls of the run order; float32 logits [R, vocab]
         at the batch's wanted rows."""
-        resid = self.embed.forward(batch.token_ids)
-        if self.position is not None:
-            resid = self.position.on_embeddings(resid, batch)
-        delta = None
-        for call in self.schedule:
+        calls = self.schedule
+        entry = [self.layers[c.layer].entry_norm() for c in calls] + [self.final_norm]
+        if self.position is None or type(self.position).on_embeddings is PositionEncoding.on_embeddings:
+            resid, pending = self.embed.forward_for(batch.token_ids, entry[0], batch.act_dtype)
+        else:
+            resid, pending = self.position.on_embeddings(self.embed.forward(batch.token_ids), batch), None
+        for i, call in enumerate(calls):
             cache = storage.layer(call.cache) if call.cache is not None else None
-            resid, delta = self.layers[call.layer].forward(resid, delta, batch, cache, call.store)
+            resid, pending = self.layers[call.layer].forward(resid, pending, batch, cache, call.store, next_norm=entry[i + 1])
         if batch.R == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=resid.device)
-        normed = self.final_norm.add_norm(resid, delta, batch.act_dtype, batch.logit_rows)
+        if isinstance(pending, ScaledInput):
+            if pending.norm is self.final_norm and batch.all_rows_wanted and self.lm_head.can_fold(batch):
+                return self.lm_head.forward(pending)
+            pending = None                       # the stream is complete
+        normed = self.final_norm.add_norm(resid, pending, batch.act_dtype, batch.logit_rows)
         return self.lm_head.forward(normed)

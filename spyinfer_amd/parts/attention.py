@@ -65,9 +65,15 @@ class PagedAttention(Mixer):
         batch.add_attention_tiles(self.num_heads // self.num_kv_heads, ops.prefill_attention_ok(self.head_dim, batch.page_size))
 
     # ---- step ------------------------------------------------------------
-    def forward(self, x, batch, cache, store=True):
+    def can_fold(self, batch):
+        return ops.fused_decode_ok(batch.T, batch.act_dtype, self.w_qkv_tiled, self.w_o_tiled)
+
+    def _attend(self, x, batch, cache, store):
         nq, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
-        qkv = ops.linear(x, self.w_qkv, tiled=self.w_qkv_tiled)
+        if isinstance(x, ops.ScaledInput):
+            qkv = ops.decode_linear(x, self.w_qkv_tiled)
+        else:
+            qkv = ops.linear(x, self.w_qkv, tiled=self.w_qkv_tiled)
         rot = self.position.rotary() if self.position is not None else None
         cos, sin, rdim = rot if rot is not None else (None, None, 0)
         slots = batch.slot_mapping(cache.group) if store else None
@@ -75,5 +81,11 @@ class PagedAttention(Mixer):
                                    self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
                                    cos, sin, rdim, batch.positions, cache.k, cache.v, cache.page_size, slots)
         meta = batch.attention_meta(cache.group, nq // nkv)
-        a = ops.paged_attention(q, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window)
-        return ops.linear(a, self.w_o, tiled=self.w_o_tiled)
+        return ops.paged_attention(q, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window)
+
+    def forward(self, x, batch, cache, store=True):
+        return ops.linear(self._attend(x, batch, cache, store), self.w_o, tiled=self.w_o_tiled)
+
+    def forward_into(self, x, batch, cache, store, resid, next_norm):
+        weight, eps = next_norm.foldable(batch.act_dtype)
+        return ops.decode_linear_residual(self._attend(x, batch, cache, store), self.w_o_tiled, resid, weight, eps, next_norm)

@@ -39,6 +39,12 @@ class Norm(Part):
         the hidden state."""
         raise NotImplementedError
 
+    def foldable(self, out_dtype: torch.dtype):
+        """None, or (weight, eps) if this norm can be folded into the products around it when a step has few rows:
+        the product before it adds to the stream and prepares this norm's input, the product after it applies the
+        scale (``spyinfer_amd.kernels.ops.ScaledInput``).  Parts that do not know of this are never asked."""
+        return None
+
 
 class PositionEncoding(Part):
     """How positions enter the model.  A rotary encoding hands its tables to the mixer,
@@ -73,10 +79,26 @@ class Mixer(Part):
         another layer without writing to it."""
         raise NotImplementedError
 
+    def can_fold(self, batch) -> bool:
+        """True if, for this step, ``forward`` takes a ``ScaledInput`` in place of x and ``forward_into`` exists."""
+        return False
+
+    def forward_into(self, x, batch, cache, store, resid: torch.Tensor, next_norm: Norm):
+        """Optional: resid += mixer(x) in place; returns the ``ScaledInput`` for ``next_norm`` (which is foldable)."""
+        raise NotImplementedError
+
 
 class FeedForward(Part):
     def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
         """x [T, H] (normed) -> [T, H]."""
+        raise NotImplementedError
+
+    def can_fold(self, batch) -> bool:
+        """As ``Mixer.can_fold``."""
+        return False
+
+    def forward_into(self, x, batch, resid: torch.Tensor, next_norm: Norm):
+        """Optional: resid += ffn(x) in place; returns the ``ScaledInput`` for ``next_norm`` (which is foldable)."""
         raise NotImplementedError
 
 
@@ -85,7 +107,14 @@ class Block(Part):
 
     mixer: Mixer
 
-    def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], batch, cache, store: bool = True):
-        """(residual stream, pending addend) -> (residual stream, pending addend).  The addend
-        is summed into the stream by the next norm."""
+    def forward(self, resid: torch.Tensor, delta, batch, cache, store: bool = True, next_norm: Optional[Norm] = None):
+        """(residual stream, pending) -> (residual stream, pending).  ``pending`` is None, an addend [T, H] that
+        the next norm sums into the stream, or a ``ScaledInput``: then the stream is complete and the input of
+        the norm named in it is prepared (a block that cannot use it ignores it).  ``next_norm``: the norm that
+        reads the stream after this block, if the caller knows it; only then may a ``ScaledInput`` be returned."""
         raise NotImplementedError
+
+    def entry_norm(self) -> Optional[Norm]:
+        """The norm that reads the stream first in this block, if it wants the block before it to prepare its
+        input."""
+        return None

@@ -2,6 +2,7 @@
 The sums are carried as a pending addend and folded into the next norm's kernel."""
 from __future__ import annotations
 
+from ..kernels import ops
 from .base import Block, FeedForward, Mixer, Norm
 
 
@@ -21,9 +22,23 @@ class PreNormBlock(Block):
         for part, p in self._parts(prefix):
             part.bind(p, weights)
 
-    def forward(self, resid, delta, batch, cache, store=True):
+    def entry_norm(self):
+        return self.norm1
+
+    def forward(self, resid, pending, batch, cache, store=True, next_norm=None):
         act = batch.act_dtype
-        n1 = self.norm1.add_norm(resid, delta, act)
+        ready = isinstance(pending, ops.ScaledInput)
+        if self.norm2.foldable(act) is not None and self.mixer.can_fold(batch) and self.ffn.can_fold(batch):
+            # few rows: the sums go into the stream inside the products, the norms' scales into the products after them
+            if ready and pending.norm is self.norm1:
+                n1 = pending
+            else:
+                n1 = self.norm1.add_norm(resid, None if ready else pending, act)
+            n2 = self.mixer.forward_into(n1, batch, cache, store, resid, self.norm2)
+            if next_norm is not None and next_norm.foldable(act) is not None:
+                return resid, self.ffn.forward_into(n2, batch, resid, next_norm)
+            return resid, self.ffn.forward(n2, batch)
+        n1 = self.norm1.add_norm(resid, None if ready else pending, act)
         a = self.mixer.forward(n1, batch, cache, store)
         n2 = self.norm2.add_norm(resid, a, act)
         return resid, self.ffn.forward(n2, batch)

@@ -24,6 +24,13 @@ class TokenEmbedding(Part):
     def forward(self, ids):
         return ops.embedding(ids, self.weight)
 
+    def forward_for(self, ids, norm, act_dtype):
+        """(stream, pending) with the input of ``norm`` prepared where few rows and a foldable norm allow it."""
+        fold = norm.foldable(act_dtype) if norm is not None else None
+        if fold is None or not ops.fused_decode_ok(ids.shape[0], act_dtype):
+            return ops.embedding(ids, self.weight), None
+        return ops.embedding_scaled(ids, self.weight, fold[0], fold[1], norm)
+
 
 class LMHead(Part):
     def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding = None):
@@ -40,5 +47,10 @@ class LMHead(Part):
         self.weight = self.tied_to.weight if self.tied_to is not None else weights[prefix + ".weight"]
         self.weight_tiled = ops.tile_weight(self.weight)
 
+    def can_fold(self, batch):
+        return ops.fused_decode_ok(batch.T, batch.act_dtype, self.weight_tiled)
+
     def forward(self, normed):
+        if isinstance(normed, ops.ScaledInput):
+            return ops.decode_linear(normed, self.weight_tiled, torch.float32)
         return ops.linear(normed, self.weight, torch.float32, tiled=self.weight_tiled)

@@ -32,5 +32,15 @@ class GatedMLP(FeedForward):
         self.w_gate_up_tiled = ops.tile_weight(self.w_gate_up) if self.intermediate_size % 16 == 0 else None
         self.w_down_tiled = ops.tile_weight(self.w_down)
 
+    def can_fold(self, batch):
+        return ops.fused_decode_ok(batch.T, batch.act_dtype, self.w_gate_up_tiled, self.w_down_tiled)
+
     def forward(self, x, batch):
+        if isinstance(x, ops.ScaledInput):
+            return ops.linear(ops.decode_linear_swiglu(x, self.w_gate_up_tiled), self.w_down, tiled=self.w_down_tiled)
         return ops.linear(ops.linear_swiglu(x, self.w_gate_up, self.w_gate_up_tiled), self.w_down, tiled=self.w_down_tiled)
+
+    def forward_into(self, x, batch, resid, next_norm):
+        weight, eps = next_norm.foldable(batch.act_dtype)
+        return ops.decode_linear_residual(ops.decode_linear_swiglu(x, self.w_gate_up_tiled), self.w_down_tiled, resid, weight, eps,
+                                          next_norm)

@@ -3,6 +3,8 @@ root, the weight multiplies as it is (src/backends/cpu/x64/kernels.cpp:168-180;
 src/backends/cuda/native/common.cuh:57-188)."""
 from __future__ import annotations
 
+import torch
+
 from ..kernels import ops
 from ..weights.loader import WeightSpec
 from .base import Norm
@@ -22,3 +24,8 @@ class RMSNorm(Norm):
 
     def add_norm(self, resid, delta, out_dtype, rows=None):
         return ops.add_rms_norm(resid, delta, self.weight, self.eps, out_dtype, rows)
+
+    def foldable(self, out_dtype):
+        if out_dtype == torch.bfloat16 and self.weight is not None and self.weight.dtype == torch.bfloat16:
+            return self.weight, self.eps
+        return None

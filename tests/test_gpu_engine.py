@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from tests import replay_cases as rc
-from tests.configs import INIT, TINY_A, TINY_B, TINY_C
+from tests.configs import INIT, TINY_A, TINY_B, TINY_C, TINY_D
 from tests.gpu_util import require_gpu
 from tests.plain.qwen3_plain import PlainQwen3
 
@@ -108,6 +108,64 @@ def test_graph_replays_equal_eager_steps(folder_c, dtype):
     tol = TOL[dtype]
     for i, (a, b) in enumerate(zip(*runs)):
         assert torch.allclose(a, b, atol=tol["atol"], rtol=tol["rtol"]), "step %d: graph and eager differ by %g" % (i, (a - b).abs().max())
+
+
+def test_folded_decode_steps(tmp_path_factory):
+    """Steps of few rows in bfloat16 with sizes that allow it run the products with the norms folded in.  With
+    that switched off the same steps give the same logits up to bfloat16 rounding, eagerly and from graphs; a
+    step of 3 decoded tokens beside a 5-token portion of which only some logits are wanted takes the folded
+    layers and the plain output head."""
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.runner import ModelRunner, load_model
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.weights import write_random_model
+    dev = require_gpu()
+    folder = write_random_model(str(tmp_path_factory.mktemp("eng_d")), TINY_D, 63, torch.bfloat16, **INIT)
+    plain = PlainQwen3(folder)
+    model = load_model(folder, "bfloat16", dev)
+    ps = prompts(400, [40, 3, 130, 21], 3)
+    runs, calls = [], []
+    real = ops.decode_linear_residual
+    for folded, eager in ((True, True), (True, False), (False, True)):
+        ops.FUSED_DECODE = folded
+        n = [0]
+        ops.decode_linear_residual = lambda *a, **k: (n.__setitem__(0, n[0] + 1), real(*a, **k))[1]
+        try:
+            runner = ModelRunner(model, "bfloat16", dev, 16, 64, 4, enforce_eager=eager, max_model_len=320)
+            caches = [runner.manager.admit(i) for i in range(4)]
+            for c, p in zip(caches[:3], ps):
+                runner.manager.reserve(c, len(p))
+            runner.step([StepEntry(c, p, []) for c, p in zip(caches[:3], ps)])
+            g = torch.Generator().manual_seed(4)
+            outs, seqs = [], [list(p) for p in ps[:3]]
+            for i in range(12):
+                toks = torch.randint(0, 400, (3,), generator=g).tolist()
+                for c in caches[:3]:
+                    runner.manager.reserve(c, 1)
+                entries = [StepEntry(c, [t], [0]) for c, t in zip(caches[:3], toks)]
+                for q, t in zip(seqs, toks):
+                    q.append(t)
+                if i == 5:
+                    runner.manager.reserve(caches[3], 5)
+                    entries.insert(1, StepEntry(caches[3], ps[3][:5], [1, 4]))
+                outs.append(runner.step(entries).cpu().clone())
+            runs.append(outs)
+            calls.append(n[0])
+        finally:
+            ops.FUSED_DECODE = True
+            ops.decode_linear_residual = real
+    assert calls[0] >= 12 * 2 * 3 and calls[2] == 0
+    for i, (a, b, c) in enumerate(zip(*runs)):
+        for x, what in ((b, "graphs"), (c, "plain norms")):
+            assert a.shape == x.shape and torch.allclose(a, x, **TOL["bfloat16"]), "step %d: folded and %s differ by %g" % (
+                i, what, (a - x).abs().max())
+    # the last step against the plain implementation
+    ref = torch.stack([plain.forward(q)[-1] for q in seqs])
+    assert torch.allclose(runs[0][-1], ref, **TOL["bfloat16"]), (runs[0][-1] - ref).abs().max()
+    mixed = runs[0][5]
+    assert mixed.shape[0] == 5
+    ref4 = plain.forward(ps[3][:5])
+    assert torch.allclose(mixed[1:3], ref4[[1, 4]], **TOL["bfloat16"])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -111,6 +111,75 @@ def test_linear_with_tiled_weights(M, N, K):
     assert ops.tile_weight(rnd((24, 128), torch.bfloat16, dev, 1)) is None and ops.tile_weight(rnd((32, 96), torch.bfloat16, dev, 1)) is None
 
 
+@pytest.mark.parametrize("M,H,I,NQKV,eps", [(1, 128, 256, 192, 1e-6), (7, 256, 384, 400, 1e-5), (16, 4096, 1024, 6144, 1e-6),
+                                            (3, 5120, 128, 64, 1e-2)])
+def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
+    """The chain of a decode step's products with the norms folded in: the residual epilogue adds to the stream,
+    prepares bf16(h * w) and the parts of sum(h^2); the next products scale their sums by rsqrt(mean(h^2) + eps).
+    Compared with float64 formulas: RMS norm, product, SwiGLU, residual sum."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    resid0 = rnd((M, H), torch.float32, dev, 31, 1.5)
+    wn1 = (1 + 0.1 * rnd((H,), torch.float32, dev, 32)).bfloat16()
+    wn2 = (1 + 0.1 * rnd((H,), torch.float32, dev, 33)).bfloat16()
+    w_in = rnd((H, I), torch.bfloat16, dev, 34, 0.05)
+    w_qkv = rnd((NQKV, H), torch.bfloat16, dev, 35, 0.05)
+    w_gu = rnd((2 * I, H), torch.bfloat16, dev, 36, 0.05)
+    a = rnd((M, I), torch.bfloat16, dev, 37)
+
+    def norm64(h, w):
+        h = h.double()
+        return h * torch.rsqrt((h * h).mean(1, keepdim=True) + eps) * w.double()
+
+    # 1. the residual epilogue
+    resid = resid0.clone()
+    si = ops.decode_linear_residual(a, ops.tile_weight(w_in), resid, wn1, eps)
+    h = resid0.double() + a.double() @ w_in.double().t()
+    close(resid, h, torch.float32, scale=4.0, what="stream after the residual epilogue")
+    assert torch.equal(si.xw, (resid * wn1.float()).bfloat16()), "the prepared input is bf16(h * w) of the new stream"
+    ss = si.ss_parts.sum(0)
+    assert torch.allclose(ss[:M], (resid * resid).sum(1), rtol=1e-5) and (M == 16 or float(ss[M:].abs().max()) == 0.0)
+    # 2. products of the normed rows: plain, float32 result (logits), gated
+    for od in (torch.bfloat16, torch.float32):
+        close(ops.decode_linear(si, ops.tile_weight(w_qkv), od), norm64(resid, wn1) @ w_qkv.double().t(), torch.bfloat16,
+              scale=2.0, what="scaled decode_linear")
+    y = norm64(resid, wn1) @ w_gu.double().t()
+    close(ops.decode_linear_swiglu(si, ops.tile_weight(w_gu)), y[:, :I] / (1 + torch.exp(-y[:, :I])) * y[:, I:], torch.bfloat16,
+          scale=2.0, what="scaled decode_linear_swiglu")
+    # 3. a scaled input into a residual epilogue (the chain of two layers), with the second norm's weight
+    w_sq = rnd((H, H), torch.bfloat16, dev, 38, 0.05)
+    resid2 = resid.clone()
+    si2 = ops.decode_linear_residual(si, ops.tile_weight(w_sq), resid2, wn2, eps)
+    h2 = resid.double() + norm64(resid, wn1) @ w_sq.double().t()
+    close(resid2, h2, torch.bfloat16, scale=2.0, what="stream after a scaled product")
+    assert torch.equal(si2.xw, (resid2 * wn2.float()).bfloat16())
+    # 4. the scale matters: another eps or a missing part changes the result by far more than the tolerance
+    far = ops.decode_linear(ops.ScaledInput(si.xw, si.ss_parts * 4.0, eps), ops.tile_weight(w_qkv), torch.float32)
+    ref = (norm64(resid, wn1) @ w_qkv.double().t()).float()
+    assert float((far - ref).abs().max()) > 0.3 * float(ref.abs().max())
+    # 5. the embedding that starts such a chain
+    table = rnd((50, H), torch.bfloat16, dev, 39)
+    ids = torch.tensor([7, 0, 49, 7][:min(M, 4)], dtype=torch.int32, device=dev)
+    out, e = ops.embedding_scaled(ids, table, wn1, eps)
+    assert torch.equal(out, ops.embedding(ids, table)) and torch.equal(e.xw, (out * wn1.float()).bfloat16())
+    assert torch.allclose(e.ss_parts[0, :len(ids)], (out * out).sum(1), rtol=1e-5) and float(e.ss_parts[0, len(ids):].abs().max()) == 0.0
+
+
+def test_decode_products_refuse_wrong_operands():
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    w = ops.tile_weight(rnd((64, 128), torch.bfloat16, dev, 1))
+    with pytest.raises(ops.KernelError, match="rows"):
+        ops.decode_linear(rnd((17, 128), torch.bfloat16, dev, 2), w)
+    with pytest.raises(ops.KernelError, match="bfloat16"):
+        ops.decode_linear(rnd((4, 128), torch.float32, dev, 2), w)
+    with pytest.raises(ops.KernelError, match="stream"):
+        ops.decode_linear_residual(rnd((4, 128), torch.bfloat16, dev, 2), w, torch.zeros(4, 128, device=dev),
+                                   torch.ones(64, dtype=torch.bfloat16, device=dev), 1e-6)
+    with pytest.raises(ops.KernelError, match="parts"):
+        ops.decode_linear(ops.ScaledInput(rnd((4, 128), torch.bfloat16, dev, 2), torch.zeros(3, 8, device=dev), 1e-6), w)
+
+
 def test_linear_reference_vector():
     """test/test_linear.cpp:53-60 of the reference: x . W^T before the bias."""
     from spyinfer_amd.kernels import ops
