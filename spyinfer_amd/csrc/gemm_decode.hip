@@ -12,8 +12,12 @@
 //   EPI_GATED W = [gate | up] tiles, the block stores silu(gate) * up.
 //   EPI_STORE the block stores the result (bfloat16 or float32).
 //
-// W is in MFMA tile order (see gemm_skinny.hip, TILED): [N/16][K/32][64 lanes][8].  One 16-row tile (two for
-// EPI_GATED) per block, 8 waves split K in interleaved chunks of 128 and add through LDS in a fixed order.
+// W comes as a copy in the order the kernel reads it (ops.tile_weight): [K/128 chunks][N/16 tiles][4 steps][64 lanes][8],
+// lane 16 g + r of step j of chunk c of tile t holding W[16 t + r][128 c + 32 j + 8 g ..]: the MFMA operand of a wave
+// is one load of 1 KiB in one piece, and, chunks being outermost, the tiles that all blocks read at one time lie next
+// to each other in memory (with tiles outermost the blocks' addresses differ by multiples of the tile size and crowd
+// on a part of the memory channels: 8-10 % slower).  One 16-row tile (two for EPI_GATED: gate tile t and up tile
+// N/16 + t) per block; its waves split K in interleaved chunks and add through LDS in a fixed order.
 #include "common.h"
 #include <math.h>
 
@@ -21,13 +25,15 @@ typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 
-#define GD_WAVES 8
 #define GD_CHUNK 128
+#ifndef GD_WAVES_GATED
+#define GD_WAVES_GATED 4
+#endif
 #define EPI_STORE 0
 #define EPI_GATED 1
 #define EPI_RESID 2
 
-template <int EPI, bool SCALED, typename TC>
+template <int EPI, bool SCALED, typename TC, int GD_WAVES>
 __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, float* __restrict__ resid_out,
     bf16_t* __restrict__ xw_out, const bf16_t* __restrict__ w_next, float* __restrict__ ss_out, const float* __restrict__ ss_in,
@@ -43,10 +49,11 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     // Loads whose values are needed only after the product are issued now, so that they are on their way while
     // the matrix streams: every thread's share of the parts of sum(h^2) of row r (the first 256 parts; more are
     // summed here), and for the residual epilogue wave 0's piece of the stream and of the next norm's weight.
-    float pv[8], part = 0.f;
+    constexpr int NPV = 256 / (GD_WAVES * 4);
+    float pv[NPV], part = 0.f;
     if (SCALED) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < NPV; ++i) {
             const int p = wave * 4 + g + GD_WAVES * 4 * i;
             pv[i] = p < n_parts ? ss_in[p * 16 + r] : 0.f;
         }
@@ -62,17 +69,18 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     f32x4_t acc[NT], acc2[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) { acc[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f}; acc2[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f}; }
-    const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)n_base * K * 2;
+    const size_t chunk_stride = (size_t)(NT * N / 16) * 4096;         // bytes of one chunk of all tiles
+    const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)blockIdx.x * 4096;
     unsigned woff[NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) woff[nt] = (unsigned)(nt * N / 16) * (unsigned)K * 32u + 16u * lane;
+    for (int nt = 0; nt < NT; ++nt) woff[nt] = (unsigned)(nt * N / 16) * 4096u + 16u * lane;
     const char* xbase = reinterpret_cast<const char*>(X);
     const unsigned xoff = (unsigned)min(r, M - 1) * (unsigned)K * 2u + 16u * g;
 
     bf16x8_t a0[NT][4], a1[NT][4], b0[4], b1[4];
 #define GD_LOAD(A, B, CHUNK)                                                                             \
     {                                                                                                    \
-        const char* wb_ = wbase + (size_t)(CHUNK) * 4096;                                                \
+        const char* wb_ = wbase + (size_t)(CHUNK) * chunk_stride;                                        \
         const char* xb_ = xbase + (size_t)(CHUNK) * (GD_CHUNK * 2) + xoff;                               \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                  \
             _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                            \
@@ -104,7 +112,7 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
 
     if (SCALED) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) part += pv[i];
+        for (int i = 0; i < NPV; ++i) part += pv[i];
         ss_red[(wave * 4 + g) * 16 + r] = part;
     }
     // ---- add the waves' tiles, in a fixed order ---------------------------------------------------------------
@@ -162,6 +170,20 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     }
 }
 
+struct GdArgs {
+    const bf16_t* x; const bf16_t* w; void* c; float* resid; bf16_t* xw_out; const bf16_t* w_next; float* ss_out; const float* ss_in;
+    int n_parts; float eps; int M, N, K; hipStream_t st;
+};
+
+// Blocks of 8 waves, one per 16 columns; the gated product (two tiles per block, usually three blocks per CU)
+// takes blocks of GD_WAVES_GATED waves so that all of them are resident at once.
+template <int EPI, bool SCALED, typename TC>
+static void gd_launch(const GdArgs& a) {
+    constexpr int W = EPI == EPI_GATED ? GD_WAVES_GATED : 8;
+    gemm_decode_kernel<EPI, SCALED, TC, W><<<a.N / 16, W * 64, 0, a.st>>>(a.x, a.w, (TC*)a.c, a.resid, a.xw_out, a.w_next, a.ss_out, a.ss_in,
+                                                                        a.n_parts, a.eps, a.M, a.N, a.K);
+}
+
 // x: bfloat16 [M, K].  scaled != 0: x = bf16(h * w_norm) and ss_in [n_parts, 16] holds the parts of sum(h^2); the
 // result is multiplied by rsqrt(sum / K + eps).
 // epi 0: C [M, N] (c_dtype);  epi 1: W = [gate | up], C [M, N] = silu(gate) * up;  epi 2: resid [M, N] += result,
@@ -178,20 +200,17 @@ extern "C" int spy_gemm_decode(const void* X, int scaled, const float* ss_in, in
                                      ((uintptr_t)xw_out % 8) == 0 && ((uintptr_t)w_next % 8) == 0),
                 "spy_gemm_decode: the residual epilogue needs the stream, the next norm's weight and its outputs");
     SPY_REQUIRE(epi == EPI_RESID || (C && ((uintptr_t)C % 16) == 0), "spy_gemm_decode: no output");
-    SPY_REQUIRE((long long)(N + 16) * K * 2 < (1ll << 32), "spy_gemm_decode: the matrix is too large for 32-bit offsets inside a block");
-    const bf16_t* x = (const bf16_t*)X;
-    const bf16_t* w = (const bf16_t*)Wt;
-    const int blocks = N / 16;
-#define GD_LAUNCH(EPI_, SCALED_, TC_)                                                                             \
-    gemm_decode_kernel<EPI_, SCALED_, TC_><<<blocks, GD_WAVES * 64, 0, st>>>(x, w, (TC_*)C, resid, (bf16_t*)xw_out, (const bf16_t*)w_next, \
-                                                                             ss_out, ss_in, n_parts, eps, M, N, K)
-#define GD_TYPES(EPI_, SCALED_)                                                  \
-    if (c_dtype == SPY_F32) GD_LAUNCH(EPI_, SCALED_, float); else GD_LAUNCH(EPI_, SCALED_, bf16_t)
-    if (epi == EPI_RESID) { if (scaled) GD_LAUNCH(EPI_RESID, true, bf16_t); else GD_LAUNCH(EPI_RESID, false, bf16_t); }
-    else if (epi == EPI_GATED) { if (scaled) { GD_TYPES(EPI_GATED, true); } else { GD_TYPES(EPI_GATED, false); } }
-    else { if (scaled) { GD_TYPES(EPI_STORE, true); } else { GD_TYPES(EPI_STORE, false); } }
-#undef GD_TYPES
-#undef GD_LAUNCH
+    SPY_REQUIRE((long long)N * 256 + 8192 < (1ll << 32), "spy_gemm_decode: N = %d is too large for 32-bit offsets inside a chunk", N);
+    GdArgs a = {(const bf16_t*)X, (const bf16_t*)Wt, C, resid, (bf16_t*)xw_out, (const bf16_t*)w_next, ss_out, ss_in, n_parts, eps, M, N, K, st};
+    const bool f32 = c_dtype == SPY_F32;
+    if (epi == EPI_RESID) { if (scaled) gd_launch<EPI_RESID, true, bf16_t>(a); else gd_launch<EPI_RESID, false, bf16_t>(a); }
+    else if (epi == EPI_GATED) {
+        if (scaled) { if (f32) gd_launch<EPI_GATED, true, float>(a); else gd_launch<EPI_GATED, true, bf16_t>(a); }
+        else { if (f32) gd_launch<EPI_GATED, false, float>(a); else gd_launch<EPI_GATED, false, bf16_t>(a); }
+    } else {
+        if (scaled) { if (f32) gd_launch<EPI_STORE, true, float>(a); else gd_launch<EPI_STORE, true, bf16_t>(a); }
+        else { if (f32) gd_launch<EPI_STORE, false, float>(a); else gd_launch<EPI_STORE, false, bf16_t>(a); }
+    }
     SPY_CHECK_LAUNCH("spy_gemm_decode");
     return 0;
 }

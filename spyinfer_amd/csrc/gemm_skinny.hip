@@ -24,10 +24,8 @@ __device__ __forceinline__ bf16x8_t load8(const bf16_t* p, bool ok) {
 // GATED (with NT = 2): W holds [gate rows | up rows], N is the number of gate rows; tile 0 of a block is
 // 16 gate rows, tile 1 the 16 up rows of the same columns, and the block stores silu(gate) * up [M, N]:
 // the SwiGLU of a gated feed-forward without a pass of its own.
-// TILED: W is stored in the order the MFMA operands want it, [N/16 tiles][K/32 steps][64 lanes][8 values]
-// with lane = 16 g + r holding W[16 tile + r][32 step + 8 g ..]: every load of a wave is 1 KiB in one piece
-// (8 full cache lines instead of 16 half lines), which is what bounds this kernel.  N % 16 = 0, K % 128 = 0.
-template <int MT, int NT, int WAVES, typename TC, bool GATED = false, bool TILED = false>
+// (The products of at most 16 rows with weights copied into MFMA tile order are in gemm_decode.hip.)
+template <int MT, int NT, int WAVES, typename TC, bool GATED = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                                  TC* __restrict__ C, int M, int N, int K) {
     __shared__ float red[(WAVES - 1) * NT * MT * 64 * 4];
@@ -52,8 +50,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
     for (int nt = 0; nt < NT; ++nt) {
         const int row = GATED ? nt * N + min(n_base + r, N - 1) : min(n_base + nt * 16 + r, N - 1);
         woff[nt] = (unsigned)(row - n_base) * (unsigned)K * 2u + 16u * g;
-        // tiled: a tile's K/32 steps of 1 KiB follow each other; a lane's 16 bytes sit at 16 * lane
-        if (TILED) woff[nt] = (unsigned)((GATED ? nt * N : nt * 16) / 16) * (unsigned)K * 32u + 16u * lane;
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) xoff[mt] = (unsigned)min(mt * 16 + r, M - 1) * (unsigned)K * 2u + 16u * g;
@@ -72,11 +68,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
     bf16x8_t a0[NT][4], b0[MT][4], a1[NT][4], b1[MT][4];
 #define SK_LOAD(A, B, CHUNK)                                                                         \
     {                                                                                                \
-        const char* wb_ = wbase + (size_t)(CHUNK) * (TILED ? 4096 : SK_CHUNK * 2);                   \
+        const char* wb_ = wbase + (size_t)(CHUNK) * (SK_CHUNK * 2);                                  \
         const char* xb_ = xbase + (size_t)(CHUNK) * (SK_CHUNK * 2);                                  \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                              \
             _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                        \
-                A[nt][j] = *reinterpret_cast<const bf16x8_t*>(wb_ + woff[nt] + (TILED ? 1024 : 64) * j); \
+                A[nt][j] = *reinterpret_cast<const bf16x8_t*>(wb_ + woff[nt] + 64 * j);                  \
             _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                        \
                 B[mt][j] = load8(reinterpret_cast<const bf16_t*>(xb_ + xoff[mt] + 64 * j), xok[mt]); \
         }                                                                                            \
@@ -114,7 +110,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] += acc2[nt][mt];
     // the rest of K (fewer than 128 values; K is a multiple of 8), by the wave whose turn it is
-    if (!TILED && nfull * SK_CHUNK < K && wave == nfull % WAVES) {
+    if (nfull * SK_CHUNK < K && wave == nfull % WAVES) {
         const int kc = nfull * SK_CHUNK;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -193,39 +189,6 @@ static void pick_skinny(const bf16_t* X, const bf16_t* W, void* C, int M, int N,
     // Measured on MI355X at the Qwen3-8B shapes (N 4096..151936, K 4096..12288) with 1 and 8 rows:
     // one 16-row tile per block and 8 waves sharing K was the best or within 3 % of it everywhere.
     launch_skinny<MT, 1, 8, TC>(X, W, C, M, N, K, st);
-}
-
-// Explicit configuration, for tuning runs: MT = 1 only.
-extern "C" int spy_gemm_skinny_cfg(const void* X, const void* W, void* C, int M, int N, int K, int nt, int waves, hipStream_t st) {
-    SPY_REQUIRE(M > 0 && M <= 16 && K % 8 == 0, "spy_gemm_skinny_cfg: M <= 16 and K %% 8 == 0 expected");
-    const bf16_t* x = (const bf16_t*)X;
-    const bf16_t* w = (const bf16_t*)W;
-#define CFG(NT_, W_) if (nt == NT_ && waves == W_) { launch_skinny<1, NT_, W_, bf16_t>(x, w, C, M, N, K, st); SPY_CHECK_LAUNCH("cfg"); return 0; }
-    CFG(1, 2) CFG(1, 4) CFG(1, 8) CFG(1, 16) CFG(2, 2) CFG(2, 4) CFG(2, 8) CFG(2, 16) CFG(4, 2) CFG(4, 4) CFG(4, 8)
-#undef CFG
-    return spy_fail("spy_gemm_skinny_cfg: no such configuration");
-}
-
-// The same products with W in MFMA tile order (see the kernel).  gated != 0: W = [gate | up] tiles, N = gate rows.
-extern "C" int spy_gemm_skinny_tiled(const void* X, const void* Wt, void* C, int c_dtype, int M, int N, int K, int gated,
-                                     hipStream_t st) {
-    SPY_REQUIRE(M > 0 && N > 0 && K > 0, "spy_gemm_skinny_tiled: empty operand");
-    SPY_REQUIRE(M <= 16, "spy_gemm_skinny_tiled: M = %d exceeds 16 rows", M);
-    SPY_REQUIRE(N % 16 == 0 && K % 128 == 0, "spy_gemm_skinny_tiled: N = %d must be a multiple of 16 and K = %d of 128", N, K);
-    SPY_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)Wt % 16) == 0, "spy_gemm_skinny_tiled: operands must be 16-byte aligned");
-    SPY_REQUIRE((long long)(N + 16) * K * 2 < (1ll << 32), "spy_gemm_skinny_tiled: the gate and up tiles lie too far apart");
-    const bf16_t* x = (const bf16_t*)X;
-    const bf16_t* w = (const bf16_t*)Wt;
-    const int blocks = N / 16;
-    if (gated) {
-        if (c_dtype == SPY_F32) gemm_skinny_kernel<1, 2, 8, float, true, true><<<blocks, 8 * 64, 0, st>>>(x, w, (float*)C, M, N, K);
-        else gemm_skinny_kernel<1, 2, 8, bf16_t, true, true><<<blocks, 8 * 64, 0, st>>>(x, w, (bf16_t*)C, M, N, K);
-    } else {
-        if (c_dtype == SPY_F32) gemm_skinny_kernel<1, 1, 8, float, false, true><<<blocks, 8 * 64, 0, st>>>(x, w, (float*)C, M, N, K);
-        else gemm_skinny_kernel<1, 1, 8, bf16_t, false, true><<<blocks, 8 * 64, 0, st>>>(x, w, (bf16_t*)C, M, N, K);
-    }
-    SPY_CHECK_LAUNCH("spy_gemm_skinny_tiled");
-    return 0;
 }
 
 // out[M, I] = silu(X . Wgate^T) * (X . Wup^T) with W = [Wgate | Wup] stored [2 I, K]

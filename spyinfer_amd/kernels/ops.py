@@ -75,7 +75,7 @@ class _Hip:
                      "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_prefill",
                      "spy_attention_prefill_workspace", "spy_swiglu",
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
-                     "spy_gemm_skinny_tiled", "spy_gemm_decode", "spy_embedding_sumsq"):
+                     "spy_gemm_decode", "spy_embedding_sumsq"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: rebuild it (python -c 'import __graft_entry__ as g; g.build()')"
                                   % (self.lib._name, name))
@@ -171,18 +171,19 @@ _LIBRARY_F32_OUT = True      # torch.mm(..., out_dtype=float32) exists in this t
 #: then whole cache lines).  Costs the weights' size again in device memory; the row-major copy stays for the
 #: library product of prefill.
 TILED_WEIGHTS = True
+FUSED_DECODE_MAX_ROWS = 16   # rows of the decode kernel that reads the tiled copies
 
 
 def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
-    """``w [N, K]`` in the order the streaming MFMA kernel reads it: [N/16][K/32][g = 4][r = 16][8], the values
-    of lane 16 g + r being w[16 tile + r][32 step + 8 g ..].  None if the copy is switched off or the shape or
-    dtype does not allow it (then the kernel reads the row-major matrix)."""
+    """``w [N, K]`` in the order the decode kernel reads it: [K/128 chunks][N/16 tiles][4 steps][g = 4][r = 16][8], the
+    values of lane 16 g + r being w[16 tile + r][128 chunk + 32 step + 8 g ..].  None if the copy is switched off or
+    the shape or dtype does not allow it (then the kernel for row-major matrices stands)."""
     if not TILED_WEIGHTS or _impl is not None or not w.is_cuda or w.dtype != torch.bfloat16 or w.dim() != 2:
         return None
     N, K = w.shape
-    if N % 16 or K % 128:
+    if N % 16 or K % 128 or N * 256 + 8192 >= (1 << 32):
         return None
-    return w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(N, K)
+    return w.view(N // 16, 16, K // 128, 4, 4, 8).permute(2, 0, 3, 4, 1, 5).contiguous().view(N, K)
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
@@ -204,14 +205,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     if M == 0:
         return torch.empty((0, N), dtype=out_dtype, device=x.device)
     all_bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-    if all_bf16 and tiled is not None and M <= 16:
-        _dev(tiled)
-        _check(tiled.shape == w.shape and tiled.dtype == w.dtype and N % 16 == 0 and K % 128 == 0,
-               "linear: the tiled copy does not fit the matrix")
-        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
-        hip().call("spy_gemm_skinny_tiled", _ptr(x), _ptr(tiled), _ptr(out), _code(out, "out"), ctypes.c_int(M), ctypes.c_int(N),
-                   ctypes.c_int(K), ctypes.c_int(0), _Hip.stream())
-        return out
+    if all_bf16 and tiled is not None and M <= FUSED_DECODE_MAX_ROWS:
+        _check(tiled.shape == w.shape, "linear: the tiled copy does not fit the matrix")
+        return decode_linear(x, tiled, out_dtype)
     global _LIBRARY_F32_OUT
     if all_bf16 and out_dtype == torch.float32 and M > SKINNY_MAX_ROWS and _LIBRARY_F32_OUT:
         try:
@@ -241,14 +237,9 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, tiled: Optional[torc
            "linear_swiglu: x [M, K] and w [2 I, K] expected")
     M, K = x.shape
     I = w_gate_up.shape[0] // 2
-    if x.dtype == torch.bfloat16 and tiled is not None and 0 < M <= 16 and I % 16 == 0 and K % 128 == 0 \
-            and (I + 16) * K * 2 < (1 << 32):
-        _dev(tiled)
-        _check(tiled.shape == w_gate_up.shape and tiled.dtype == torch.bfloat16, "linear_swiglu: the tiled copy does not fit")
-        out = torch.empty((M, I), dtype=x.dtype, device=x.device)
-        hip().call("spy_gemm_skinny_tiled", _ptr(x), _ptr(tiled), _ptr(out), _code(out, "out"), ctypes.c_int(M), ctypes.c_int(I),
-                   ctypes.c_int(K), ctypes.c_int(1), _Hip.stream())
-        return out
+    if x.dtype == torch.bfloat16 and tiled is not None and 0 < M <= FUSED_DECODE_MAX_ROWS and I % 16 == 0:
+        _check(tiled.shape == w_gate_up.shape, "linear_swiglu: the tiled copy does not fit")
+        return decode_linear_swiglu(x, tiled)
     if x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 \
             and (I + 16) * K * 2 < (1 << 32):
         out = torch.empty((M, I), dtype=x.dtype, device=x.device)
@@ -274,7 +265,6 @@ class ScaledInput:
 
 #: False switches the folded decode products off (every norm then runs as a kernel of its own).
 FUSED_DECODE = True
-FUSED_DECODE_MAX_ROWS = 16
 
 
 def fused_decode_ok(rows: int, act_dtype, *tiled_weights) -> bool:
@@ -283,7 +273,7 @@ def fused_decode_ok(rows: int, act_dtype, *tiled_weights) -> bool:
     if not FUSED_DECODE or _impl is not None or act_dtype != torch.bfloat16 or not 0 < rows <= FUSED_DECODE_MAX_ROWS:
         return False
     return all(t is not None and t.dtype == torch.bfloat16 and t.shape[0] % 16 == 0 and t.shape[1] % 128 == 0
-               and (t.shape[0] + 16) * t.shape[1] * 2 < (1 << 32) for t in tiled_weights)
+               for t in tiled_weights)
 
 
 def _gemm_decode(x, tiled: torch.Tensor, epi: int, n_out: int, out, resid, xw_out, w_next, ss_out) -> None:
