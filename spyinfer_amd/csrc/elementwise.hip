@@ -311,6 +311,112 @@ __global__ __launch_bounds__(QK_WAVES * 64) void qknorm_rope_store_kernel(
     }
 }
 
+// The same for many tokens of bfloat16 with the whole head rotated (rot == d) and d in {16, 32, 64, 128, 256}:
+// d / 16 lanes per (token, q or k head), each with 8 + 8 values that pair up in the rotation, so all loads and
+// stores are 16 bytes; and the values of 16 tokens of a kv head go through LDS, so that 8 tokens that follow each
+// other in a page are stored as one 16-byte piece of each row of the transposed page (single stores otherwise).
+// Blocks [0, qk_blocks) do q and k, the rest one (16 tokens, kv head) tile of v each.
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t qk_u32x4;
+template <typename TW, int LPH>
+__global__ __launch_bounds__(256) void qknorm_rope_store_vec_kernel(
+    const bf16_t* __restrict__ qkv, bf16_t* __restrict__ q_out, int T, int n_q, int n_kv, const TW* __restrict__ qw,
+    const TW* __restrict__ kw, float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int max_pos,
+    const int* __restrict__ positions, bf16_t* __restrict__ kc, bf16_t* __restrict__ vc, int P, int num_pages,
+    const int* __restrict__ slots, int qk_blocks) {
+    constexpr int d = LPH * 16, half = LPH * 8;
+    __shared__ __align__(16) bf16_t tile[16 * (d + 8)];
+    const int heads = n_q + 2 * n_kv, qk_heads = n_q + n_kv;
+    if ((int)blockIdx.x < qk_blocks) {
+        const long long u = (long long)blockIdx.x * (256 / LPH) + threadIdx.x / LPH;
+        const int sub = threadIdx.x % LPH;
+        if (u >= (long long)T * qk_heads) return;
+        const int t = (int)(u / qk_heads), h = (int)(u % qk_heads);
+        const bool is_q = h < n_q;
+        int page = 0, off = 0;
+        if (!is_q) {
+            if (!slots) return;
+            const int slot = slots[t];
+            if (slot < 0 || slot >= num_pages * P) return;      // (all LPH lanes of a head take the same way)
+            page = slot / P;
+            off = slot - page * P;
+        }
+        const bf16_t* x = qkv + (size_t)t * heads * d + (size_t)h * d + 8 * sub;
+        const qk_u32x4 ra = *reinterpret_cast<const qk_u32x4*>(x), rb = *reinterpret_cast<const qk_u32x4*>(x + half);
+        float a[8], b[8], ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            a[2 * i] = __uint_as_float(ra[i] << 16); a[2 * i + 1] = __uint_as_float(ra[i] & 0xffff0000u);
+            b[2 * i] = __uint_as_float(rb[i] << 16); b[2 * i + 1] = __uint_as_float(rb[i] & 0xffff0000u);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += a[i] * a[i] + b[i] * b[i];
+        const TW* w = is_q ? qw : kw;
+        if (w) {
+#pragma unroll
+            for (int o = 1; o < LPH; o <<= 1) ss += __shfl_xor(ss, o, 64);
+            const float scale = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                a[i] = (scale * a[i]) * to_f32<TW>(w[8 * sub + i]);
+                b[i] = (scale * b[i]) * to_f32<TW>(w[half + 8 * sub + i]);
+            }
+        }
+        int p = positions[t];
+        p = p < 0 ? 0 : (p >= max_pos ? max_pos - 1 : p);
+        const float* cp = cos_t + (size_t)p * half + 8 * sub;
+        const float* sp = sin_t + (size_t)p * half + 8 * sub;
+        float ya[8], yb[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float c = cp[i], sn = sp[i];
+            ya[i] = a[i] * c - b[i] * sn;
+            yb[i] = a[i] * sn + b[i] * c;
+        }
+        bf16_t* dst = (is_q ? q_out + ((size_t)t * n_q + h) * d : kc + (((size_t)page * n_kv + (h - n_q)) * P + off) * d) + 8 * sub;
+        const qk_u32x4 oa = {pack_bf16x2(ya[0], ya[1]), pack_bf16x2(ya[2], ya[3]), pack_bf16x2(ya[4], ya[5]), pack_bf16x2(ya[6], ya[7])};
+        const qk_u32x4 ob = {pack_bf16x2(yb[0], yb[1]), pack_bf16x2(yb[2], yb[3]), pack_bf16x2(yb[4], yb[5]), pack_bf16x2(yb[6], yb[7])};
+        *reinterpret_cast<qk_u32x4*>(dst) = oa;
+        *reinterpret_cast<qk_u32x4*>(dst + half) = ob;
+        return;
+    }
+    // ---- values: 16 tokens of one kv head ---------------------------------------------------------------------
+    const int vb = blockIdx.x - qk_blocks;
+    const int t0 = (vb / n_kv) * 16, hv = vb % n_kv;
+    for (int i = threadIdx.x; i < 16 * (d / 8); i += 256) {
+        const int tt = i / (d / 8), c8 = i % (d / 8);
+        qk_u32x4 v = {0u, 0u, 0u, 0u};
+        if (t0 + tt < T) v = *reinterpret_cast<const qk_u32x4*>(qkv + (size_t)(t0 + tt) * heads * d + (size_t)(qk_heads + hv) * d + 8 * c8);
+        *reinterpret_cast<qk_u32x4*>(tile + tt * (d + 8) + 8 * c8) = v;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 2 * d; i += 256) {
+        const int j = i % d, tg = i / d;                      // dim j of tokens t0 + 8 tg .. + 7
+        const int tb = t0 + 8 * tg;
+        if (tb >= T) continue;
+        const int s0 = slots[tb];
+        bool run = tb + 8 <= T && s0 >= 0 && s0 % 8 == 0 && s0 + 8 <= num_pages * P;
+        if (run) {
+#pragma unroll
+            for (int e = 1; e < 8; ++e) run = run && slots[tb + e] == s0 + e;
+        }
+        if (run) {                                            // P is a multiple of 8: the 8 slots lie in one page
+            uint32_t pk[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                pk[e] = (uint32_t)tile[(8 * tg + 2 * e) * (d + 8) + j] | ((uint32_t)tile[(8 * tg + 2 * e + 1) * (d + 8) + j] << 16);
+            const int page = s0 / P, off = s0 - page * P;
+            *reinterpret_cast<qk_u32x4*>(vc + (((size_t)page * n_kv + hv) * d + j) * P + off) = qk_u32x4{pk[0], pk[1], pk[2], pk[3]};
+        } else {
+            for (int e = 0; e < 8 && tb + e < T; ++e) {
+                const int slot = slots[tb + e];
+                if (slot < 0 || slot >= num_pages * P) continue;
+                const int page = slot / P, off = slot - page * P;
+                vc[(((size_t)page * n_kv + hv) * d + j) * P + off] = tile[(8 * tg + e) * (d + 8) + j];
+            }
+        }
+    }
+}
+
 extern "C" int spy_qknorm_rope_store(const void* qkv, int dtype, void* q_out, int T, int n_q, int n_kv, int d, const void* qw,
                                      const void* kw, int w_dtype, float eps, const float* cos_t, const float* sin_t, int rot,
                                      int max_pos, const int* positions, void* kc, void* vc, int P, int num_pages,
@@ -321,8 +427,32 @@ extern "C" int spy_qknorm_rope_store(const void* qkv, int dtype, void* q_out, in
     SPY_REQUIRE(rot == 0 || (cos_t && sin_t && max_pos > 0), "spy_qknorm_rope_store: rotation without tables");
     SPY_REQUIRE(!slots || (kc && vc && P > 0 && num_pages > 0), "spy_qknorm_rope_store: slots without a cache");
     SPY_REQUIRE(n_q + 2 * n_kv <= 65535 * QK_WAVES, "spy_qknorm_rope_store: too many heads");
-    const dim3 grid(T, (n_q + 2 * n_kv + QK_WAVES - 1) / QK_WAVES);
     const int wd = w_dtype < 0 ? SPY_F32 : w_dtype;
+    // many bfloat16 tokens, whole head rotated, a head size that is 16 times a power of two: the kernel with wide accesses
+    if (dtype == SPY_BF16 && T >= 64 && rot == d && (d == 16 || d == 32 || d == 64 || d == 128 || d == 256) && slots && P % 8 == 0 &&
+        ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)q_out % 16) == 0 && ((uintptr_t)kc % 16) == 0 && ((uintptr_t)vc % 16) == 0 &&
+        (!qw) == (!kw)) {
+        const int lph = d / 16;
+        const long long units = (long long)T * (n_q + n_kv);
+        const long long qk_blocks = (units + 256 / lph - 1) / (256 / lph);
+        const long long v_blocks = (long long)((T + 15) / 16) * n_kv;
+        SPY_REQUIRE(qk_blocks + v_blocks < (1ll << 31), "spy_qknorm_rope_store: too many tokens");
+#define QKV_CASE(L)                                                                                                             \
+    SPY_DISPATCH(wd, TW, (qknorm_rope_store_vec_kernel<TW, L><<<(unsigned)(qk_blocks + v_blocks), 256, 0, st>>>(               \
+        (const bf16_t*)qkv, (bf16_t*)q_out, T, n_q, n_kv, (const TW*)qw, (const TW*)kw, eps, cos_t, sin_t, max_pos, positions,  \
+        (bf16_t*)kc, (bf16_t*)vc, P, num_pages, slots, (int)qk_blocks)))
+        switch (lph) {
+            case 1: QKV_CASE(1); break;
+            case 2: QKV_CASE(2); break;
+            case 4: QKV_CASE(4); break;
+            case 8: QKV_CASE(8); break;
+            default: QKV_CASE(16); break;
+        }
+#undef QKV_CASE
+        SPY_CHECK_LAUNCH("spy_qknorm_rope_store");
+        return 0;
+    }
+    const dim3 grid(T, (n_q + 2 * n_kv + QK_WAVES - 1) / QK_WAVES);
     SPY_DISPATCH(dtype, TA, SPY_DISPATCH(wd, TW, (qknorm_rope_store_kernel<TA, TW><<<grid, QK_WAVES * 64, 0, st>>>(
         (const TA*)qkv, (TA*)q_out, n_q, n_kv, d, (const TW*)qw, (const TW*)kw, eps, cos_t, sin_t, rot, max_pos, positions,
         (TA*)kc, (TA*)vc, P, num_pages, slots))));

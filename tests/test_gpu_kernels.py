@@ -265,12 +265,17 @@ def plain_qk(qkv, n_q, n_kv, d, qw, kw, eps, theta, rot, pos):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_q,n_kv,d,rot,P,norm", [(4, 2, 16, 16, 16, True), (8, 2, 32, 32, 8, True), (6, 3, 48, 48, 16, True),
-                                                   (3, 1, 80, 40, 4, False), (32, 8, 128, 128, 16, True), (5, 5, 256, 256, 32, True)])
-def test_qk_norm_rope_store(dtype, n_q, n_kv, d, rot, P, norm):
+                                                   (3, 1, 80, 40, 4, False), (32, 8, 128, 128, 16, True), (5, 5, 256, 256, 32, True),
+                                                   (2, 2, 64, 64, 16, False)])
+@pytest.mark.parametrize("T", [23, 150])
+def test_qk_norm_rope_store(dtype, n_q, n_kv, d, rot, P, norm, T):
+    """T = 150 takes, in bfloat16 and for head sizes that allow it, the kernel with 16-byte accesses; its slots hold runs
+    of tokens that follow each other in a page from an aligned slot (stored in pieces of 8), runs from an unaligned
+    slot, scattered slots and a token without a slot."""
     from spyinfer_amd.kernels import ops
     from spyinfer_amd.parts.rotary import RotaryEmbedding
     dev = require_gpu()
-    T, pages, theta, eps = 23, 9, 12345.0, 1e-5
+    pages, theta, eps = (9 if T == 23 else 2 * T // P + 4), 12345.0, 1e-5
     qkv = rnd((T, (n_q + 2 * n_kv) * d), dtype, dev, 10)
     qw = (1 + 0.2 * rnd((d,), torch.float32, dev, 11)).to(dtype) if norm else None
     kw = (1 + 0.2 * rnd((d,), torch.float32, dev, 12)).to(dtype) if norm else None
@@ -278,6 +283,10 @@ def test_qk_norm_rope_store(dtype, n_q, n_kv, d, rot, P, norm):
     rope = RotaryEmbedding(d, theta, rot)
     rope.prepare(dev, 512)
     slots = torch.randperm(pages * P, generator=torch.Generator().manual_seed(14))[:T].int()
+    if T > 100:
+        free = [x for x in range(120, pages * P)]
+        rest = torch.tensor(free)[torch.randperm(len(free), generator=torch.Generator().manual_seed(15))][:T - 75].int()
+        slots = torch.cat([torch.arange(8, 8 + 45).int(), torch.arange(67, 67 + 30).int(), rest])
     slots[3] = -1
     kc = torch.full((pages, n_kv, P, d), 7.0, dtype=dtype, device=dev)
     vc = torch.full((pages, n_kv, d, P), 7.0, dtype=dtype, device=dev)
