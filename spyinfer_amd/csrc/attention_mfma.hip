@@ -16,6 +16,13 @@
 //                   (d row, g) loads the 8 keys c0 + 8g .. +7 of row d with one 16-byte load.
 // Keys lie [key][d] within a page: lane (key, g) loads 16 bytes K[key][32 kk + 8 g ..].
 // With several parts per tile the partial (O, m, l) go to a workspace and a second kernel merges.
+//
+// FUSED (steps in which every entry is a single token, head_dim 64, 128 or 256, whole head rotated): the kernel reads
+// the raw q, k, v of the step's product itself.  A query row's values lie in one lane and the three lanes beside it the
+// way the rotation pairs them (dims j and j + d/2 are 32-wide chunks kk and kk + KK/2 of the same lane), so the
+// per-head RMS norm costs two lane exchanges and the rotation none.  The entry's new key is prepared the same way
+// by every lane for its own 8-value pieces, put in the place of the cache's row in the one block and round that reach
+// its position, and stored to the cache from there; so is the new value.  No other block reads that position.
 // (Letting the block that finishes last merge, found with a counter and device-scope fences, was
 // measured slower: 26 us against 17 us at 8 requests, because each fence writes back and invalidates L2.)
 #include "common.h"
@@ -24,17 +31,91 @@
 
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 
 __device__ __forceinline__ bf16x8_t zero8() { return bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
 
 #define AW 4   // waves per block
 
-template <int DMAX>
-__global__ __launch_bounds__(AW * 64) void attention_mfma_kernel(
-    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+// What the fused variant needs beside the cache: the step's raw [q | k | v] rows, the norm weights, the rotation tables.
+struct FusedQKV {
+    const bf16_t* qkv;      // [T, (n_q + 2 n_kv) d]
+    const void* qw;         // [d] or null (no norm)
+    const void* kw;
+    int w_dtype;
+    float eps;
+    const float* cos_t;     // [max_pos, d / 2], null: no rotation
+    const float* sin_t;
+    int max_pos;
+    int store;              // 0: the new key and value are neither stored nor used (the cache of another call is read)
+};
+
+// This lane's pieces (dims 32 kk + 8 g + e) of a [d] weight vector, as float.
+template <int KK>
+__device__ __forceinline__ void load_weight_pieces(float (&wv)[KK][8], const void* w, int dtype, int g) {
+    if (dtype == SPY_F32) {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(reinterpret_cast<const float*>(w) + kk * 32 + 8 * g);
+            const f32x4_t hi = *reinterpret_cast<const f32x4_t*>(reinterpret_cast<const float*>(w) + kk * 32 + 8 * g + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { wv[kk][e] = lo[e]; wv[kk][e + 4] = hi[e]; }
+        }
+    } else {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(reinterpret_cast<const bf16_t*>(w) + kk * 32 + 8 * g);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) wv[kk][e] = bf16_to_f32((bf16_t)v[e]);
+        }
+    }
+}
+
+// Raw head row -> normed and rotated, for this lane's pieces.  `x` holds the raw pieces; wv the norm weight's pieces
+// (used if normed); cs, sn the cosines and sines of dims 32 kk + 8 g + e, kk < KK / 2 (used if rotated).
+template <int KK>
+__device__ __forceinline__ void norm_rotate(bf16x8_t (&x)[KK], bool normed, const float (&wv)[KK][8], float eps, bool rotated,
+                                            const float (&cs)[KK / 2][8], const float (&sn)[KK / 2][8], int d) {
+    float v[KK][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { v[kk][e] = bf16_to_f32((bf16_t)x[kk][e]); ss += v[kk][e] * v[kk][e]; }
+    if (normed) {
+        ss += __shfl_xor(ss, 16, 64);
+        ss += __shfl_xor(ss, 32, 64);
+        const float scale = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[kk][e] = (scale * v[kk][e]) * wv[kk][e];
+    }
+    if (rotated) {
+        constexpr int HK = KK / 2;
+#pragma unroll
+        for (int kk = 0; kk < HK; ++kk)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float a = v[kk][e], b = v[kk + HK][e];
+                v[kk][e] = a * cs[kk][e] - b * sn[kk][e];
+                v[kk + HK][e] = a * sn[kk][e] + b * cs[kk][e];
+            }
+    }
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        const u32x4_t pk = {pack_bf16x2(v[kk][0], v[kk][1]), pack_bf16x2(v[kk][2], v[kk][3]), pack_bf16x2(v[kk][4], v[kk][5]),
+                            pack_bf16x2(v[kk][6], v[kk][7])};
+        x[kk] = __builtin_bit_cast(bf16x8_t, pk);
+    }
+}
+
+template <int DMAX, bool FUSED>
+__global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void attention_mfma_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, bf16_t* kc, bf16_t* vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
-    int n_q, int n_kv, int d, float scale, int window, int splits, float* __restrict__ ws) {
+    int n_q, int n_kv, int d, float scale, int window, int splits, float* __restrict__ ws, FusedQKV fz) {
     constexpr int KK = DMAX / 32;   // 32-wide chunks of the head dim for Q.K
     constexpr int DT = DMAX / 16;   // 16-row tiles of the head dim for P.V
     extern __shared__ float lds[];   // (AW - 1) * (DT * 4 + 2) * 64 floats: the other waves' O, m, l
@@ -61,7 +142,7 @@ __global__ __launch_bounds__(AW * 64) void attention_mfma_kernel(
 
     bf16x8_t bq[KK];
     {
-        const bf16_t* qp = q + ((size_t)(q0 + tq) * n_q + head) * d;
+        const bf16_t* qp = FUSED ? fz.qkv + ((size_t)(q0 + tq) * (n_q + 2 * n_kv) + head) * d : q + ((size_t)(q0 + tq) * n_q + head) * d;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
             const int dofs = kk * 32 + 8 * g;
@@ -81,6 +162,50 @@ __global__ __launch_bounds__(AW * 64) void attention_mfma_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
+
+    // FUSED: the entry's one new token lies at position p0 = kvl - 1; its query rows have that position too.  The block
+    // whose keys reach it prepares the new key (every lane its pieces for its g, as for q) and takes the new value's
+    // elements of its rows dd.  All loads of this preparation are issued together, before anything waits for them.
+    const int newpos = p0;
+    bool has_new = false;
+    bf16x8_t knew[KK];
+    bf16_t vnew[DT];
+    int new_page = -1;
+    if (FUSED) {
+        constexpr int HK = KK / 2;
+        has_new = fz.store && n == 1 && newpos >= lo + 32 * b_begin && newpos < lo + 32 * b_end;
+        const bool normed = fz.qw != nullptr, rotated = fz.cos_t != nullptr;
+        float wq[KK][8], wk[KK][8], cs[HK][8], sn[HK][8];
+        if (has_new) {
+            const bf16_t* base = fz.qkv + (size_t)q0 * (n_q + 2 * n_kv) * d;
+            const bf16_t* kp_raw = base + (size_t)(n_q + hk) * d;
+            const bf16_t* vp_raw = base + (size_t)(n_q + n_kv + hk) * d;
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) knew[kk] = *reinterpret_cast<const bf16x8_t*>(kp_raw + kk * 32 + 8 * g);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vnew[dt] = vp_raw[dt * 16 + r16];
+            new_page = bt[newpos / P];
+            if (normed) load_weight_pieces<KK>(wk, fz.kw, fz.w_dtype, g);
+        }
+        if (normed) load_weight_pieces<KK>(wq, fz.qw, fz.w_dtype, g);
+        if (rotated) {
+            const size_t trow = (size_t)min(newpos, fz.max_pos - 1) * (d / 2);
+#pragma unroll
+            for (int kk = 0; kk < HK; ++kk) {
+                const f32x4_t c0 = *reinterpret_cast<const f32x4_t*>(fz.cos_t + trow + kk * 32 + 8 * g);
+                const f32x4_t c1 = *reinterpret_cast<const f32x4_t*>(fz.cos_t + trow + kk * 32 + 8 * g + 4);
+                const f32x4_t s0 = *reinterpret_cast<const f32x4_t*>(fz.sin_t + trow + kk * 32 + 8 * g);
+                const f32x4_t s1 = *reinterpret_cast<const f32x4_t*>(fz.sin_t + trow + kk * 32 + 8 * g + 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { cs[kk][e] = c0[e]; cs[kk][e + 4] = c1[e]; sn[kk][e] = s0[e]; sn[kk][e + 4] = s1[e]; }
+            }
+        }
+        norm_rotate<KK>(bq, normed, wq, fz.eps, rotated, cs, sn, d);
+        if (has_new) {
+            norm_rotate<KK>(knew, normed, wk, fz.eps, rotated, cs, sn, d);
+            if (new_page < 0 || new_page >= num_pages) has_new = false;   // no page: nothing to store or to use
+        }
+    }
 
     // Pages are looked up one block ahead, both lookups together, and a block's K and V loads are
     // all issued before its first product: a block costs one memory round trip, not four.
@@ -116,6 +241,31 @@ __global__ __launch_bounds__(AW * 64) void attention_mfma_kernel(
         for (int dt = 0; dt < DT; ++dt) {
             const int dd = dt * 16 + r16;
             vt[dt] = (v_ok && dd < d) ? *reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P) : zero8();
+        }
+        if (FUSED && has_new && newpos >= c0 && newpos < c0 + 32) {
+            // the new key: the four lanes of its row take the prepared pieces; the lanes with r16 % 16 == its row store it
+            const bool mine_a = key_a == newpos, mine_b = key_a + 4 == newpos;
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                if (mine_a) ka[kk] = knew[kk];
+                if (mine_b) kb[kk] = knew[kk];
+            }
+            if (mine_a || mine_b) {
+                bf16_t* dst = kc + (((size_t)new_page * n_kv + hk) * P + newpos % P) * d + 8 * g;
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) *reinterpret_cast<bf16x8_t*>(dst + kk * 32) = knew[kk];
+            }
+            // the new value: element newpos - key_v of the lanes whose 8 keys hold it
+            const int jn = newpos - key_v;
+            if (jn >= 0 && jn < 8) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (j == jn) vt[dt][j] = (short)vnew[dt];
+                    vc[(((size_t)new_page * n_kv + hk) * d + dt * 16 + r16) * P + newpos % P] = vnew[dt];
+                }
+            }
         }
         const int v_valid = min(8, kvl - key_v);                  // keys of the group that exist (slots beyond hold anything)
         // the next block's pages
@@ -251,10 +401,14 @@ extern "C" int64_t spy_attention_mfma_workspace(int num_tiles, int n_kv, int d, 
     return (int64_t)num_tiles * n_kv * splits * 16 * (dmax_of(d) + 2);
 }
 
-extern "C" int spy_attention_mfma(void* out, const void* q, const void* kc, const void* vc, int P, int num_pages, const int* cu_q,
+// qkv != null: the fused variant (see the top of the file).  Then q is not read, every entry must be a single token
+// (T == S), head_dim 64, 128 or 256 with the whole head rotated (or no rotation: cos_t == null), and the new keys and
+// values are written to kc and vc by this call (store != 0).
+extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, int P, int num_pages, const int* cu_q,
                                   const int* pos0, const int* kv_len, const int* block_table, int max_blocks, const int* tile_entry,
                                   const int* tile_row0, int num_tiles, int S, int T, int n_q, int n_kv, int d, float scale,
-                                  int window, int splits, float* ws, hipStream_t st) {
+                                  int window, int splits, float* ws, const void* qkv, const void* qw, const void* kw, int w_dtype,
+                                  float eps, const float* cos_t, const float* sin_t, int max_pos, int store, hipStream_t st) {
     SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
                 "spy_attention_mfma: empty operand");
     SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 256, "spy_attention_mfma: head_dim %d is not a multiple of 16 in 16..256", d);
@@ -263,12 +417,25 @@ extern "C" int spy_attention_mfma(void* out, const void* q, const void* kc, cons
     SPY_REQUIRE(splits >= 1 && splits <= 64, "spy_attention_mfma: %d parts (1..64 allowed)", splits);
     SPY_REQUIRE(splits == 1 || ws, "spy_attention_mfma: parts without a workspace");
     SPY_REQUIRE(n_kv <= 65535, "spy_attention_mfma: too many kv heads");
+    FusedQKV fz = {(const bf16_t*)qkv, qw, kw, w_dtype, eps, cos_t, sin_t, max_pos, store};
+    if (qkv) {
+        SPY_REQUIRE(T == S && num_tiles == S, "spy_attention_mfma: the fused variant takes single tokens only (%d tokens of %d entries)", T, S);
+        SPY_REQUIRE(d == 64 || d == 128 || d == 256, "spy_attention_mfma: the fused variant takes head_dim 64, 128 or 256, not %d", d);
+        SPY_REQUIRE((!cos_t) == (!sin_t) && (!cos_t || max_pos > 0), "spy_attention_mfma: rotation tables are incomplete");
+        SPY_REQUIRE((!qw) == (!kw) && (!qw || w_dtype == SPY_F32 || w_dtype == SPY_BF16), "spy_attention_mfma: norm weights are incomplete");
+        SPY_REQUIRE(n_q / n_kv <= 16, "spy_attention_mfma: the fused variant takes groups of at most 16 heads");
+        SPY_REQUIRE(((uintptr_t)qkv % 16) == 0, "spy_attention_mfma: qkv must be 16-byte aligned");
+    } else {
+        SPY_REQUIRE(q, "spy_attention_mfma: no queries");
+    }
     const dim3 grid(num_tiles, n_kv, splits);
     const dim3 mgrid(num_tiles, n_kv);
+#define ATT_LAUNCH(DM, FZ)                                                                                                    \
+    attention_mfma_kernel<DM, FZ><<<grid, AW * 64, (AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>(                \
+        (bf16_t*)out, (const bf16_t*)q, (bf16_t*)kc, (bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,  \
+        tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz)
 #define ATT_CASE(DM)                                                                                                          \
-    attention_mfma_kernel<DM><<<grid, AW * 64, (AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, P,    \
-                                                   num_pages, cu_q, pos0, kv_len, block_table, max_blocks, tile_entry,        \
-                                                   tile_row0, n_q, n_kv, d, scale, window, splits, ws);                       \
+    if (qkv) ATT_LAUNCH(DM, true); else ATT_LAUNCH(DM, false);                                                                \
     if (splits > 1)                                                                                                           \
         attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits, 1);
     switch (dmax_of(d)) {
@@ -277,6 +444,7 @@ extern "C" int spy_attention_mfma(void* out, const void* q, const void* kc, cons
         default: ATT_CASE(256) break;
     }
 #undef ATT_CASE
+#undef ATT_LAUNCH
     SPY_CHECK_LAUNCH("spy_attention_mfma");
     return 0;
 }

@@ -432,15 +432,57 @@ def mfma_attention_ok(dtype, d: int, page_size: int) -> bool:
     return MFMA_ATTENTION and dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256 and page_size % 8 == 0
 
 
-def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_size: int, meta: AttentionMeta,
-                    n_q: int, n_kv: int, d: int, scale: float, window: Optional[int]) -> torch.Tensor:
+class RawQKV:
+    """The step's raw product [q | k | v] with what turns it into queries, keys and values: the per-head norm weights
+    (or None), eps, the rotation tables (or None) and whether this call stores its keys and values.  Handed to
+    ``paged_attention`` in place of q when ``fused_attention_ok`` allows it: the attention kernel then does the norm,
+    the rotation and the store itself (no kernel of their own in a decode step)."""
+    __slots__ = ("qkv", "q_norm_w", "k_norm_w", "eps", "cos", "sin", "store")
+
+    def __init__(self, qkv, q_norm_w, k_norm_w, eps, cos, sin, store):
+        self.qkv, self.q_norm_w, self.k_norm_w, self.eps, self.cos, self.sin, self.store = qkv, q_norm_w, k_norm_w, eps, cos, sin, store
+
+
+FUSED_ATTENTION = True     # False: the norm, rotation and store always run as a kernel of their own
+
+
+def fused_attention_ok(dtype, meta: AttentionMeta, n_q: int, n_kv: int, d: int, page_size: int, rotary_dim: int, q_norm_w, k_norm_w) -> bool:
+    """True if this step's attention may take the raw product (``RawQKV``): every entry a single token, bfloat16,
+    head_dim 64, 128 or 256 rotated whole or not at all, 16-row tiles built for this group size."""
+    if not FUSED_ATTENTION or _impl is not None or not mfma_attention_ok(dtype, d, page_size):
+        return False
+    if meta.T != meta.S or meta.max_q_len != 1 or meta.tiles is None or meta.tiles_group != n_q // n_kv or n_q // n_kv > 16:
+        return False
+    if meta.tiles["small"][2] != meta.S or meta.tiles["big"][2] != 0:
+        return False
+    if d not in (64, 128, 256) or rotary_dim not in (0, d) or (q_norm_w is None) != (k_norm_w is None):
+        return False
+    return q_norm_w is None or (q_norm_w.dtype == k_norm_w.dtype and q_norm_w.dtype in _CODES)
+
+
+def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: torch.Tensor, page_size: int, meta: AttentionMeta,
+                    n_q: int, n_kv: int, d: int, scale: float, window: Optional[int], raw: Optional[RawQKV] = None) -> torch.Tensor:
     """Causal grouped-query attention of the step's query tokens over the paged cache
-    (which already holds this step's keys and values).  Query at position p reads keys
-    max(0, p - window + 1) .. p.  Scores, softmax and the weighted sum are float32."""
+    (which already holds this step's keys and values, or gets them from ``raw`` in this call).  Query at position p
+    reads keys max(0, p - window + 1) .. p.  Scores, softmax and the weighted sum are float32."""
     if _impl is not None:
         return _impl.paged_attention(q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window)
-    _dev(q, k_cache, v_cache, meta.cu_q, meta.pos0, meta.kv_len, meta.block_table, meta.token_entry, meta.positions)
     T, S = meta.T, meta.S
+    if raw is not None:
+        _dev(raw.qkv, raw.q_norm_w, raw.k_norm_w, raw.cos, raw.sin)
+        _check(raw.qkv.dtype == torch.bfloat16 and raw.qkv.shape == (T, (n_q + 2 * n_kv) * d), "paged_attention: raw qkv must be bfloat16 [T, (n_q + 2 n_kv) d]")
+        rot = 0 if raw.cos is None else d
+        _check(fused_attention_ok(raw.qkv.dtype, meta, n_q, n_kv, d, page_size, rot, raw.q_norm_w, raw.k_norm_w),
+               "paged_attention: this step cannot take the raw product (ops.fused_attention_ok)")
+        if raw.cos is not None:
+            _check(raw.cos.dtype == torch.float32 and raw.sin.dtype == torch.float32 and raw.cos.dim() == 2 and raw.cos.shape[1] == d // 2
+                   and raw.sin.shape == raw.cos.shape, "paged_attention: rotation tables must be float32 [positions, d / 2]")
+        if raw.q_norm_w is not None:
+            _check(raw.q_norm_w.shape == (d,) and raw.k_norm_w.shape == (d,), "paged_attention: head norm weights must be [d]")
+        for t in (raw.qkv, raw.q_norm_w, raw.k_norm_w, raw.cos, raw.sin):
+            _check(t is None or t.data_ptr() % 16 == 0, "paged_attention: operands of the raw product must be 16-byte aligned")
+        q = torch.empty((T, n_q * d), dtype=raw.qkv.dtype, device=raw.qkv.device)     # shape and dtype of the result only
+    _dev(q, k_cache, v_cache, meta.cu_q, meta.pos0, meta.kv_len, meta.block_table, meta.token_entry, meta.positions)
     _check(q.shape == (T, n_q * d), "paged_attention: q must be [T, n_q d]")
     _check(n_q % n_kv == 0, "paged_attention: n_q must be a multiple of n_kv")
     num_pages = k_cache.shape[0]
@@ -454,7 +496,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _check(meta.max_kv_len <= meta.max_blocks * page_size, "paged_attention: block tables are shorter than the longest request")
     win = 0 if window is None else int(window)
     _check(win >= 0, "paged_attention: window must be positive")
-    out = torch.empty_like(q)
+    out = q if raw is not None else torch.empty_like(q)
     if T == 0:
         return out
     group = n_q // n_kv
@@ -490,8 +532,17 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             ws_floats = hip().lib.spy_attention_mfma_workspace(ctypes.c_int(n_small), ctypes.c_int(n_kv), ctypes.c_int(d),
                                                                ctypes.c_int(splits))
             ws = torch.empty((max(1, ws_floats),), dtype=torch.float32, device=q.device)
-            hip().call("spy_attention_mfma", _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), *common, _ptr(small_entry),
-                       _ptr(small_row0), ctypes.c_int(n_small), *sizes, ctypes.c_int(splits), _ptr(ws), _Hip.stream())
+            if raw is not None:
+                wcode = _code(raw.q_norm_w, "head norm weight") if raw.q_norm_w is not None else F32
+                fused = (_ptr(raw.qkv), _ptr(raw.q_norm_w), _ptr(raw.k_norm_w), ctypes.c_int(wcode), ctypes.c_float(raw.eps),
+                         _ptr(raw.cos), _ptr(raw.sin), ctypes.c_int(0 if raw.cos is None else raw.cos.shape[0]),
+                         ctypes.c_int(1 if raw.store else 0))
+            else:
+                fused = (_ptr(None), _ptr(None), _ptr(None), ctypes.c_int(0), ctypes.c_float(0.0), _ptr(None), _ptr(None),
+                         ctypes.c_int(0), ctypes.c_int(0))
+            hip().call("spy_attention_mfma", _ptr(out), _ptr(None if raw is not None else q), _ptr(k_cache), _ptr(v_cache), *common,
+                       _ptr(small_entry), _ptr(small_row0), ctypes.c_int(n_small), *sizes, ctypes.c_int(splits), _ptr(ws), *fused,
+                       _Hip.stream())
         return out
     hip().call("spy_attention_generic", _ptr(out), _ptr(q), _code(q, "q"), _ptr(k_cache), _ptr(v_cache),
                ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(meta.kv_len), _ptr(meta.block_table),

@@ -76,11 +76,15 @@ class PagedAttention(Mixer):
             qkv = ops.linear(x, self.w_qkv, tiled=self.w_qkv_tiled)
         rot = self.position.rotary() if self.position is not None else None
         cos, sin, rdim = rot if rot is not None else (None, None, 0)
-        slots = batch.slot_mapping(cache.group) if store else None
-        q = ops.qk_norm_rope_store(qkv, nq, nkv, d, self.q_norm, self.k_norm,
-                                   self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
-                                   cos, sin, rdim, batch.positions, cache.k, cache.v, cache.page_size, slots)
+        eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
         meta = batch.attention_meta(cache.group, nq // nkv)
+        if ops.fused_attention_ok(qkv.dtype, meta, nq, nkv, d, cache.page_size, rdim, self.q_norm, self.k_norm):
+            # single tokens only: the attention kernel norms, rotates and stores by itself
+            raw = ops.RawQKV(qkv, self.q_norm, self.k_norm, eps, cos if rdim else None, sin if rdim else None, store)
+            return ops.paged_attention(None, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window, raw)
+        slots = batch.slot_mapping(cache.group) if store else None
+        q = ops.qk_norm_rope_store(qkv, nq, nkv, d, self.q_norm, self.k_norm, eps,
+                                   cos, sin, rdim, batch.positions, cache.k, cache.v, cache.page_size, slots)
         return ops.paged_attention(q, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window)
 
     def forward(self, x, batch, cache, store=True):

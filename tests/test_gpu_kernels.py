@@ -411,6 +411,71 @@ def test_paged_attention(dtype, case, mfma):
     close(out, ref, dtype, scale=2.0, what="attention case %d" % case)
 
 
+FUSED_CASES = [
+    # n_q, n_kv, d, P, cached tokens of each single-token entry, window, norm, rotation
+    (32, 8, 128, 16, [1151, 70, 2000, 0, 15, 16, 31, 32], None, True, True),
+    (4, 1, 64, 16, [5, 0, 200], None, False, True),
+    (8, 8, 256, 32, [300, 63, 64], 50, True, False),
+    (16, 1, 64, 8, [99, 7], None, True, True),
+    (6, 2, 128, 16, [33], 8, False, False),
+]
+
+
+@pytest.mark.parametrize("case", range(len(FUSED_CASES)))
+@pytest.mark.parametrize("wdtype", DTYPES)
+@pytest.mark.parametrize("fixed", [False, True])
+def test_attention_taking_the_raw_product(case, wdtype, fixed):
+    """Single tokens: the attention kernel norms and rotates q and the new key itself, uses the new key and value and
+    stores them.  The slots of the new tokens hold NaN before the call, so a kernel that read them before writing, or
+    did not write, fails; the rest of the cache must stay as it was.  Positions at the edges of pages and of 32-key
+    blocks; one and several parts of the keys (fixed shapes take 16 parts)."""
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.parts.rotary import RotaryEmbedding
+    dev = require_gpu()
+    n_q, n_kv, d, P, cached, window, norm, rotate = FUSED_CASES[case]
+    dtype, theta, eps = torch.bfloat16, 23456.0, 1e-5
+    entries = [(a, 1) for a in cached]
+    _q, kc, vc, bt, te, ps, meta = make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed=50 + case, window=window)
+    meta.fixed_shape = fixed
+    T = len(entries)
+    qkv = rnd((T, (n_q + 2 * n_kv) * d), dtype, "cpu", 60 + case)
+    qw = (1 + 0.2 * rnd((d,), torch.float32, "cpu", 61)).to(wdtype) if norm else None
+    kw = (1 + 0.2 * rnd((d,), torch.float32, "cpu", 62)).to(wdtype) if norm else None
+    pos = torch.tensor(cached, dtype=torch.int32)
+    rope = RotaryEmbedding(d, theta, d)
+    rope.prepare(dev, 2100)
+    rq, rk, rv = plain_qk(qkv, n_q, n_kv, d, qw, kw, eps, theta, d if rotate else 0, pos)
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    kc_dev, vc_dev = kc.clone(), vc.clone()
+    for s, a in enumerate(cached):
+        page = bt[s][a // P]
+        kc_ref[page, :, a % P, :] = rk[s].to(dtype)
+        vc_ref[page, :, :, a % P] = rv[s].to(dtype)
+        kc_dev[page, :, a % P, :] = float("nan")
+        vc_dev[page, :, :, a % P] = float("nan")
+    scale = 1.0 / math.sqrt(d)
+    ref = plain_paged_attention(rq.reshape(T, n_q * d).to(dtype), kc_ref, vc_ref, P, bt, te, ps, n_q, n_kv, d, scale, window)
+    kc_dev, vc_dev = kc_dev.to(dev), vc_dev.to(dev)
+    assert ops.fused_attention_ok(dtype, meta, n_q, n_kv, d, P, d if rotate else 0, qw, kw)
+    raw = ops.RawQKV(qkv.to(dev), None if qw is None else qw.to(dev), None if kw is None else kw.to(dev), eps,
+                     rope.cos if rotate else None, rope.sin if rotate else None, True)
+    out = ops.paged_attention(None, kc_dev, vc_dev, P, meta, n_q, n_kv, d, scale, window, raw)
+    close(out, ref, dtype, scale=3.0, what="fused attention case %d" % case)
+    same = lambda a, b: torch.equal(torch.nan_to_num(a.float().cpu(), nan=-77.0), torch.nan_to_num(b.float(), nan=-77.0))
+    assert same(vc_dev, vc_ref), "values must be stored unchanged, and nothing else written"
+    new = torch.zeros(kc.shape[:3], dtype=torch.bool)
+    for s, a in enumerate(cached):
+        new[bt[s][a // P], :, a % P] = True
+    assert same(kc_dev[~new.to(dev)], kc_ref[~new]), "keys of other positions must stay as they were"
+    close(kc_dev[new.to(dev)], kc_ref[new], dtype, scale=8.0, what="stored keys")
+    # store = False: nothing is written and the new position is not read (the cache of another call)
+    kc2, vc2 = kc_ref.to(dev), vc_ref.to(dev)
+    raw.store = False
+    out2 = ops.paged_attention(None, kc2, vc2, P, meta, n_q, n_kv, d, scale, window, raw)
+    close(out2, ref, dtype, scale=3.0, what="fused attention without store, case %d" % case)
+    assert same(kc2, kc_ref) and same(vc2, vc_ref)
+
+
 def test_attention_without_rotation_is_library_sdpa():
     """One request from an empty cache equals softmax(QK^T / sqrt(d) + causal) V of a library routine."""
     from spyinfer_amd.kernels import ops
