@@ -17,16 +17,19 @@
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
-#define PF_WAVES 4
-#define PF_ROWS 128      // rows per block
 #define PF_KEYS 64       // keys staged per round
+#define PF_ROWS 128      // rows per block
 #define PF_SLACK 8.0f    // a score may exceed the running maximum by 2^8 before the maximum is raised
-#define PF_KG (PF_KEYS / 8)   // groups of 8 keys per round
 
 __device__ __forceinline__ bf16x8_t pf_zero8() { return bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
 
-template <int DMAX>
-__global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
+// DFULL: head_dim == DMAX, so no part of the head-dim loops is conditional and the compiler may move the LDS reads of
+// a whole 32-key half ahead of its products.
+// RT: 16-row tiles per wave.  2 (4 waves per block): every K and V fragment read from LDS serves two row tiles.  1 (8
+// waves per block): for grids with one block per CU only, where 4 waves would leave every SIMD with a single wave and
+// nothing to run while that wave waits (measured at 2048 tokens: 60 % of the cycles were such waits).
+template <int DMAX, bool DFULL, int RT>
+__global__ __launch_bounds__(PF_ROWS / RT * 4, RT == 1 ? 1 : 2) void attention_prefill_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
@@ -34,7 +37,8 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     constexpr int KK = DMAX / 32, DT = DMAX / 16;
     constexpr int KLD = DMAX + 8;            // bf16 per staged key row
     constexpr int VLD = PF_KEYS + 8;         // bf16 per staged value row (one head dim, 64 keys)
-    constexpr int NV = PF_KEYS * DMAX / 8 / 256;   // 16-byte vectors per thread and operand per round
+    constexpr int NT = PF_ROWS / RT * 4;        // threads per block: a wave per 16 RT rows
+    constexpr int NV = PF_KEYS * DMAX / 8 / NT; // 16-byte vectors per thread and operand per round
     __shared__ __attribute__((aligned(16))) bf16_t ks[PF_KEYS * KLD];
     __shared__ __attribute__((aligned(16))) bf16_t vs[DMAX * VLD];
 
@@ -63,12 +67,12 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     const int d8 = d >> 3;
 
     // this lane's two query rows
-    bool row_ok[2];
-    int tq[2], head[2], pos[2], lo_row[2];
-    bf16x8_t bq[2][KK];
+    bool row_ok[RT];
+    int tq[RT], head[RT], pos[RT], lo_row[RT];
+    bf16x8_t bq[RT][KK];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        const int row = row0 + 32 * wave + 16 * t + r16;
+    for (int t = 0; t < RT; ++t) {
+        const int row = row0 + 16 * RT * wave + 16 * t + r16;
         row_ok[t] = row < nrows;
         tq[t] = row_ok[t] ? row / G : 0;
         head[t] = hk * G + (row_ok[t] ? row % G : 0);
@@ -87,25 +91,27 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     int lo = window > 0 ? max(0, p0 + row0 / G - window + 1) : 0;
     lo &= ~(PF_KEYS - 1);
     const int nblk = hi >= lo ? (hi - lo) / PF_KEYS + 1 : 0;
-    const int w_first_row = row0 + 32 * wave;
-    const int w_last_row = min(nrows, w_first_row + 32) - 1;
+    const int w_first_row = row0 + 16 * RT * wave;
+    const int w_last_row = min(nrows, w_first_row + 16 * RT) - 1;
     const int w_hi = w_last_row >= w_first_row ? p0 + w_last_row / G : -1;               // last key any row of the wave reads
     const int w_lo = window > 0 ? max(0, p0 + w_first_row / G - window + 1) : 0;           // first key any row of the wave reads
-    const bool w_rows_full = w_first_row + 31 < nrows;                                     // all 32 rows of the wave exist
+    const bool w_rows_full = w_first_row + 16 * RT - 1 < nrows;                             // all rows of the wave exist
     const int w_min_pos = p0 + w_first_row / G;                                            // keys up to here are before every row
     const int w_max_lo = window > 0 ? max(0, w_hi - window + 1) : 0;                       // keys from here on are in every window
     const float scale2 = scale * 1.4426950408889634f;                                      // scores times log2(e)
 
-    f32x4_t acc[2][DT];
+    f32x4_t acc[RT][DT];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < RT; ++t)
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) acc[t][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+    float m[RT], l[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) { m[t] = -INFINITY; l[t] = 0.f; }
 
     bf16x8_t pk[NV], pv[NV];
     int kpg[NV], vpg[NV];        // pages of this thread's vectors, looked up one round ahead of the data
-    // vector v = tid + 256 i of a round:  K: key = v / d8, chunk = v % d8 (16 bytes of one key row)
+    // vector v = tid + NT i of a round:  K: key = v / d8, chunk = v % d8 (16 bytes of one key row)
     //                                     V: kgrp = v % 8, dd = v / 8     (8 keys of one head dim)
     // What does not change from round to round is worked out once: the local key, the offsets inside a
     // page and the places in LDS.  Pages are powers of two here, so a key's page is a shift away.
@@ -113,7 +119,7 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     bool v_on[NV];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        const int v = tid + 256 * i;
+        const int v = tid + NT * i;
         v_on[i] = v < PF_KEYS * d8;
         const int key = v_on[i] ? v / d8 : 0, ch = v_on[i] ? v % d8 : 0;
         k_local[i] = key;
@@ -122,7 +128,7 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
         // row order inside a 32-key half: tile a reads keys 8j + {0..3}, tile b keys 8j + {4..7}
         const int rho = (key & ~31) + (((k32 & 7) < 4) ? (4 * (k32 >> 3) + (k32 & 3)) : (16 + 4 * (k32 >> 3) + (k32 & 3)));
         k_lds[i] = rho * KLD + ch * 8;
-        const int kg = v % PF_KG, dd = v / PF_KG;
+        const int kg = v % (PF_KEYS / 8), dd = v / (PF_KEYS / 8);
         v_goff[i] = dd * P;
         v_lds[i] = dd * VLD + 8 * kg;
     }
@@ -131,13 +137,13 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     // memory round trip (the data), not one per vector.
 #define PF_PAGES(C0)                                                                                          \
     _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                          \
-        const int key = (C0) + k_local[i], key0 = (C0) + 8 * ((tid + 256 * i) % PF_KG);                       \
+        const int key = (C0) + k_local[i], key0 = (C0) + 8 * ((tid + NT * i) % (PF_KEYS / 8));                       \
         kpg[i] = (v_on[i] && key < kvl) ? bt[key >> log2p] : -1;                                              \
         vpg[i] = (v_on[i] && key0 < kvl) ? bt[key0 >> log2p] : -1;                                            \
     }
 #define PF_PREFETCH(C0)                                                                                       \
     _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                          \
-        const int key = (C0) + k_local[i], key0 = (C0) + 8 * ((tid + 256 * i) % PF_KG);                       \
+        const int key = (C0) + k_local[i], key0 = (C0) + 8 * ((tid + NT * i) % (PF_KEYS / 8));                       \
         pk[i] = pf_zero8();                                                                                   \
         pv[i] = pf_zero8();                                                                                   \
         if (kpg[i] >= 0 && kpg[i] < num_pages)                                                                \
@@ -147,7 +153,7 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
     }                                                                                                         \
     if ((C0) + PF_KEYS > kvl) {                        /* slots beyond the request's keys hold anything */     \
         _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                      \
-            const int valid = kvl - ((C0) + 8 * ((tid + 256 * i) % PF_KG));                                   \
+            const int valid = kvl - ((C0) + 8 * ((tid + NT * i) % (PF_KEYS / 8)));                                   \
             if (valid < 8) { _Pragma("unroll") for (int j = 0; j < 8; ++j) if (j >= valid) pv[i][j] = 0; }     \
         }                                                                                                     \
     }
@@ -180,18 +186,18 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
             const int h0 = c0 + 32 * half;
             if (h0 > w_hi || h0 + 31 < w_lo) continue;             // no row of this wave reads these keys (wave-uniform)
             // ---- S^T = K . Q^T for both row tiles ------------------------------------------------
-            f32x4_t sa[2], sb[2];
+            f32x4_t sa[RT], sb[RT];
 #pragma unroll
-            for (int t = 0; t < 2; ++t) { sa[t] = f32x4_t{0.f, 0.f, 0.f, 0.f}; sb[t] = f32x4_t{0.f, 0.f, 0.f, 0.f}; }
+            for (int t = 0; t < RT; ++t) { sa[t] = f32x4_t{0.f, 0.f, 0.f, 0.f}; sb[t] = f32x4_t{0.f, 0.f, 0.f, 0.f}; }
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk) {
-                if (kk * 32 < d) {
+                if (DFULL || kk * 32 < d) {
                     // columns at and beyond d were never staged: they must read as zero, not as what LDS held before
-                    const bool in_d = kk * 32 + 8 * g < d;
+                    const bool in_d = DFULL || kk * 32 + 8 * g < d;
                     const bf16x8_t ka = in_d ? *reinterpret_cast<const bf16x8_t*>(ks + (32 * half + r16) * KLD + kk * 32 + 8 * g) : pf_zero8();
                     const bf16x8_t kb = in_d ? *reinterpret_cast<const bf16x8_t*>(ks + (32 * half + 16 + r16) * KLD + kk * 32 + 8 * g) : pf_zero8();
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) {
+                    for (int t = 0; t < RT; ++t) {
                         sa[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, bq[t][kk], sa[t], 0, 0, 0);
                         sb[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, bq[t][kk], sb[t], 0, 0, 0);
                     }
@@ -201,10 +207,10 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
             // so that the exponentials are single v_exp_f32; the result does not change. ---------------------
             // Most key blocks lie wholly before every row of the wave and inside every window: no masks then.
             const bool unmasked = w_rows_full && h0 + 31 <= w_min_pos && h0 >= w_max_lo && h0 + 31 < kvl;
-            bf16x8_t pb[2];
-            float alpha[2];
+            bf16x8_t pb[RT];
+            float alpha[RT];
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
+            for (int t = 0; t < RT; ++t) {
                 float sc[8];                          // raw scores; the scale goes into the exponent's fma
 #pragma unroll
                 for (int j = 0; j < 8; ++j) sc[j] = j < 4 ? sa[t][j] : sb[t][j - 4];
@@ -242,7 +248,7 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
             }
             // ---- O^T = O^T * alpha + V^T . P^T (the rescale is skipped while no row's maximum moves) -------
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
+            for (int t = 0; t < RT; ++t) {
                 if (__any(alpha[t] != 1.f)) {
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) acc[t][dt] *= alpha[t];
@@ -250,10 +256,10 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
             }
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                if (dt * 16 < d) {
+                if (DFULL || dt * 16 < d) {
                     const bf16x8_t vt = *reinterpret_cast<const bf16x8_t*>(vs + (dt * 16 + r16) * VLD + 32 * half + 8 * g);
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pb[t], acc[t][dt], 0, 0, 0);
+                    for (int t = 0; t < RT; ++t) acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pb[t], acc[t][dt], 0, 0, 0);
                 }
             }
         }
@@ -261,13 +267,13 @@ __global__ __launch_bounds__(PF_WAVES * 64, 2) void attention_prefill_kernel(
 #undef PF_PREFETCH
 #undef PF_PAGES
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < RT; ++t) {
         float lt = l[t];
         lt += __shfl_xor(lt, 16, 64);
         lt += __shfl_xor(lt, 32, 64);
         if (splits > 1) {
             // this part's share of the 16-row unit: O unnormalised, m back in the natural-log domain, l
-            const int unit = tile * (PF_ROWS / 16) + wave * 2 + t;
+            const int unit = tile * (PF_ROWS / 16) + wave * RT + t;
             float* w = ws + (((size_t)unit * n_kv + hk) * splits + part) * (16 * (DMAX + 2));
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4_t*>(w + r16 * DMAX + dt * 16 + 4 * g) = acc[t][dt];
@@ -299,6 +305,9 @@ extern "C" int64_t spy_attention_prefill_workspace(int num_tiles, int n_kv, int 
     return (int64_t)num_tiles * (PF_ROWS / 16) * n_kv * splits * 16 * ((d <= 64 ? 64 : 128) + 2);
 }
 
+static long long g_thin_below = 384;     // blocks: up to a CU count and a half, a wave takes one row tile
+extern "C" int spy_attention_prefill_set_thin(long long blocks) { g_thin_below = blocks; return 0; }
+
 extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, const void* vc, int P, int num_pages, const int* cu_q,
                                      const int* pos0, const int* kv_len, const int* block_table, int max_blocks,
                                      const int* tile_entry, const int* tile_row0, int num_tiles, int S, int T, int n_q, int n_kv,
@@ -315,15 +324,23 @@ extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, c
     SPY_REQUIRE(splits == 1 || ws, "spy_attention_prefill: key parts without a workspace");
     const dim3 grid(splits > 1 ? num_tiles : (num_tiles + 1) / 2, n_kv, splits);
     const dim3 mgrid(num_tiles * (PF_ROWS / 16), n_kv);
-#define PF_CASE(DM)                                                                                                              \
-    attention_prefill_kernel<DM><<<grid, PF_WAVES * 64, 0, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, \
+    bool thin = (long long)grid.x * grid.y * grid.z <= g_thin_below;     // (only for head sizes 64 and 128: the others need too many registers)
+#define PF_LAUNCH(DM, FULL)                                                                                                      \
+    if (thin) attention_prefill_kernel<DM, FULL, 1><<<grid, PF_ROWS * 4, 0, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, \
                                                                  P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,      \
                                                                  tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p,      \
                                                                  num_tiles, splits, ws);                                         \
+    else attention_prefill_kernel<DM, FULL, 2><<<grid, PF_ROWS * 2, 0, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, \
+                                                                 P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,      \
+                                                                 tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p,      \
+                                                                 num_tiles, splits, ws)
+#define PF_CASE(DM)                                                                                                              \
+    if (d == DM) { PF_LAUNCH(DM, true); } else { thin = false; PF_LAUNCH(DM, false); }                                           \
     if (splits > 1)                                                                                                              \
         attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits,    \
                                                           PF_ROWS / 16);
     if (d <= 64) { PF_CASE(64) } else { PF_CASE(128) }
+#undef PF_LAUNCH
 #undef PF_CASE
     SPY_CHECK_LAUNCH("spy_attention_prefill");
     return 0;
