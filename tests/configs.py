@@ -25,5 +25,11 @@ TINY_D = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_act
               vocab_size=400, rope_theta=20000.0, rms_norm_eps=2e-6, tie_word_embeddings=True,
               max_position_embeddings=320, bos_token_id=0, eos_token_id=3)
 
+#: the head size and group shape of the large models (128-wide heads, several query heads per kv head), small otherwise
+TINY_E = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_act="silu", num_hidden_layers=2,
+              hidden_size=256, num_attention_heads=8, num_key_value_heads=2, head_dim=128, intermediate_size=640,
+              vocab_size=592, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+              max_position_embeddings=448, bos_token_id=0, eos_token_id=4)
+
 #: init that makes attention and logits informative: matrices N(0, std), norms 1 + N(0, 0.1)
 INIT = dict(matrix_std=0.08, norm_std=0.1)

@@ -11,14 +11,14 @@ import pytest
 import torch
 
 from tests import replay_cases as rc
-from tests.configs import INIT, TINY_A, TINY_B, TINY_C, TINY_D
+from tests.configs import INIT, TINY_A, TINY_B, TINY_C, TINY_D, TINY_E
 from tests.gpu_util import require_gpu
 from tests.plain.qwen3_plain import PlainQwen3
 
 pytestmark = pytest.mark.gpu
 
 CASES = {"A": (TINY_A, [5, 17, 33, 60], 16), "B": (TINY_B, [1, 40, 130], 8), "C": (TINY_C, [3, 70, 200, 45, 64, 97, 333], 16),
-         "D": (TINY_D, [9, 50, 190, 77, 300], 16)}
+         "D": (TINY_D, [9, 50, 190, 77, 300], 16), "E": (TINY_E, [2, 130, 425, 61], 16)}
 # float32: only the order of sums differs.  bfloat16: activations are rounded to 8 bits between
 # kernels; with these weights the CPU model of that rounding differs from float32 by up to 0.04
 # on logits of standard deviation 0.7 ("tolerances").
@@ -38,7 +38,7 @@ def models(tmp_path_factory):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
 def test_replay_matches_plain(dtype, name, mode, models, tmp_path, monkeypatch):
     require_gpu()
@@ -52,8 +52,8 @@ def test_replay_matches_plain(dtype, name, mode, models, tmp_path, monkeypatch):
     rc.run_replay_inprocess(folder, dtype, str(tmp_path), steps, rc.max_live_tokens(steps), ["--kvcache-block-size", str(page)])
     got = rc.collect(str(tmp_path), steps, cfg["vocab_size"])
     rc.compare(got, ref, what="%s/%s/%s" % (name, mode, dtype), **TOL[dtype])
-    # configuration D in bfloat16 is there for the decode products with folded norms: they must have run
-    assert bool(folded) == (name == "D" and dtype == "bfloat16")
+    # configurations D and E in bfloat16 are there for the decode products with folded norms: they must have run
+    assert bool(folded) == (name in "DE" and dtype == "bfloat16")
 
 
 @pytest.fixture(scope="module")
