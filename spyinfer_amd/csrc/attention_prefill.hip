@@ -115,45 +115,56 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, RT == 1 ? 1 : 2) void attention_p
     //                                     V: kgrp = v % 8, dd = v / 8     (8 keys of one head dim)
     // What does not change from round to round is worked out once: the local key, the offsets inside a
     // page and the places in LDS.  Pages are powers of two here, so a key's page is a shift away.
-    int k_local[NV], k_goff[NV], v_goff[NV], k_lds[NV], v_lds[NV];
+    // An address is  cache + page * (bytes of a page) + (what depends on the thread only) + (what depends on the round
+    // only):  one 64-bit multiply-add per vector and round.  Inside a page, key c0 + k lies at ((c0 & (P - 1) & ~63) +
+    // (k & (P - 1))): c0 is a multiple of 64 and pages are powers of two, so the two terms never carry into each other.
+    int k_local[NV], v_local[NV], k_toff[NV], v_toff[NV], k_lds[NV], v_lds[NV];
     bool v_on[NV];
+    const int pmask = P - 1;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int v = tid + NT * i;
         v_on[i] = v < PF_KEYS * d8;
         const int key = v_on[i] ? v / d8 : 0, ch = v_on[i] ? v % d8 : 0;
         k_local[i] = key;
-        k_goff[i] = ch * 8;
+        k_toff[i] = (key & pmask) * d + ch * 8;
         const int k32 = key & 31;
         // row order inside a 32-key half: tile a reads keys 8j + {0..3}, tile b keys 8j + {4..7}
         const int rho = (key & ~31) + (((k32 & 7) < 4) ? (4 * (k32 >> 3) + (k32 & 3)) : (16 + 4 * (k32 >> 3) + (k32 & 3)));
         k_lds[i] = rho * KLD + ch * 8;
         const int kg = v % (PF_KEYS / 8), dd = v / (PF_KEYS / 8);
-        v_goff[i] = dd * P;
+        v_local[i] = 8 * kg;
+        v_toff[i] = dd * P + ((8 * kg) & pmask);
         v_lds[i] = dd * VLD + 8 * kg;
     }
-    const int pmask = P - 1;
+    const size_t page_elems = (size_t)n_kv * P * d;                 // elements of one page of K (and of V)
+    const bf16_t* kc_h = kc + (size_t)hk * P * d;
+    const bf16_t* vc_h = vc + (size_t)hk * d * P;
     // The page lookups of a round are issued together and a round early, so that a round costs one
     // memory round trip (the data), not one per vector.
 #define PF_PAGES(C0)                                                                                          \
     _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                          \
-        const int key = (C0) + k_local[i], key0 = (C0) + 8 * ((tid + NT * i) % (PF_KEYS / 8));                       \
+        const int key = (C0) + k_local[i], key0 = (C0) + v_local[i];                                          \
         kpg[i] = (v_on[i] && key < kvl) ? bt[key >> log2p] : -1;                                              \
         vpg[i] = (v_on[i] && key0 < kvl) ? bt[key0 >> log2p] : -1;                                            \
     }
 #define PF_PREFETCH(C0)                                                                                       \
-    _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                          \
-        const int key = (C0) + k_local[i], key0 = (C0) + 8 * ((tid + NT * i) % (PF_KEYS / 8));                       \
-        pk[i] = pf_zero8();                                                                                   \
-        pv[i] = pf_zero8();                                                                                   \
-        if (kpg[i] >= 0 && kpg[i] < num_pages)                                                                \
-            pk[i] = *reinterpret_cast<const bf16x8_t*>(kc + (((size_t)kpg[i] * n_kv + hk) * P + (key & pmask)) * d + k_goff[i]); \
-        if (vpg[i] >= 0 && vpg[i] < num_pages)                                                                \
-            pv[i] = *reinterpret_cast<const bf16x8_t*>(vc + ((size_t)vpg[i] * n_kv + hk) * d * P + v_goff[i] + (key0 & pmask)); \
+    {                                                                                                         \
+        const int in_page = (C0) & pmask & ~(PF_KEYS - 1);       /* of the round's first key; 0 for pages up to 64 */ \
+        const bf16_t* kr = kc_h + (size_t)in_page * d;                                                        \
+        const bf16_t* vr = vc_h + in_page;                                                                    \
+        _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                      \
+            pk[i] = pf_zero8();                                                                               \
+            pv[i] = pf_zero8();                                                                               \
+            if ((unsigned)kpg[i] < (unsigned)num_pages)                                                       \
+                pk[i] = *reinterpret_cast<const bf16x8_t*>(kr + (size_t)(unsigned)kpg[i] * page_elems + k_toff[i]); \
+            if ((unsigned)vpg[i] < (unsigned)num_pages)                                                       \
+                pv[i] = *reinterpret_cast<const bf16x8_t*>(vr + (size_t)(unsigned)vpg[i] * page_elems + v_toff[i]); \
+        }                                                                                                     \
     }                                                                                                         \
     if ((C0) + PF_KEYS > kvl) {                        /* slots beyond the request's keys hold anything */     \
         _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                                      \
-            const int valid = kvl - ((C0) + 8 * ((tid + NT * i) % (PF_KEYS / 8)));                                   \
+            const int valid = kvl - ((C0) + v_local[i]);                                                      \
             if (valid < 8) { _Pragma("unroll") for (int j = 0; j < 8; ++j) if (j >= valid) pv[i][j] = 0; }     \
         }                                                                                                     \
     }
