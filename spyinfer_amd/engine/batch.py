@@ -122,6 +122,25 @@ class StepBatch:
             self._arrays["slot_mapping_%d" % g.index] = (pages * P + positions % P).astype(np.int32)
         self.num_groups = len(manager.page_groups)
         self.page_size = manager.page_size
+        self.token_ids_late = False      # True: the token ids came after the arrays were packed for the transfer
+        self._graph_key = None
+
+    def set_token_ids(self, entries: Sequence["StepEntry"], vocab_size: Optional[int]) -> None:
+        """The tokens of a batch that was built ahead with placeholders (same requests, same numbers of tokens)."""
+        if self._dev:
+            raise RuntimeError("the batch is already on the device")
+        if len(entries) != self.S:
+            raise ValueError("the batch was built for %d entries, not %d" % (self.S, len(entries)))
+        for e, n, b in zip(entries, self.lens, self.entries):
+            if e.cache is not b.cache or len(e.tokens) != int(n):
+                raise ValueError("the batch was built for other requests or other numbers of tokens")
+        ids = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=self.T)
+        if vocab_size is not None and self.T and (ids.min() < 0 or ids.max() >= vocab_size):
+            bad = ids[(ids < 0) | (ids >= vocab_size)][0]
+            raise ValueError("token id %d is outside the vocabulary of %d" % (int(bad), vocab_size))
+        self._arrays["token_ids"] = ids.astype(np.int32)
+        self.entries = list(entries)
+        self.token_ids_late = True
 
     # ---- additions by parts, before upload ---------------------------------
     def add_array(self, name: str, values) -> None:
@@ -166,6 +185,15 @@ class StepBatch:
 
     def layout_key(self):
         return tuple((name, int(v.shape[0])) for name, v in self._arrays.items())
+
+    def graph_key(self):
+        """What a captured graph of this step depends on beside the arrays' contents."""
+        if self._graph_key is None:
+            self._graph_key = (self.layout_key(), self.all_rows_wanted)
+        return self._graph_key
+
+    def host_array(self, name: str) -> np.ndarray:
+        return self._arrays[name]
 
     def pack_into(self, host: torch.Tensor):
         """Write all arrays into the int32 host tensor; returns (layout, total ints)."""

@@ -59,6 +59,7 @@ class LLMEngine:
         self._sequences: Dict[int, Sequence] = {}
         self._next_id = 0
         self.stats = dict(steps=0, prefill_tokens=0, decode_tokens=0)
+        self._ahead = None
 
     def _pages_from_free_memory(self) -> int:
         per_page = ModelRunner.bytes_per_page(self.model, self.config.kvcache_block_size, self.config.dtype)
@@ -126,7 +127,9 @@ class LLMEngine:
 
     # ---- one step --------------------------------------------------------
     def step(self) -> List[StepOutput]:
-        scheduled = self.scheduler.schedule()
+        scheduled, prepared = self._take_ahead()
+        if scheduled is None:
+            scheduled = self.scheduler.schedule()
         if not scheduled:
             return []
         entries = []
@@ -134,12 +137,15 @@ class LLMEngine:
             seq = sc.seq
             lo = seq.num_computed
             entries.append(StepEntry(seq.cache, seq.tokens[lo:lo + sc.num_tokens], [sc.num_tokens - 1] if sc.samples else []))
-        logits = self.runner.step(entries)
+        logits = self.runner.step(entries, prepared)
         sampling = [sc.seq for sc in scheduled if sc.samples]
-        tokens = self.sampler.sample(
+        picked = self.sampler.sample_device(
             logits, [s.params.temperature for s in sampling],
             [s.params.seed if s.params.seed is not None else self.config.seed + s.id for s in sampling],
             [s.num_generated for s in sampling])
+        # the device is busy with the step now: the host prepares the next one meanwhile, if it can tell what it will be
+        self._ahead = self._prepare_ahead(scheduled)
+        tokens = [] if picked is None else [int(x) for x in picked.tolist()]
         outputs = []
         for seq, tok in zip(sampling, tokens):
             seq.tokens.append(tok)
@@ -158,6 +164,47 @@ class LLMEngine:
         for sc in scheduled:
             self.stats["decode_tokens" if sc.num_tokens == 1 and sc.samples else "prefill_tokens"] += sc.num_tokens
         return outputs
+
+    # While the device runs a step in which every running request decodes one token, the next step is known but for
+    # its token ids, unless a request ends or another arrives: the same requests, one position on.  Its batch is
+    # built then (pages reserved, arrays, plans), off the critical path between two steps.  When the next ``step``
+    # finds anything changed, what was prepared is dropped; the pages it reserved are pages the requests need anyway.
+    def _prepare_ahead(self, scheduled):
+        sch = self.scheduler
+        if sch.waiting or len(scheduled) != len(sch.running):
+            return None
+        for sc in scheduled:
+            seq = sc.seq
+            if sc.num_tokens != 1 or not sc.samples:
+                return None
+            # after this step's token the request goes on only if neither limit is reached (the end-of-sequence token
+            # cannot be foreseen: it makes the prepared step invalid)
+            if seq.params.max_new_tokens is not None and seq.num_generated + 1 >= seq.params.max_new_tokens:
+                return None
+            if len(seq) + 1 >= self.config.max_model_len:
+                return None
+        manager = self.runner.manager
+        for sc in scheduled:
+            if not manager.can_reserve(sc.seq.cache, 1):
+                return None
+            manager.reserve(sc.seq.cache, 1)
+        entries = [StepEntry(sc.seq.cache, [0], [0]) for sc in scheduled]
+        nxt = [type(sc)(sc.seq, 1, True) for sc in scheduled]
+        return nxt, self.runner.prepare(entries), [(sc.seq, sc.seq.cache) for sc in scheduled]
+
+    def _take_ahead(self):
+        ahead, self._ahead = self._ahead, None
+        if ahead is None:
+            return None, None
+        scheduled, prepared, state = ahead
+        sch = self.scheduler
+        if sch.waiting or len(sch.running) != len(state):
+            return None, None
+        for (seq, cache), running in zip(state, sorted(sch.running, key=lambda s: s.admit_order)):
+            if seq is not running or seq.status is not SequenceStatus.RUNNING or seq.cache is not cache or not cache.live \
+                    or len(seq) - seq.num_computed != 1:
+                return None, None
+        return scheduled, prepared
 
     def generate(self, prompts: Seq[Seq[int]], params: Optional[SamplingParams] = None) -> List[List[int]]:
         """Convenience loop: all prompts at once, generated tokens of each."""

@@ -42,6 +42,14 @@ def load_model(folder: str, dtype, device) -> DecoderModel:
     return model
 
 
+class PreparedStep:
+    """A step's batch built ahead of its token ids, and the state of the requests' caches it was built for."""
+    __slots__ = ("batch", "graphable", "state")
+
+    def __init__(self, batch: StepBatch, graphable: bool, state):
+        self.batch, self.graphable, self.state = batch, graphable, state
+
+
 class ModelRunner:
     def __init__(self, model: DecoderModel, dtype, device, page_size: int, num_pages: int, max_num_seqs: int,
                  max_num_batched_tokens: int = 16384, enforce_eager: bool = True, max_model_len: Optional[int] = None):
@@ -62,6 +70,7 @@ class ModelRunner:
         self._seen = {}
         self._pinned = None
         self._copied = None
+        self._packed = None        # the batch whose arrays the pinned buffer holds
         self.graph_replays = 0
 
     @staticmethod
@@ -70,14 +79,11 @@ class ModelRunner:
         act = 2 if resolve_dtype(dtype) == torch.bfloat16 else 4
         return sum(2 * s.num_kv_heads * s.head_dim * page_size * act for s in model.cache_specs() if isinstance(s, PagedKV))
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """Run the entries' tokens as one batch.  Pages for them must have been reserved
-        (``manager.reserve``).  Returns float32 logits [wanted rows, vocab] in the order of the
-        entries and of their ``want`` (valid until the next step); afterwards the tokens count
-        as cached."""
+    def prepare(self, entries: Sequence[StepEntry]) -> "PreparedStep":
+        """The host work of a step that does not need the device: the batch's arrays, the checks, the parts' plans.
+        The entries' requests must be in the state in which the step will find them (earlier steps committed, pages
+        reserved); their token ids may still be placeholders (``step`` puts the real ones in)."""
         entries = list(entries)
-        if not entries:
-            return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         graphable = self.use_graphs and all(len(e.tokens) == 1 for e in entries) \
             and all(len(t) <= self.fixed_max_blocks for e in entries for t in e.cache.tables)
         batch = StepBatch(entries, self.manager, self.act_dtype, self.device, self.model.vocab_size,
@@ -88,6 +94,28 @@ class ModelRunner:
             raise ValueError("a request would reach %d tokens, the model's positions end at %d"
                              % (batch.max_kv_len, self.model.max_positions))
         self.model.plan(batch)
+        if self.device.type == "cuda":
+            self._pack(batch)
+        if graphable:
+            batch.graph_key()
+        return PreparedStep(batch, graphable, [(e.cache, e.cache.num_tokens, tuple(e.cache.versions)) for e in entries])
+
+    def step(self, entries: Sequence[StepEntry], prepared: Optional["PreparedStep"] = None) -> torch.Tensor:
+        """Run the entries' tokens as one batch.  Pages for them must have been reserved
+        (``manager.reserve``).  Returns float32 logits [wanted rows, vocab] in the order of the
+        entries and of their ``want`` (valid until the next step); afterwards the tokens count
+        as cached.  ``prepared``: what ``prepare`` made of the same entries ahead of time."""
+        entries = list(entries)
+        if not entries:
+            return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
+        if prepared is not None:
+            if any(c is not e.cache or c.num_tokens != n or tuple(c.versions) != v
+                   for e, (c, n, v) in zip(entries, prepared.state)) or len(entries) != len(prepared.state):
+                raise ValueError("the prepared step does not fit the requests' caches any more")
+            prepared.batch.set_token_ids(entries, self.model.vocab_size)
+        else:
+            prepared = self.prepare(entries)
+        batch, graphable = prepared.batch, prepared.graphable
         self._reset_fresh_state(batch)
         if graphable:
             logits = self._step_graph(batch)
@@ -103,29 +131,45 @@ class ModelRunner:
         return logits
 
     # ---- metadata to the device ----------------------------------------------
-    def _upload(self, batch: StepBatch, dev_buf: Optional[torch.Tensor]) -> None:
-        """Pack the batch's arrays into pinned host memory and copy them with one transfer."""
-        _layout, total = batch.layout()
+    def _pack(self, batch: StepBatch) -> None:
+        """The batch's arrays into the pinned host buffer (one buffer: the batch packed last owns it)."""
+        layout, total = batch.layout()
         if self._pinned is None or self._pinned.numel() < total:
             self._pinned = torch.empty(max(total, 1 << 16), dtype=torch.int32, pin_memory=True)
             self._copied = None
         if self._copied is not None:
             self._copied.synchronize()          # the last transfer has read the pinned buffer
-        layout, total = batch.pack_into(self._pinned)
+            self._copied = None
+        batch.pack_into(self._pinned)
+        batch.packed_layout, batch.packed_total = layout, total
+        self._packed = batch
+
+    def _upload(self, batch: StepBatch, dev_buf: Optional[torch.Tensor], bind: bool = True) -> None:
+        """Copy the packed arrays to the device with one transfer.  A batch that was packed ahead of its token ids
+        gets them patched in.  ``bind=False``: the device views are not needed (a graph that has them is replayed)."""
+        if self._packed is not batch:
+            self._pack(batch)
+        elif batch.token_ids_late:
+            off, n = batch.packed_layout["token_ids"]
+            self._pinned.numpy()[off:off + n] = batch.host_array("token_ids")
+        batch.token_ids_late = False
+        layout, total = batch.packed_layout, batch.packed_total
         if dev_buf is None:
             dev_buf = torch.empty(total, dtype=torch.int32, device=self.device)
         dev_buf[:total].copy_(self._pinned[:total], non_blocking=True)
         self._copied = torch.cuda.Event()
         self._copied.record()
-        batch.bind_device(dev_buf, layout)
+        self._packed = None                      # the buffer is in flight until the event
+        if bind:
+            batch.bind_device(dev_buf, layout)
 
     # ---- graphs -----------------------------------------------------------------
     def _step_graph(self, batch: StepBatch) -> torch.Tensor:
-        key = (batch.layout_key(), batch.all_rows_wanted)
+        key = batch.graph_key()
         held = self._graphs.get(key)
         if held is not None:
             graph, dev_buf, logits = held
-            self._upload(batch, dev_buf)
+            self._upload(batch, dev_buf, bind=False)
             graph.replay()
             self.graph_replays += 1
             return logits

@@ -50,14 +50,21 @@ class Sampler:
     def __init__(self, device):
         self.device = torch.device(device)
 
-    def sample(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
-               indices: Sequence[int]) -> List[int]:
-        """One token per row of ``logits [R, vocab]``; row r is draw ``indices[r]`` of seed ``seeds[r]``."""
+    def sample_device(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
+                      indices: Sequence[int]) -> Optional[torch.Tensor]:
+        """One token per row of ``logits [R, vocab]``, still on the device (int32 [R]); row r is draw ``indices[r]`` of
+        seed ``seeds[r]``.  Nothing waits for the device here."""
         R = logits.shape[0]
         if R == 0:
-            return []
-        temp = torch.tensor(list(temperatures), dtype=torch.float32)
-        u = torch.tensor([uniform_for(s, i) if t > 0 else 0.0 for s, i, t in zip(seeds, indices, temperatures)],
-                         dtype=torch.float32)
-        out = ops.sample(logits, temp.to(self.device), u.to(self.device))
-        return [int(x) for x in out.tolist()]
+            return None
+        host = torch.empty((2, R), dtype=torch.float32, pin_memory=self.device.type == "cuda")
+        flat = host.numpy()
+        flat[0] = temperatures
+        flat[1] = [uniform_for(s, i) if t > 0 else 0.0 for s, i, t in zip(seeds, indices, temperatures)]
+        dev = host.to(self.device, non_blocking=True)
+        return ops.sample(logits, dev[0], dev[1])
+
+    def sample(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
+               indices: Sequence[int]) -> List[int]:
+        out = self.sample_device(logits, temperatures, seeds, indices)
+        return [] if out is None else [int(x) for x in out.tolist()]

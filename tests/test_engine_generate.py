@@ -105,3 +105,55 @@ def test_cli_usage(capsys):
     assert main([]) == 1
     assert main(["-m", "x", "-b", "cuda"]) == 1
     assert "Available backends: hip" in capsys.readouterr().err
+
+
+def test_steps_prepared_ahead_change_nothing(folder_a, emu_ops):
+    """While a step of decoded tokens runs, the engine builds the next step's batch; it is dropped when a request ends
+    (by count or by its end token), arrives, or is removed in between.  The tokens that come out are those of an engine
+    that never prepares ahead, event by event; no page is lost."""
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    ps = prompts(256, [9, 30, 4, 21, 12], seed=7)
+    plain = PlainQwen3(folder_a)
+    # an end token that the second request really produces, so that it ends early
+    g1 = plain.greedy(ps[1], 12)
+    k = max(i for i in range(12) if g1[i] not in g1[:i])       # the last place where a token appears for the first time
+    assert k >= 1
+    eos = g1[k]
+
+    def run(ahead):
+        eng = LLMEngine(folder_a, dtype="float32", device="cpu", max_model_len=128, num_kvcache_blocks=40, max_num_seqs=8)
+        eng.eos_token_id = eos
+        used = [0]
+        if not ahead:
+            eng._prepare_ahead = lambda scheduled: None
+        else:
+            real = eng._take_ahead
+            def counted():
+                got = real()
+                used[0] += got[0] is not None
+                return got
+            eng._take_ahead = counted
+        ids = [eng.add_request(ps[0], SamplingParams(max_new_tokens=25, ignore_eos=True)),
+               eng.add_request(ps[1], SamplingParams(max_new_tokens=25)),                   # ends at its end token
+               eng.add_request(ps[2], SamplingParams(max_new_tokens=7, ignore_eos=True))]   # ends by count
+        log = []
+        for step in range(60):
+            if step == 10:
+                ids.append(eng.add_request(ps[3], SamplingParams(max_new_tokens=9, ignore_eos=True)))   # arrives in between
+            if step == 16:
+                eng.remove_request(ids[0])                                                   # leaves in between
+                ids[0] = None
+            if step == 20:
+                ids.append(eng.add_request(ps[4], SamplingParams(temperature=0.7, max_new_tokens=8, ignore_eos=True, seed=5)))
+            log.append(sorted(tuple(o) for o in eng.step()))
+        assert not eng.has_unfinished_requests()
+        eng.runner.manager.check()
+        assert eng.runner.manager.num_free_pages() == [40]
+        return log, [eng.get_generated_tokens(i) for i in ids if i is not None], used[0]
+
+    log_a, out_a, used = run(True)
+    log_b, out_b, _ = run(False)
+    assert log_a == log_b and out_a == out_b
+    assert used >= 15, "steps of decoded tokens alone must have come from the batch prepared ahead (%d did)" % used
+    assert out_a[0] == g1[:k + 1]                              # the second request ended at its end token
+    assert out_a[1] == plain.greedy(ps[2], 7) and out_a[2] == plain.greedy(ps[3], 9)
