@@ -122,25 +122,7 @@ class StepBatch:
             self._arrays["slot_mapping_%d" % g.index] = (pages * P + positions % P).astype(np.int32)
         self.num_groups = len(manager.page_groups)
         self.page_size = manager.page_size
-        self.token_ids_late = False      # True: the token ids came after the arrays were packed for the transfer
         self._graph_key = None
-
-    def set_token_ids(self, entries: Sequence["StepEntry"], vocab_size: Optional[int]) -> None:
-        """The tokens of a batch that was built ahead with placeholders (same requests, same numbers of tokens)."""
-        if self._dev:
-            raise RuntimeError("the batch is already on the device")
-        if len(entries) != self.S:
-            raise ValueError("the batch was built for %d entries, not %d" % (self.S, len(entries)))
-        for e, n, b in zip(entries, self.lens, self.entries):
-            if e.cache is not b.cache or len(e.tokens) != int(n):
-                raise ValueError("the batch was built for other requests or other numbers of tokens")
-        ids = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=self.T)
-        if vocab_size is not None and self.T and (ids.min() < 0 or ids.max() >= vocab_size):
-            bad = ids[(ids < 0) | (ids >= vocab_size)][0]
-            raise ValueError("token id %d is outside the vocabulary of %d" % (int(bad), vocab_size))
-        self._arrays["token_ids"] = ids.astype(np.int32)
-        self.entries = list(entries)
-        self.token_ids_late = True
 
     # ---- additions by parts, before upload ---------------------------------
     def add_array(self, name: str, values) -> None:

@@ -25,6 +25,21 @@ class StepOutput(NamedTuple):
     finished: bool
 
 
+class _Flight(NamedTuple):
+    scheduled: list            # what the step runs (Scheduled)
+    rows: list                 # (request, its cache at launch) of every sampled row, in the order of ``picked``
+    picked: Optional[torch.Tensor]   # sampled token ids, on the device
+    host: Optional[torch.Tensor]     # the same, on their way to the host (the copy is queued right behind the sampling,
+    copied: object                   # ahead of any later step; this event tells when it is done)
+
+    def tokens(self) -> List[int]:
+        if self.picked is None:
+            return []
+        if self.copied is not None:
+            self.copied.synchronize()
+        return [int(x) for x in self.host.tolist()]
+
+
 class LLMEngine:
     def __init__(self, model_path: str, device="cuda:0", **params):
         known = {f for f in EngineConfig.__dataclass_fields__}
@@ -59,7 +74,9 @@ class LLMEngine:
         self._sequences: Dict[int, Sequence] = {}
         self._next_id = 0
         self.stats = dict(steps=0, prefill_tokens=0, decode_tokens=0)
-        self._ahead = None
+        self._flight = None        # a step that runs on the device and whose tokens have not been read yet
+        #: False: every step waits for its tokens before the next one is built (as the reference does)
+        self.run_ahead = True
 
     def _pages_from_free_memory(self) -> int:
         per_page = ModelRunner.bytes_per_page(self.model, self.config.kvcache_block_size, self.config.dtype)
@@ -127,27 +144,28 @@ class LLMEngine:
 
     # ---- one step --------------------------------------------------------
     def step(self) -> List[StepOutput]:
-        scheduled, prepared = self._take_ahead()
-        if scheduled is None:
-            scheduled = self.scheduler.schedule()
-        if not scheduled:
-            return []
-        entries = []
-        for sc in scheduled:
-            seq = sc.seq
-            lo = seq.num_computed
-            entries.append(StepEntry(seq.cache, seq.tokens[lo:lo + sc.num_tokens], [sc.num_tokens - 1] if sc.samples else []))
-        logits = self.runner.step(entries, prepared)
-        sampling = [sc.seq for sc in scheduled if sc.samples]
-        picked = self.sampler.sample_device(
-            logits, [s.params.temperature for s in sampling],
-            [s.params.seed if s.params.seed is not None else self.config.seed + s.id for s in sampling],
-            [s.num_generated for s in sampling])
-        # the device is busy with the step now: the host prepares the next one meanwhile, if it can tell what it will be
-        self._ahead = self._prepare_ahead(scheduled)
-        tokens = [] if picked is None else [int(x) for x in picked.tolist()]
+        """One step of the engine: the tokens it sampled, request by request.
+
+        Steps in which every running request decodes one token are run ahead: before this step's tokens are read
+        from the device, the next step is already launched for the same requests, its token ids handed over on the
+        device (the sampler's output is copied into the next step's input).  So the device does not wait for the
+        host between two such steps.  What cannot be foreseen is a request that ends at its end-of-sequence token
+        (or is removed): its row in the step in flight is then ignored, and its pages, given back at once, are safe
+        because whatever reuses them runs later on the same stream.  A request that ends by count is known ahead,
+        and so is a request that waits for admission: no step is run ahead then."""
+        flight, self._flight = self._flight, None
+        if flight is not None and not any(self._alive(seq, cache) for seq, cache in flight.rows):
+            flight = None                                  # every request of the step in flight has ended meanwhile
+        if flight is None:
+            flight = self._launch(self.scheduler.schedule())
+            if flight is None:
+                return []
+        ahead = self._launch_ahead(flight) if self.run_ahead else None
+        tokens = flight.tokens()
         outputs = []
-        for seq, tok in zip(sampling, tokens):
+        for (seq, cache), tok in zip(flight.rows, tokens):
+            if not self._alive(seq, cache):
+                continue                                   # ended or removed while the step was in flight
             seq.tokens.append(tok)
             reason = None
             # the end-of-sequence token stays in the request's tokens (src/engine/model_runner.cpp:141-151)
@@ -160,25 +178,55 @@ class LLMEngine:
             if reason:
                 self.scheduler.finish(seq, reason)
             outputs.append(StepOutput(seq.id, tok, reason is not None))
+        self._flight = ahead
+        return outputs
+
+    @staticmethod
+    def _alive(seq: Sequence, cache) -> bool:
+        return seq.status is SequenceStatus.RUNNING and seq.cache is cache and cache.live
+
+    def _launch(self, scheduled, token_source=None, ahead: int = 0) -> Optional["_Flight"]:
+        """Run a scheduled step on the device and start its sampling; nothing waits for the device.  ``ahead`` = 1:
+        the requests' newest tokens are not on the host yet (they come from ``token_source`` on the device)."""
+        if not scheduled:
+            return None
+        entries = []
+        for sc in scheduled:
+            seq = sc.seq
+            lo = seq.num_computed
+            toks = [0] * sc.num_tokens if ahead else seq.tokens[lo:lo + sc.num_tokens]
+            entries.append(StepEntry(seq.cache, toks, [sc.num_tokens - 1] if sc.samples else []))
+        logits = self.runner.step(entries, token_source)
+        sampling = [sc.seq for sc in scheduled if sc.samples]
+        picked = self.sampler.sample_device(
+            logits, [s.params.temperature for s in sampling],
+            [s.params.seed if s.params.seed is not None else self.config.seed + s.id for s in sampling],
+            [s.num_generated + ahead for s in sampling])
         self.stats["steps"] += 1
         for sc in scheduled:
             self.stats["decode_tokens" if sc.num_tokens == 1 and sc.samples else "prefill_tokens"] += sc.num_tokens
-        return outputs
+        host = copied = None
+        if picked is not None:
+            if picked.is_cuda:
+                host = torch.empty(picked.shape, dtype=picked.dtype, pin_memory=True)
+                host.copy_(picked, non_blocking=True)
+                copied = torch.cuda.Event()
+                copied.record()
+            else:
+                host = picked
+        return _Flight(scheduled, [(s, s.cache) for s in sampling], picked, host, copied)
 
-    # While the device runs a step in which every running request decodes one token, the next step is known but for
-    # its token ids, unless a request ends or another arrives: the same requests, one position on.  Its batch is
-    # built then (pages reserved, arrays, plans), off the critical path between two steps.  When the next ``step``
-    # finds anything changed, what was prepared is dropped; the pages it reserved are pages the requests need anyway.
-    def _prepare_ahead(self, scheduled):
+    def _launch_ahead(self, flight: "_Flight") -> Optional["_Flight"]:
+        """The step after ``flight``, if it can be told without ``flight``'s tokens: the same requests, one token on."""
         sch = self.scheduler
-        if sch.waiting or len(scheduled) != len(sch.running):
+        scheduled = flight.scheduled
+        if sch.waiting or len(scheduled) != len(sch.running) or flight.picked is None:
             return None
         for sc in scheduled:
             seq = sc.seq
-            if sc.num_tokens != 1 or not sc.samples:
+            if sc.num_tokens != 1 or not sc.samples or not self._alive(seq, seq.cache):
                 return None
-            # after this step's token the request goes on only if neither limit is reached (the end-of-sequence token
-            # cannot be foreseen: it makes the prepared step invalid)
+            # with the token of the step in flight the request goes on only if neither limit is reached
             if seq.params.max_new_tokens is not None and seq.num_generated + 1 >= seq.params.max_new_tokens:
                 return None
             if len(seq) + 1 >= self.config.max_model_len:
@@ -188,23 +236,7 @@ class LLMEngine:
             if not manager.can_reserve(sc.seq.cache, 1):
                 return None
             manager.reserve(sc.seq.cache, 1)
-        entries = [StepEntry(sc.seq.cache, [0], [0]) for sc in scheduled]
-        nxt = [type(sc)(sc.seq, 1, True) for sc in scheduled]
-        return nxt, self.runner.prepare(entries), [(sc.seq, sc.seq.cache) for sc in scheduled]
-
-    def _take_ahead(self):
-        ahead, self._ahead = self._ahead, None
-        if ahead is None:
-            return None, None
-        scheduled, prepared, state = ahead
-        sch = self.scheduler
-        if sch.waiting or len(sch.running) != len(state):
-            return None, None
-        for (seq, cache), running in zip(state, sorted(sch.running, key=lambda s: s.admit_order)):
-            if seq is not running or seq.status is not SequenceStatus.RUNNING or seq.cache is not cache or not cache.live \
-                    or len(seq) - seq.num_computed != 1:
-                return None, None
-        return scheduled, prepared
+        return self._launch([type(sc)(sc.seq, 1, True) for sc in scheduled], flight.picked, ahead=1)
 
     def generate(self, prompts: Seq[Seq[int]], params: Optional[SamplingParams] = None) -> List[List[int]]:
         """Convenience loop: all prompts at once, generated tokens of each."""

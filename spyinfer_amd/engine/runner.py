@@ -43,11 +43,11 @@ def load_model(folder: str, dtype, device) -> DecoderModel:
 
 
 class PreparedStep:
-    """A step's batch built ahead of its token ids, and the state of the requests' caches it was built for."""
-    __slots__ = ("batch", "graphable", "state")
+    """The host half of a step: its batch, planned and packed for the transfer."""
+    __slots__ = ("batch", "graphable")
 
-    def __init__(self, batch: StepBatch, graphable: bool, state):
-        self.batch, self.graphable, self.state = batch, graphable, state
+    def __init__(self, batch: StepBatch, graphable: bool):
+        self.batch, self.graphable = batch, graphable
 
 
 class ModelRunner:
@@ -80,9 +80,7 @@ class ModelRunner:
         return sum(2 * s.num_kv_heads * s.head_dim * page_size * act for s in model.cache_specs() if isinstance(s, PagedKV))
 
     def prepare(self, entries: Sequence[StepEntry]) -> "PreparedStep":
-        """The host work of a step that does not need the device: the batch's arrays, the checks, the parts' plans.
-        The entries' requests must be in the state in which the step will find them (earlier steps committed, pages
-        reserved); their token ids may still be placeholders (``step`` puts the real ones in)."""
+        """The host work of a step that does not need the device: the batch's arrays, the checks, the parts' plans."""
         entries = list(entries)
         graphable = self.use_graphs and all(len(e.tokens) == 1 for e in entries) \
             and all(len(t) <= self.fixed_max_blocks for e in entries for t in e.cache.tables)
@@ -98,32 +96,31 @@ class ModelRunner:
             self._pack(batch)
         if graphable:
             batch.graph_key()
-        return PreparedStep(batch, graphable, [(e.cache, e.cache.num_tokens, tuple(e.cache.versions)) for e in entries])
+        return PreparedStep(batch, graphable)
 
-    def step(self, entries: Sequence[StepEntry], prepared: Optional["PreparedStep"] = None) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], token_source: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Run the entries' tokens as one batch.  Pages for them must have been reserved
         (``manager.reserve``).  Returns float32 logits [wanted rows, vocab] in the order of the
         entries and of their ``want`` (valid until the next step); afterwards the tokens count
-        as cached.  ``prepared``: what ``prepare`` made of the same entries ahead of time."""
+        as cached.  ``token_source``: int32 [T] on the device; the step's token ids are taken from there (on the
+        stream, after what produced them) instead of from the entries, whose tokens are placeholders then."""
         entries = list(entries)
         if not entries:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
-        if prepared is not None:
-            if any(c is not e.cache or c.num_tokens != n or tuple(c.versions) != v
-                   for e, (c, n, v) in zip(entries, prepared.state)) or len(entries) != len(prepared.state):
-                raise ValueError("the prepared step does not fit the requests' caches any more")
-            prepared.batch.set_token_ids(entries, self.model.vocab_size)
-        else:
-            prepared = self.prepare(entries)
+        prepared = self.prepare(entries)
         batch, graphable = prepared.batch, prepared.graphable
+        if token_source is not None and (token_source.dtype != torch.int32 or tuple(token_source.shape) != (batch.T,)):
+            raise ValueError("token_source must be int32 [%d]" % batch.T)
         self._reset_fresh_state(batch)
         if graphable:
-            logits = self._step_graph(batch)
+            logits = self._step_graph(batch, token_source)
         else:
             if self.device.type == "cuda":
                 self._upload(batch, None)
             else:
                 batch.upload()
+            if token_source is not None:
+                batch.token_ids.copy_(token_source)
             logits = self.model.forward(batch, self.storage)
         for e in entries:
             self.manager.commit(e.cache, len(e.tokens))
@@ -145,14 +142,10 @@ class ModelRunner:
         self._packed = batch
 
     def _upload(self, batch: StepBatch, dev_buf: Optional[torch.Tensor], bind: bool = True) -> None:
-        """Copy the packed arrays to the device with one transfer.  A batch that was packed ahead of its token ids
-        gets them patched in.  ``bind=False``: the device views are not needed (a graph that has them is replayed)."""
+        """Copy the packed arrays to the device with one transfer.  ``bind=False``: the device views are not needed (a
+        graph that has them is replayed)."""
         if self._packed is not batch:
             self._pack(batch)
-        elif batch.token_ids_late:
-            off, n = batch.packed_layout["token_ids"]
-            self._pinned.numpy()[off:off + n] = batch.host_array("token_ids")
-        batch.token_ids_late = False
         layout, total = batch.packed_layout, batch.packed_total
         if dev_buf is None:
             dev_buf = torch.empty(total, dtype=torch.int32, device=self.device)
@@ -164,12 +157,15 @@ class ModelRunner:
             batch.bind_device(dev_buf, layout)
 
     # ---- graphs -----------------------------------------------------------------
-    def _step_graph(self, batch: StepBatch) -> torch.Tensor:
+    def _step_graph(self, batch: StepBatch, token_source: Optional[torch.Tensor] = None) -> torch.Tensor:
         key = batch.graph_key()
         held = self._graphs.get(key)
         if held is not None:
             graph, dev_buf, logits = held
             self._upload(batch, dev_buf, bind=False)
+            if token_source is not None:
+                off, n = batch.packed_layout["token_ids"]
+                dev_buf[off:off + n].copy_(token_source)
             graph.replay()
             self.graph_replays += 1
             return logits
@@ -177,10 +173,14 @@ class ModelRunner:
             # first step of this shape: run it kernel by kernel (this also warms the library up)
             self._seen[key] = 1
             self._upload(batch, None)
+            if token_source is not None:
+                batch.token_ids.copy_(token_source)
             return self.model.forward(batch, self.storage)
         _layout, total = batch.layout()
         dev_buf = torch.empty(total, dtype=torch.int32, device=self.device)
         self._upload(batch, dev_buf)
+        if token_source is not None:
+            batch.token_ids.copy_(token_source)
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):

@@ -107,10 +107,11 @@ def test_cli_usage(capsys):
     assert "Available backends: hip" in capsys.readouterr().err
 
 
-def test_steps_prepared_ahead_change_nothing(folder_a, emu_ops):
-    """While a step of decoded tokens runs, the engine builds the next step's batch; it is dropped when a request ends
-    (by count or by its end token), arrives, or is removed in between.  The tokens that come out are those of an engine
-    that never prepares ahead, event by event; no page is lost."""
+def test_steps_run_ahead_change_nothing(folder_a, emu_ops):
+    """Before a step of decoded tokens has handed its tokens to the host, the engine launches the next one for the same
+    requests; not when a request ends by count or waits for admission; and when a request ends at its end token or is
+    removed, its row in the step in flight is ignored.  The tokens that come out are those of an engine that never
+    runs ahead, request by request; no page is lost."""
     from spyinfer_amd.engine.llm_engine import LLMEngine
     ps = prompts(256, [9, 30, 4, 21, 12], seed=7)
     plain = PlainQwen3(folder_a)
@@ -124,15 +125,13 @@ def test_steps_prepared_ahead_change_nothing(folder_a, emu_ops):
         eng = LLMEngine(folder_a, dtype="float32", device="cpu", max_model_len=128, num_kvcache_blocks=40, max_num_seqs=8)
         eng.eos_token_id = eos
         used = [0]
-        if not ahead:
-            eng._prepare_ahead = lambda scheduled: None
-        else:
-            real = eng._take_ahead
-            def counted():
-                got = real()
-                used[0] += got[0] is not None
-                return got
-            eng._take_ahead = counted
+        eng.run_ahead = ahead
+        real = eng._launch_ahead
+        def counted(flight):
+            got = real(flight)
+            used[0] += got is not None
+            return got
+        eng._launch_ahead = counted
         ids = [eng.add_request(ps[0], SamplingParams(max_new_tokens=25, ignore_eos=True)),
                eng.add_request(ps[1], SamplingParams(max_new_tokens=25)),                   # ends at its end token
                eng.add_request(ps[2], SamplingParams(max_new_tokens=7, ignore_eos=True))]   # ends by count
@@ -153,7 +152,10 @@ def test_steps_prepared_ahead_change_nothing(folder_a, emu_ops):
 
     log_a, out_a, used = run(True)
     log_b, out_b, _ = run(False)
-    assert log_a == log_b and out_a == out_b
-    assert used >= 15, "steps of decoded tokens alone must have come from the batch prepared ahead (%d did)" % used
+    # a request that arrives while a step is in flight joins one step later: the calls differ, the requests' tokens do not
+    per_request = lambda log: {rid: [t for step in log for r, t, _ in step if r == rid] for rid in range(5)}
+    assert per_request(log_a) == per_request(log_b) and out_a == out_b
+    assert [f for step in log_a for _, _, f in step].count(True) == [f for step in log_b for _, _, f in step].count(True) == 4
+    assert used >= 15, "steps of decoded tokens alone must have been launched ahead (%d were)" % used
     assert out_a[0] == g1[:k + 1]                              # the second request ended at its end token
     assert out_a[1] == plain.greedy(ps[2], 7) and out_a[2] == plain.greedy(ps[3], 9)
