@@ -53,6 +53,32 @@ def test_greedy_float32_equals_plain(folder_a, eager):
         eng.runner.manager.check()
 
 
+@pytest.mark.parametrize("eager", [True, False])
+def test_requests_ending_while_a_step_is_in_flight(folder_a, eager):
+    """Decode steps are launched ahead of the host.  Requests here end at an end-of-sequence token, which the host learns
+    one step late: the step in flight still holds their row, their pages go back at once and are taken by requests
+    that waited (the pool is small).  Every request's tokens are the plain implementation's, cut at its end token."""
+    from collections import Counter
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    require_gpu()
+    ps = prompts(256, [5, 17, 33, 9, 26, 40, 12, 21], 11)
+    plain = PlainQwen3(folder_a)
+    full = [plain.greedy(p, 14) for p in ps]
+    eos = Counter(t for g in full for t in g[2:]).most_common(1)[0][0]
+    want = [g[:g.index(eos) + 1] if eos in g else g for g in full]
+    assert sum(len(w) < 14 for w in want) >= 2, "the chosen end token must end some requests early"
+    eng = LLMEngine(folder_a, dtype="float32", max_model_len=128, num_kvcache_blocks=11, max_num_seqs=3, enforce_eager=eager)
+    eng.eos_token_id = eos
+    ahead = [0]
+    real = eng._launch_ahead
+    eng._launch_ahead = lambda flight: (lambda got: (ahead.__setitem__(0, ahead[0] + (got is not None)), got)[1])(real(flight))
+    assert eng.generate(ps, SamplingParams(max_new_tokens=14)) == want
+    assert ahead[0] >= 10
+    eng.runner.manager.check()
+    assert eng.runner.manager.num_free_pages() == [11]
+
+
 def test_greedy_bfloat16_follows_plain(folder_a):
     """bfloat16 may leave the plain tokens only where the plain logits nearly tie."""
     from spyinfer_amd.engine.llm_engine import LLMEngine
