@@ -145,7 +145,7 @@ def main() -> int:
         "config": {"model": "Qwen3-8B shape", "layers": L, "layers_of_model": model_layers, "hidden": H, "q_heads": nq,
                    "kv_heads": nkv, "head_dim": d, "intermediate": I, "vocab": V, "global_batch": args.batch,
                    "seq_len": args.context, "prompt_len": args.prompt_len, "mean_context": round(ctx, 1), "page_size": page,
-                   "graphs": not args.enforce_eager, "parallelism": "single GPU"},
+                   "graphs": not args.enforce_eager, "run_ahead": bool(eng.run_ahead), "parallelism": "single GPU"},
         "prefill": {"value": round(T / pf, 1), "tokens": T, "ms": round(pf * 1e3, 3),
                     "frac": round(pf_flops / pf / PEAK_FLOPS[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
