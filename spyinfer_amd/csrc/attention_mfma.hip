@@ -122,11 +122,13 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     const int tile = blockIdx.x, hk = blockIdx.y, sp = blockIdx.z;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: loops over it stay scalar
     const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
-    const int s = tile_entry[tile];
-    const int row0 = tile_row0[tile];
+    // FUSED: every entry is one token and has one tile (the host has checked it), so tile t is entry t with query token t:
+    // two dependent loads less before the first key can be asked for
+    const int s = FUSED ? tile : tile_entry[tile];
+    const int row0 = FUSED ? 0 : tile_row0[tile];
     const int G = n_q / n_kv;
-    const int q0 = cu_q[s];
-    const int n = cu_q[s + 1] - q0;
+    const int q0 = FUSED ? s : cu_q[s];
+    const int n = FUSED ? 1 : cu_q[s + 1] - q0;
     const int nrows = n * G;
     const int p0 = pos0[s];
     const int kvl = kv_len[s];
