@@ -16,7 +16,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, RequestCache
-from ..kernels.ops import AttentionMeta
+from ..kernels.ops import AttentionMeta, key_parts_for
 
 ROWS_PER_TILE = 16        # rows of (token, head-in-group) pairs in a small attention tile
 ROWS_PER_BIG_TILE = 128   # rows in a tile of the prefill attention kernel
@@ -171,7 +171,7 @@ class StepBatch:
     def graph_key(self):
         """What a captured graph of this step depends on beside the arrays' contents."""
         if self._graph_key is None:
-            self._graph_key = (self.layout_key(), self.all_rows_wanted)
+            self._graph_key = (self.layout_key(), self.all_rows_wanted, key_parts_for(self.max_kv_len))
         return self._graph_key
 
     def host_array(self, name: str) -> np.ndarray:

@@ -410,11 +410,20 @@ class AttentionMeta:
         self.token_entry, self.positions = token_entry, positions
         self.S, self.T, self.max_blocks, self.max_kv_len, self.max_q_len = S, T, max_blocks, max_kv_len, max_q_len
         self.tiles, self.tiles_group = tiles, tiles_group
-        #: True: launch shapes must not depend on the requests' lengths (the step is captured in a graph)
+        #: True: the step is captured in a graph (block tables have a fixed width; what a launch's shape takes from the
+        #: requests' lengths, the number of key parts, is part of the graph's key)
         self.fixed_shape = fixed_shape
 
 
 MFMA_ATTENTION = True      # False forces the plain kernel for bfloat16 too (used by tests)
+DECODE_MAX_SPLITS = 16      # most key parts of a tile (the merge kernel's time grows with them)
+DECODE_KEYS_PER_SPLIT = 256  # a part wants this many keys at least (measured at 1100 keys, 1 to 4 requests: 4-8 parts best)
+
+
+def key_parts_for(max_kv_len: int) -> int:
+    """The most parts into which the keys of 16-row tiles are split when the longest request has ``max_kv_len`` keys.
+    A step captured in a graph keeps the number it was captured with, so this number belongs to the graph's key."""
+    return max(1, min(DECODE_MAX_SPLITS, -(-int(max_kv_len) // DECODE_KEYS_PER_SPLIT)))
 DECODE_SPLIT_TARGET = 256   # blocks (of 4 waves) wanted in flight when all entries are single tokens (measured: B=8 best at 4 parts)
 
 
@@ -527,8 +536,7 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
             # Few 16-row tiles cannot fill the chip by themselves (decoding requests, short portions): their keys are
             # split into parts, each part a block of 4 waves that wants 128 keys at least, and a second kernel merges.
             want = max(1, DECODE_SPLIT_TARGET // max(1, n_small * n_kv))
-            by_len = 16 if meta.fixed_shape else -(-meta.max_kv_len // 128)
-            splits = max(1, min(want, by_len, 16))
+            splits = max(1, min(want, key_parts_for(meta.max_kv_len)))
             ws_floats = hip().lib.spy_attention_mfma_workspace(ctypes.c_int(n_small), ctypes.c_int(n_kv), ctypes.c_int(d),
                                                                ctypes.c_int(splits))
             ws = torch.empty((max(1, ws_floats),), dtype=torch.float32, device=q.device)

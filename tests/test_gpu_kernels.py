@@ -423,12 +423,12 @@ FUSED_CASES = [
 
 @pytest.mark.parametrize("case", range(len(FUSED_CASES)))
 @pytest.mark.parametrize("wdtype", DTYPES)
-@pytest.mark.parametrize("fixed", [False, True])
-def test_attention_taking_the_raw_product(case, wdtype, fixed):
+@pytest.mark.parametrize("keys_per_part", [256, 32])
+def test_attention_taking_the_raw_product(case, wdtype, keys_per_part, monkeypatch):
     """Single tokens: the attention kernel norms and rotates q and the new key itself, uses the new key and value and
     stores them.  The slots of the new tokens hold NaN before the call, so a kernel that read them before writing, or
     did not write, fails; the rest of the cache must stay as it was.  Positions at the edges of pages and of 32-key
-    blocks; one and several parts of the keys (fixed shapes take 16 parts)."""
+    blocks; few and many parts of the keys."""
     from spyinfer_amd.kernels import ops
     from spyinfer_amd.parts.rotary import RotaryEmbedding
     dev = require_gpu()
@@ -436,7 +436,7 @@ def test_attention_taking_the_raw_product(case, wdtype, fixed):
     dtype, theta, eps = torch.bfloat16, 23456.0, 1e-5
     entries = [(a, 1) for a in cached]
     _q, kc, vc, bt, te, ps, meta = make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed=50 + case, window=window)
-    meta.fixed_shape = fixed
+    monkeypatch.setattr(ops, "DECODE_KEYS_PER_SPLIT", keys_per_part)
     T = len(entries)
     qkv = rnd((T, (n_q + 2 * n_kv) * d), dtype, "cpu", 60 + case)
     qw = (1 + 0.2 * rnd((d,), torch.float32, "cpu", 61)).to(wdtype) if norm else None
