@@ -10,6 +10,10 @@
 //             rounding of the operand to bfloat16 happens before the scale, which changes nothing in its
 //             relative size.
 //   EPI_GATED W = [gate | up] tiles, the block stores silu(gate) * up.
+//   XT / OT   the input X / the bfloat16 output that the next product reads (bf16(h w) of EPI_RESID, the result of
+//             EPI_GATED) in MFMA operand order instead of row-major: [K/32 steps][64 lanes][8], lane 16 g + r of step s
+//             holding x[r][32 s + 8 g ..] for the 16 rows of the tile (rows beyond M hold anything).  An operand is then
+//             one load of 1 KiB in one piece, as for W, instead of 16 pieces of 64 bytes: 5-12 % at 16 rows.
 //   EPI_STORE the block stores the result (bfloat16 or float32).
 //
 // W comes as a copy in the order the kernel reads it (ops.tile_weight): [K/128 chunks][N/16 tiles][4 steps][64 lanes][8],
@@ -33,7 +37,10 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 #define EPI_GATED 1
 #define EPI_RESID 2
 
-template <int EPI, bool SCALED, typename TC, int GD_WAVES>
+// Where element (row m, column n) of a [16, N] matrix lies in operand order (see XT / OT above), in elements.
+__device__ __forceinline__ size_t operand_order(int m, int n) { return ((size_t)(n >> 5) * 64 + ((n & 31) >> 3) * 16 + m) * 8 + (n & 7); }
+
+template <int EPI, bool SCALED, typename TC, int GD_WAVES, bool XT, bool OT>
 __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, float* __restrict__ resid_out,
     bf16_t* __restrict__ xw_out, const bf16_t* __restrict__ w_next, float* __restrict__ ss_out, const float* __restrict__ ss_in,
@@ -75,17 +82,17 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) woff[nt] = (unsigned)(nt * N / 16) * 4096u + 16u * lane;
     const char* xbase = reinterpret_cast<const char*>(X);
-    const unsigned xoff = (unsigned)min(r, M - 1) * (unsigned)K * 2u + 16u * g;
+    const unsigned xoff = XT ? 16u * lane : (unsigned)min(r, M - 1) * (unsigned)K * 2u + 16u * g;
 
     bf16x8_t a0[NT][4], a1[NT][4], b0[4], b1[4];
 #define GD_LOAD(A, B, CHUNK)                                                                             \
     {                                                                                                    \
         const char* wb_ = wbase + (size_t)(CHUNK) * chunk_stride;                                        \
-        const char* xb_ = xbase + (size_t)(CHUNK) * (GD_CHUNK * 2) + xoff;                               \
+        const char* xb_ = xbase + (size_t)(CHUNK) * (XT ? 4096 : GD_CHUNK * 2) + xoff;                   \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                  \
             _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                            \
                 A[nt][j] = *reinterpret_cast<const bf16x8_t*>(wb_ + woff[nt] + 1024 * j);                \
-            B[j] = x_ok ? *reinterpret_cast<const bf16x8_t*>(xb_ + 64 * j) : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; \
+            B[j] = x_ok ? *reinterpret_cast<const bf16x8_t*>(xb_ + (XT ? 1024 : 64) * j) : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; \
         }                                                                                                \
     }
 #define GD_MFMA(A, B, ACC)                                                                               \
@@ -153,7 +160,7 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
             uint2 o;
             o.x = pack_bf16x2(h[0] * __uint_as_float(wn.x << 16), h[1] * __uint_as_float(wn.x & 0xffff0000u));
             o.y = pack_bf16x2(h[2] * __uint_as_float(wn.y << 16), h[3] * __uint_as_float(wn.y & 0xffff0000u));
-            *reinterpret_cast<uint2*>(xw_out + (size_t)m * N + n) = o;
+            *reinterpret_cast<uint2*>(xw_out + (OT ? operand_order(m, n) : (size_t)m * N + n)) = o;
         }
         s += __shfl_xor(s, 16, 64);
         s += __shfl_xor(s, 32, 64);
@@ -161,7 +168,7 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
         return;
     }
     if (m >= M) return;
-    TC* out = C + (size_t)m * N + n;
+    TC* out = C + (OT ? operand_order(m, n) : (size_t)m * N + n);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         float v = acc[0][i];
@@ -172,25 +179,33 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
 
 struct GdArgs {
     const bf16_t* x; const bf16_t* w; void* c; float* resid; bf16_t* xw_out; const bf16_t* w_next; float* ss_out; const float* ss_in;
-    int n_parts; float eps; int M, N, K; hipStream_t st;
+    int n_parts; float eps; int M, N, K; bool xt, ot; hipStream_t st;
 };
 
 // Blocks of 8 waves, one per 16 columns; the gated product (two tiles per block, usually three blocks per CU)
 // takes blocks of GD_WAVES_GATED waves so that all of them are resident at once.
+template <int EPI, bool SCALED, typename TC, bool XT, bool OT>
+static void gd_launch2(const GdArgs& a) {
+    constexpr int W = EPI == EPI_GATED ? GD_WAVES_GATED : 8;
+    gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(a.x, a.w, (TC*)a.c, a.resid, a.xw_out, a.w_next, a.ss_out,
+                                                                                a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K);
+}
+
 template <int EPI, bool SCALED, typename TC>
 static void gd_launch(const GdArgs& a) {
-    constexpr int W = EPI == EPI_GATED ? GD_WAVES_GATED : 8;
-    gemm_decode_kernel<EPI, SCALED, TC, W><<<a.N / 16, W * 64, 0, a.st>>>(a.x, a.w, (TC*)a.c, a.resid, a.xw_out, a.w_next, a.ss_out, a.ss_in,
-                                                                        a.n_parts, a.eps, a.M, a.N, a.K);
+    constexpr bool CAN_OT = EPI != EPI_STORE && sizeof(TC) == 2;      // operand order is for bfloat16 that a product reads next
+    if (a.xt) { if (CAN_OT && a.ot) gd_launch2<EPI, SCALED, TC, true, CAN_OT>(a); else gd_launch2<EPI, SCALED, TC, true, false>(a); }
+    else { if (CAN_OT && a.ot) gd_launch2<EPI, SCALED, TC, false, CAN_OT>(a); else gd_launch2<EPI, SCALED, TC, false, false>(a); }
 }
 
 // x: bfloat16 [M, K].  scaled != 0: x = bf16(h * w_norm) and ss_in [n_parts, 16] holds the parts of sum(h^2); the
 // result is multiplied by rsqrt(sum / K + eps).
 // epi 0: C [M, N] (c_dtype);  epi 1: W = [gate | up], C [M, N] = silu(gate) * up;  epi 2: resid [M, N] += result,
 // xw_out [M, N] = bf16(resid * w_next), ss_out [N / 16, 16] = every block's part of the rows' sums of squares.
+// x_tiled / out_tiled: X / the bfloat16 output for the next product (xw_out of epi 2, C of epi 1) are in operand order.
 extern "C" int spy_gemm_decode(const void* X, int scaled, const float* ss_in, int n_parts, float eps, const void* Wt, int epi,
                                void* C, int c_dtype, float* resid, void* xw_out, const void* w_next, float* ss_out, int M, int N,
-                               int K, hipStream_t st) {
+                               int K, int x_tiled, int out_tiled, hipStream_t st) {
     SPY_REQUIRE(M > 0 && M <= 16, "spy_gemm_decode: M = %d rows (1..16 allowed)", M);
     SPY_REQUIRE(N > 0 && N % 16 == 0 && K > 0 && K % 128 == 0, "spy_gemm_decode: N = %d must be a multiple of 16 and K = %d of 128", N, K);
     SPY_REQUIRE(epi >= 0 && epi <= 2, "spy_gemm_decode: unknown epilogue %d", epi);
@@ -201,7 +216,10 @@ extern "C" int spy_gemm_decode(const void* X, int scaled, const float* ss_in, in
                 "spy_gemm_decode: the residual epilogue needs the stream, the next norm's weight and its outputs");
     SPY_REQUIRE(epi == EPI_RESID || (C && ((uintptr_t)C % 16) == 0), "spy_gemm_decode: no output");
     SPY_REQUIRE((long long)N * 256 + 8192 < (1ll << 32), "spy_gemm_decode: N = %d is too large for 32-bit offsets inside a chunk", N);
-    GdArgs a = {(const bf16_t*)X, (const bf16_t*)Wt, C, resid, (bf16_t*)xw_out, (const bf16_t*)w_next, ss_out, ss_in, n_parts, eps, M, N, K, st};
+    SPY_REQUIRE(!out_tiled || (N % 32 == 0 && (epi == EPI_RESID || (epi == EPI_GATED && c_dtype == SPY_BF16))),
+                "spy_gemm_decode: operand order is for the bfloat16 output of the gated and the residual epilogue, N a multiple of 32");
+    GdArgs a = {(const bf16_t*)X, (const bf16_t*)Wt, C, resid, (bf16_t*)xw_out, (const bf16_t*)w_next, ss_out, ss_in, n_parts, eps, M, N, K,
+                x_tiled != 0, out_tiled != 0, st};
     const bool f32 = c_dtype == SPY_F32;
     if (epi == EPI_RESID) { if (scaled) gd_launch<EPI_RESID, true, bf16_t>(a); else gd_launch<EPI_RESID, false, bf16_t>(a); }
     else if (epi == EPI_GATED) {

@@ -251,20 +251,41 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, tiled: Optional[torc
 
 # --------------------------------------------------------------------------
 # Decode-time products with the norm and the residual sum folded in
+class OperandRows:
+    """At most 16 rows of bfloat16 [M, K] in the order the MFMA operand wants them: ``data`` is [K/32 steps, 64 lanes,
+    8] with lane 16 g + r of step s holding x[r][32 s + 8 g ..]; rows M..15 hold anything.  The decode products write
+    their outputs for each other this way (an operand is then one load of 1 KiB in one piece)."""
+    __slots__ = ("data", "rows", "width")
+
+    def __init__(self, data: torch.Tensor, rows: int, width: int):
+        self.data, self.rows, self.width = data, rows, width
+
+    @staticmethod
+    def empty(rows: int, width: int, device) -> "OperandRows":
+        _check(0 < rows <= 16 and width % 32 == 0, "operand order takes 1..16 rows of a width that is a multiple of 32")
+        return OperandRows(torch.empty((width // 32, 64, 8), dtype=torch.bfloat16, device=device), rows, width)
+
+    def to_rows(self) -> torch.Tensor:
+        """The same values as an ordinary [M, K] tensor (for tests; not used by the engine)."""
+        return self.data.view(self.width // 32, 4, 16, 8).permute(2, 0, 1, 3).reshape(16, self.width)[:self.rows].contiguous()
+
+
 class ScaledInput:
     """The input of a product as 'the RMS norm of the residual stream' with the scale still to come:
-    ``xw [M, K]`` = bfloat16(h * w_norm), and the parts ``ss_parts [n, 16]`` of every row's sum of squares
-    (row r of the stream in column r; their sum over n is sum(h[r]^2)).  ``decode_linear`` and
+    ``xw`` = bfloat16(h * w_norm), as [M, K] or as OperandRows, and the parts ``ss_parts [n, 16]`` of every row's sum
+    of squares (row r of the stream in column r; their sum over n is sum(h[r]^2)).  ``decode_linear`` and
     ``decode_linear_swiglu`` multiply their result by rsqrt(sum / K + eps), which equals the product with the
     normed rows.  ``norm`` is the norm part this was prepared for."""
     __slots__ = ("xw", "ss_parts", "eps", "norm")
 
-    def __init__(self, xw: torch.Tensor, ss_parts: torch.Tensor, eps: float, norm=None):
+    def __init__(self, xw, ss_parts: torch.Tensor, eps: float, norm=None):
         self.xw, self.ss_parts, self.eps, self.norm = xw, ss_parts, float(eps), norm
 
 
 #: False switches the folded decode products off (every norm then runs as a kernel of its own).
 FUSED_DECODE = True
+#: False: the decode products hand their outputs to each other row-major
+OPERAND_ORDER = True
 
 
 def fused_decode_ok(rows: int, act_dtype, *tiled_weights) -> bool:
@@ -285,48 +306,74 @@ def _gemm_decode(x, tiled: torch.Tensor, epi: int, n_out: int, out, resid, xw_ou
                "decode product: the parts of the sums of squares must be float32 [n, 16]")
     else:
         xs, ss, eps = x, None, 0.0
-    _dev(xs, ss, tiled, out, resid, xw_out, w_next, ss_out)
-    _check(xs.dtype == torch.bfloat16 and xs.dim() == 2 and xs.shape[1] == K, "decode product: x must be bfloat16 [M, %d]" % K)
-    M = xs.shape[0]
+    x_tiled = isinstance(xs, OperandRows)
+    if x_tiled:
+        _check(xs.width == K and tuple(xs.data.shape) == (K // 32, 64, 8) and xs.data.dtype == torch.bfloat16,
+               "decode product: x in operand order must be bfloat16 [%d / 32, 64, 8]" % K)
+        M, xs = xs.rows, xs.data
+    else:
+        _check(xs.dtype == torch.bfloat16 and xs.dim() == 2 and xs.shape[1] == K, "decode product: x must be bfloat16 [M, %d]" % K)
+        M = xs.shape[0]
+    out_tiled = isinstance(out, OperandRows) or isinstance(xw_out, OperandRows)
+    for o in (out, xw_out):
+        if isinstance(o, OperandRows):
+            _check(o.rows == M and o.width == n_out and tuple(o.data.shape) == (n_out // 32, 64, 8),
+                   "decode product: the output in operand order does not fit")
+    out_t = out.data if isinstance(out, OperandRows) else out
+    xw_t = xw_out.data if isinstance(xw_out, OperandRows) else xw_out
+    _dev(xs, ss, tiled, out_t, resid, xw_t, w_next, ss_out)
     _check(0 < M <= FUSED_DECODE_MAX_ROWS, "decode product: %d rows (1..%d allowed)" % (M, FUSED_DECODE_MAX_ROWS))
     hip().call("spy_gemm_decode", _ptr(xs), ctypes.c_int(0 if ss is None else 1), _ptr(ss), ctypes.c_int(0 if ss is None else ss.shape[0]),
-               ctypes.c_float(eps), _ptr(tiled), ctypes.c_int(epi), _ptr(out), ctypes.c_int(0 if out is None else _code(out, "out")),
-               _ptr(resid), _ptr(xw_out), _ptr(w_next), _ptr(ss_out), ctypes.c_int(M), ctypes.c_int(n_out), ctypes.c_int(K),
-               _Hip.stream())
+               ctypes.c_float(eps), _ptr(tiled), ctypes.c_int(epi), _ptr(out_t), ctypes.c_int(0 if out_t is None else _code(out_t, "out")),
+               _ptr(resid), _ptr(xw_t), _ptr(w_next), _ptr(ss_out), ctypes.c_int(M), ctypes.c_int(n_out), ctypes.c_int(K),
+               ctypes.c_int(1 if x_tiled else 0), ctypes.c_int(1 if out_tiled else 0), _Hip.stream())
 
 
 def _rows_of(x) -> int:
-    return (x.xw if isinstance(x, ScaledInput) else x).shape[0]
+    x = x.xw if isinstance(x, ScaledInput) else x
+    return x.rows if isinstance(x, OperandRows) else x.shape[0]
+
+
+def _operand_order_ok(width: int) -> bool:
+    return OPERAND_ORDER and width % 32 == 0
 
 
 def decode_linear(x, tiled: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
-    """y = x . w^T for at most 16 rows; ``x`` bfloat16 [M, K] or a ScaledInput, ``tiled`` from tile_weight."""
+    """y = x . w^T for at most 16 rows; ``x`` bfloat16 [M, K], OperandRows or a ScaledInput, ``tiled`` from tile_weight."""
     N = tiled.shape[0]
     out = torch.empty((_rows_of(x), N), dtype=out_dtype, device=tiled.device)
     _gemm_decode(x, tiled, 0, N, out, None, None, None, None)
     return out
 
 
-def decode_linear_swiglu(x, tiled_gate_up: torch.Tensor) -> torch.Tensor:
-    """silu(x . Wgate^T) * (x . Wup^T) for at most 16 rows; ``tiled_gate_up [2 I, K]`` = tiles of [Wgate | Wup]."""
+def decode_linear_swiglu(x, tiled_gate_up: torch.Tensor, for_product: bool = False):
+    """silu(x . Wgate^T) * (x . Wup^T) for at most 16 rows; ``tiled_gate_up [2 I, K]`` = tiles of [Wgate | Wup].
+    ``for_product``: the result goes into another decode product only, and may come as OperandRows."""
     _check(tiled_gate_up.shape[0] % 32 == 0, "decode_linear_swiglu: [2 I, K] with I a multiple of 16 expected")
     I = tiled_gate_up.shape[0] // 2
-    out = torch.empty((_rows_of(x), I), dtype=torch.bfloat16, device=tiled_gate_up.device)
+    if for_product and _operand_order_ok(I):
+        out = OperandRows.empty(_rows_of(x), I, tiled_gate_up.device)
+    else:
+        out = torch.empty((_rows_of(x), I), dtype=torch.bfloat16, device=tiled_gate_up.device)
     _gemm_decode(x, tiled_gate_up, 1, I, out, None, None, None, None)
     return out
 
 
-def decode_linear_residual(x: torch.Tensor, tiled: torch.Tensor, resid: torch.Tensor, next_norm_weight: torch.Tensor,
+def decode_linear_residual(x, tiled: torch.Tensor, resid: torch.Tensor, next_norm_weight: torch.Tensor,
                            eps: float, norm=None) -> ScaledInput:
     """resid += x . w^T (float32, in place) for at most 16 rows -> the ScaledInput of the norm that reads the
     stream next: bfloat16(resid * next_norm_weight) and the parts [N / 16, 16] of the new rows' sums of squares."""
     N = tiled.shape[0]
-    _check(resid.dtype == torch.float32 and resid.dim() == 2 and resid.shape == (_rows_of(x), N),
+    M = _rows_of(x)
+    _check(resid.dtype == torch.float32 and resid.dim() == 2 and resid.shape == (M, N),
            "decode_linear_residual: the stream must be float32 [M, %d]" % N)
     _check(next_norm_weight.dtype == torch.bfloat16 and next_norm_weight.shape == (N,),
            "decode_linear_residual: the next norm's weight must be bfloat16 [%d]" % N)
     ss = torch.empty((N // 16, 16), dtype=torch.float32, device=resid.device)
-    xw = torch.empty((resid.shape[0], N), dtype=torch.bfloat16, device=resid.device)
+    if _operand_order_ok(N):
+        xw = OperandRows.empty(M, N, resid.device)
+    else:
+        xw = torch.empty((M, N), dtype=torch.bfloat16, device=resid.device)
     _gemm_decode(x, tiled, 2, N, None, resid, xw, next_norm_weight, ss)
     return ScaledInput(xw, ss, eps, norm)
 
@@ -339,10 +386,12 @@ def embedding_scaled(ids: torch.Tensor, table: torch.Tensor, norm_weight: torch.
     T, (V, H) = ids.shape[0], table.shape
     _check(norm_weight.dtype == torch.bfloat16 and norm_weight.shape == (H,), "embedding_scaled: the norm weight must be bfloat16 [H]")
     out = torch.empty((T, H), dtype=torch.float32, device=table.device)
-    xw = torch.empty((T, H), dtype=torch.bfloat16, device=table.device)
+    tiled = _operand_order_ok(H)
+    xw = OperandRows.empty(T, H, table.device) if tiled else torch.empty((T, H), dtype=torch.bfloat16, device=table.device)
     ss = torch.empty((1, 16), dtype=torch.float32, device=table.device)
-    hip().call("spy_embedding_sumsq", _ptr(out), _ptr(xw), _ptr(ss), _ptr(table), _code(table, "embedding table"), _ptr(norm_weight),
-               _ptr(ids), ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(V), _Hip.stream())
+    hip().call("spy_embedding_sumsq", _ptr(out), _ptr(xw.data if tiled else xw), _ptr(ss), _ptr(table), _code(table, "embedding table"),
+               _ptr(norm_weight), _ptr(ids), ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(V), ctypes.c_int(1 if tiled else 0),
+               _Hip.stream())
     return out, ScaledInput(xw, ss, eps, norm)
 
 

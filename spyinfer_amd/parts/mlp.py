@@ -42,5 +42,5 @@ class GatedMLP(FeedForward):
 
     def forward_into(self, x, batch, resid, next_norm):
         weight, eps = next_norm.foldable(batch.act_dtype)
-        return ops.decode_linear_residual(ops.decode_linear_swiglu(x, self.w_gate_up_tiled), self.w_down_tiled, resid, weight, eps,
-                                          next_norm)
+        return ops.decode_linear_residual(ops.decode_linear_swiglu(x, self.w_gate_up_tiled, for_product=True), self.w_down_tiled,
+                                          resid, weight, eps, next_norm)

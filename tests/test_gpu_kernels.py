@@ -136,7 +136,8 @@ def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
     si = ops.decode_linear_residual(a, ops.tile_weight(w_in), resid, wn1, eps)
     h = resid0.double() + a.double() @ w_in.double().t()
     close(resid, h, torch.float32, scale=4.0, what="stream after the residual epilogue")
-    assert torch.equal(si.xw, (resid * wn1.float()).bfloat16()), "the prepared input is bf16(h * w) of the new stream"
+    assert isinstance(si.xw, ops.OperandRows), "outputs for the next product come in operand order"
+    assert torch.equal(si.xw.to_rows(), (resid * wn1.float()).bfloat16()), "the prepared input is bf16(h * w) of the new stream"
     ss = si.ss_parts.sum(0)
     assert torch.allclose(ss[:M], (resid * resid).sum(1), rtol=1e-5) and (M == 16 or float(ss[M:].abs().max()) == 0.0)
     # 2. products of the normed rows: plain, float32 result (logits), gated
@@ -152,7 +153,28 @@ def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
     si2 = ops.decode_linear_residual(si, ops.tile_weight(w_sq), resid2, wn2, eps)
     h2 = resid.double() + norm64(resid, wn1) @ w_sq.double().t()
     close(resid2, h2, torch.bfloat16, scale=2.0, what="stream after a scaled product")
-    assert torch.equal(si2.xw, (resid2 * wn2.float()).bfloat16())
+    assert torch.equal(si2.xw.to_rows(), (resid2 * wn2.float()).bfloat16())
+    # the same chain with row-major hand-over gives the same numbers
+    ops.OPERAND_ORDER = False
+    try:
+        resid_r = resid0.clone()
+        si_r = ops.decode_linear_residual(a, ops.tile_weight(w_in), resid_r, wn1, eps)
+        assert not isinstance(si_r.xw, ops.OperandRows) and torch.equal(si_r.xw, si.xw.to_rows()) and torch.equal(resid_r, resid)
+        assert torch.equal(ops.decode_linear(si_r, ops.tile_weight(w_qkv)), ops.decode_linear(si, ops.tile_weight(w_qkv)))
+        g_rows = ops.decode_linear_swiglu(si_r, ops.tile_weight(w_gu), for_product=True)
+    finally:
+        ops.OPERAND_ORDER = True
+    g_tiled = ops.decode_linear_swiglu(si, ops.tile_weight(w_gu), for_product=True)
+    assert isinstance(g_tiled, ops.OperandRows) and torch.equal(g_tiled.to_rows(), g_rows)
+    w_dn = rnd((H, I), torch.bfloat16, dev, 40, 0.05)
+    ra, rb = resid.clone(), resid.clone()
+    sa = ops.decode_linear_residual(g_tiled, ops.tile_weight(w_dn), ra, wn2, eps)
+    ops.OPERAND_ORDER = False
+    try:
+        sb = ops.decode_linear_residual(g_rows, ops.tile_weight(w_dn), rb, wn2, eps)
+    finally:
+        ops.OPERAND_ORDER = True
+    assert torch.equal(ra, rb) and torch.equal(sa.xw.to_rows(), sb.xw) and torch.equal(sa.ss_parts, sb.ss_parts)
     # 4. the scale matters: another eps or a missing part changes the result by far more than the tolerance
     far = ops.decode_linear(ops.ScaledInput(si.xw, si.ss_parts * 4.0, eps), ops.tile_weight(w_qkv), torch.float32)
     ref = (norm64(resid, wn1) @ w_qkv.double().t()).float()
@@ -161,7 +183,7 @@ def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
     table = rnd((50, H), torch.bfloat16, dev, 39)
     ids = torch.tensor([7, 0, 49, 7][:min(M, 4)], dtype=torch.int32, device=dev)
     out, e = ops.embedding_scaled(ids, table, wn1, eps)
-    assert torch.equal(out, ops.embedding(ids, table)) and torch.equal(e.xw, (out * wn1.float()).bfloat16())
+    assert torch.equal(out, ops.embedding(ids, table)) and torch.equal(e.xw.to_rows(), (out * wn1.float()).bfloat16())
     assert torch.allclose(e.ss_parts[0, :len(ids)], (out * out).sum(1), rtol=1e-5) and float(e.ss_parts[0, len(ids):].abs().max()) == 0.0
 
 
