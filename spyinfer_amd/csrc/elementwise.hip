@@ -25,9 +25,10 @@ extern "C" int spy_embedding(float* out, const void* table, int table_dtype, con
     return 0;
 }
 
-// The same for at most 16 tokens, prepared for a product that applies the first RMS norm's scale after its sum:
-// xw[t] = bf16(h[t] * w_norm) and ss[t] = sum(h[t]^2) (ss[T..15] = 0).
-// tiled: xw in MFMA operand order, [H/32][64 lanes][8] with lane 16 g + t holding xw[t][32 s + 8 g ..] (H % 32 == 0).
+// The same for at most 64 tokens, prepared for a product that applies the first RMS norm's scale after its sum:
+// xw[t] = bf16(h[t] * w_norm) and ss[t] = sum(h[t]^2) (ss[T ..] = 0 up to the next multiple of 16).
+// tiled: xw in MFMA operand order, [H/32][MT row tiles][64 lanes][8] with lane 16 g + t % 16 of row tile t / 16 holding
+// xw[t][32 s + 8 g ..] (H % 32 == 0); MT = the row tiles that T tokens need.  One block per row of ss (16 MT of them).
 template <typename TW>
 __global__ __launch_bounds__(256) void embedding_sumsq_kernel(float* __restrict__ out, bf16_t* __restrict__ xw, float* __restrict__ ss,
                                                               const TW* __restrict__ table, const bf16_t* __restrict__ w_norm,
@@ -45,7 +46,7 @@ __global__ __launch_bounds__(256) void embedding_sumsq_kernel(float* __restrict_
         const float v = known ? to_f32<TW>(row[i]) : 0.f;
         o[i] = v;
         const bf16_t y = f32_to_bf16(v * bf16_to_f32(w_norm[i]));
-        if (tiled) xw[((size_t)(i >> 5) * 64 + ((i & 31) >> 3) * 16 + t) * 8 + (i & 7)] = y;
+        if (tiled) xw[(((size_t)(i >> 5) * (gridDim.x >> 4) + (t >> 4)) * 64 + ((i & 31) >> 3) * 16 + (t & 15)) * 8 + (i & 7)] = y;
         else x[i] = y;
         s += v * v;
     }
@@ -55,9 +56,9 @@ __global__ __launch_bounds__(256) void embedding_sumsq_kernel(float* __restrict_
 
 extern "C" int spy_embedding_sumsq(float* out, void* xw, float* ss, const void* table, int table_dtype, const void* w_norm,
                                    const int* ids, int T, int H, int V, int tiled, hipStream_t st) {
-    SPY_REQUIRE(T > 0 && T <= 16 && H > 0 && V > 0, "spy_embedding_sumsq: T = %d tokens (1..16 allowed)", T);
+    SPY_REQUIRE(T > 0 && T <= 64 && H > 0 && V > 0, "spy_embedding_sumsq: T = %d tokens (1..64 allowed)", T);
     SPY_REQUIRE(!tiled || H % 32 == 0, "spy_embedding_sumsq: operand order needs a width that is a multiple of 32, not %d", H);
-    SPY_DISPATCH(table_dtype, TW, embedding_sumsq_kernel<TW><<<16, 256, 0, st>>>(out, (bf16_t*)xw, ss, (const TW*)table,
+    SPY_DISPATCH(table_dtype, TW, embedding_sumsq_kernel<TW><<<(T + 15) / 16 * 16, 256, 0, st>>>(out, (bf16_t*)xw, ss, (const TW*)table,
                                                                                  (const bf16_t*)w_norm, ids, T, H, V, tiled));
     SPY_CHECK_LAUNCH("spy_embedding_sumsq");
     return 0;

@@ -37,8 +37,11 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 #define EPI_GATED 1
 #define EPI_RESID 2
 
-// Where element (row m, column n) of a [16, N] matrix lies in operand order (see XT / OT above), in elements.
-__device__ __forceinline__ size_t operand_order(int m, int n) { return ((size_t)(n >> 5) * 64 + ((n & 31) >> 3) * 16 + m) * 8 + (n & 7); }
+// Where element (row m, column n) of a matrix of MT row tiles lies in operand order (see XT / OT above), in elements:
+// [N/32 steps][MT row tiles][64 lanes][8].
+__device__ __forceinline__ size_t operand_order(int m, int n, int MT = 1) {
+    return ((((size_t)(n >> 5) * MT + (m >> 4)) * 64 + ((n & 31) >> 3) * 16 + (m & 15)) * 8) + (n & 7);
+}
 
 template <int EPI, bool SCALED, typename TC, int GD_WAVES, bool XT, bool OT>
 __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
@@ -177,6 +180,135 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     }
 }
 
+// The same for 17 to 64 rows: MT row tiles of X per tile of W, one chunk per round (the operands of MT row tiles take
+// the registers that a second chunk would).  X and the outputs in operand order have MT row tiles per step; the parts
+// of sum(h^2) have 16 MT rows each: ss[n][16 MT].
+template <int EPI, bool SCALED, typename TC, int MT, int GD_WAVES, bool XT, bool OT>
+__global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, float* __restrict__ resid_out,
+    bf16_t* __restrict__ xw_out, const bf16_t* __restrict__ w_next, float* __restrict__ ss_out, const float* __restrict__ ss_in,
+    int n_parts, float eps, int M, int N, int K) {
+    constexpr int NT = EPI == EPI_GATED ? 2 : 1;
+    constexpr int MP = 16 * MT;
+    __shared__ float red[(GD_WAVES - 1) * NT * MT * 64 * 4];
+    __shared__ float ss_red[GD_WAVES * 4 * MP];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int n_base = blockIdx.x * 16;
+
+    if (SCALED) {
+        float part[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) part[mt] = 0.f;
+        for (int p = wave * 4 + g; p < n_parts; p += GD_WAVES * 4)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) part[mt] += ss_in[p * MP + 16 * mt + r];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) ss_red[(wave * 4 + g) * MP + 16 * mt + r] = part[mt];
+    }
+
+    f32x4_t acc[NT][MT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const size_t chunk_stride = (size_t)(NT * N / 16) * 4096;
+    const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)blockIdx.x * 4096;
+    unsigned woff[NT], xoff[MT];
+    bool x_ok[MT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) woff[nt] = (unsigned)(nt * N / 16) * 4096u + 16u * lane;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        x_ok[mt] = 16 * mt + r < M;
+        xoff[mt] = XT ? (unsigned)mt * 1024u + 16u * lane : (unsigned)min(16 * mt + r, M - 1) * (unsigned)K * 2u + 16u * g;
+    }
+    const char* xbase = reinterpret_cast<const char*>(X);
+    const int nfull = K / GD_CHUNK;
+#define GDR_LOAD(A, B, CHUNK)                                                                                        \
+    {                                                                                                                \
+        const char* wb = wbase + (size_t)(CHUNK) * chunk_stride;                                                     \
+        const char* xb = xbase + (size_t)(CHUNK) * (XT ? 4 * MT * 1024 : GD_CHUNK * 2);                              \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                              \
+            _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                        \
+                A[nt][j] = *reinterpret_cast<const bf16x8_t*>(wb + woff[nt] + 1024 * j);                             \
+            _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                        \
+                B[mt][j] = x_ok[mt] ? *reinterpret_cast<const bf16x8_t*>(xb + xoff[mt] + (XT ? MT * 1024 : 64) * j)  \
+                                    : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};                                              \
+        }                                                                                                            \
+    }
+#define GDR_MFMA(A, B)                                                                                               \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                                    \
+        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                            \
+            _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                        \
+                acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[nt][j], B[mt][j], acc[nt][mt], 0, 0, 0);
+    for (int c = wave; c < nfull; c += GD_WAVES) {     // (two chunks per round were measured at two row tiles: no gain)
+        bf16x8_t a[NT][4], b[MT][4];
+        GDR_LOAD(a, b, c)
+        GDR_MFMA(a, b)
+    }
+#undef GDR_LOAD
+#undef GDR_MFMA
+    if (wave > 0) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) red[((((wave - 1) * NT + nt) * MT + mt) * 4 + i) * 64 + lane] = acc[nt][mt][i];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 1; w < GD_WAVES; ++w)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[nt][mt][i] += red[((((w - 1) * NT + nt) * MT + mt) * 4 + i) * 64 + lane];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = 16 * mt + r, n = n_base + 4 * g;
+        if (SCALED) {
+            float s = 0.f;
+            for (int i = 0; i < GD_WAVES * 4; ++i) s += ss_red[i * MP + m];
+            const float scale = 1.0f / sqrtf(s / (float)K + eps);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[nt][mt][i] *= scale;
+        }
+        if (EPI == EPI_RESID) {
+            float s = 0.f;
+            if (m < M) {
+                float* hp = resid_out + (size_t)m * N + n;
+                f32x4_t h = *reinterpret_cast<const f32x4_t*>(hp);
+                const uint2 wn = *reinterpret_cast<const uint2*>(w_next + n);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { h[i] += acc[0][mt][i]; s += h[i] * h[i]; }
+                *reinterpret_cast<f32x4_t*>(hp) = h;
+                uint2 o;
+                o.x = pack_bf16x2(h[0] * __uint_as_float(wn.x << 16), h[1] * __uint_as_float(wn.x & 0xffff0000u));
+                o.y = pack_bf16x2(h[2] * __uint_as_float(wn.y << 16), h[3] * __uint_as_float(wn.y & 0xffff0000u));
+                *reinterpret_cast<uint2*>(xw_out + (OT ? operand_order(m, n, MT) : (size_t)m * N + n)) = o;
+            }
+            s += __shfl_xor(s, 16, 64);
+            s += __shfl_xor(s, 32, 64);
+            if (g == 0) ss_out[blockIdx.x * MP + m] = s;      // rows beyond M: 0
+            continue;
+        }
+        if (m >= M) continue;
+        TC* out = C + (OT ? operand_order(m, n, MT) : (size_t)m * N + n);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float v = acc[0][mt][i];
+            if (EPI == EPI_GATED) { const float up = acc[NT - 1][mt][i]; v = (v / (1.0f + expf(-v))) * up; }
+            out[i] = from_f32<TC>(v);
+        }
+    }
+}
+
 struct GdArgs {
     const bf16_t* x; const bf16_t* w; void* c; float* resid; bf16_t* xw_out; const bf16_t* w_next; float* ss_out; const float* ss_in;
     int n_parts; float eps; int M, N, K; bool xt, ot; hipStream_t st;
@@ -187,8 +319,12 @@ struct GdArgs {
 template <int EPI, bool SCALED, typename TC, bool XT, bool OT>
 static void gd_launch2(const GdArgs& a) {
     constexpr int W = EPI == EPI_GATED ? GD_WAVES_GATED : 8;
-    gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(a.x, a.w, (TC*)a.c, a.resid, a.xw_out, a.w_next, a.ss_out,
-                                                                                a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K);
+#define GD_ARGS a.x, a.w, (TC*)a.c, a.resid, a.xw_out, a.w_next, a.ss_out, a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K
+    if (a.M <= 16) gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
+    else if (a.M <= 32) gemm_decode_rows_kernel<EPI, SCALED, TC, 2, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
+    else if (a.M <= 48) gemm_decode_rows_kernel<EPI, SCALED, TC, 3, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
+    else gemm_decode_rows_kernel<EPI, SCALED, TC, 4, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
+#undef GD_ARGS
 }
 
 template <int EPI, bool SCALED, typename TC>
@@ -198,15 +334,15 @@ static void gd_launch(const GdArgs& a) {
     else { if (CAN_OT && a.ot) gd_launch2<EPI, SCALED, TC, false, CAN_OT>(a); else gd_launch2<EPI, SCALED, TC, false, false>(a); }
 }
 
-// x: bfloat16 [M, K].  scaled != 0: x = bf16(h * w_norm) and ss_in [n_parts, 16] holds the parts of sum(h^2); the
-// result is multiplied by rsqrt(sum / K + eps).
+// x: bfloat16 [M, K], M <= 64; MP = M rounded up to a multiple of 16.  scaled != 0: x = bf16(h * w_norm) and ss_in
+// [n_parts, MP] holds the parts of sum(h^2); the result is multiplied by rsqrt(sum / K + eps).
 // epi 0: C [M, N] (c_dtype);  epi 1: W = [gate | up], C [M, N] = silu(gate) * up;  epi 2: resid [M, N] += result,
-// xw_out [M, N] = bf16(resid * w_next), ss_out [N / 16, 16] = every block's part of the rows' sums of squares.
+// xw_out [M, N] = bf16(resid * w_next), ss_out [N / 16, MP] = every block's part of the rows' sums of squares.
 // x_tiled / out_tiled: X / the bfloat16 output for the next product (xw_out of epi 2, C of epi 1) are in operand order.
 extern "C" int spy_gemm_decode(const void* X, int scaled, const float* ss_in, int n_parts, float eps, const void* Wt, int epi,
                                void* C, int c_dtype, float* resid, void* xw_out, const void* w_next, float* ss_out, int M, int N,
                                int K, int x_tiled, int out_tiled, hipStream_t st) {
-    SPY_REQUIRE(M > 0 && M <= 16, "spy_gemm_decode: M = %d rows (1..16 allowed)", M);
+    SPY_REQUIRE(M > 0 && M <= 64, "spy_gemm_decode: M = %d rows (1..64 allowed)", M);
     SPY_REQUIRE(N > 0 && N % 16 == 0 && K > 0 && K % 128 == 0, "spy_gemm_decode: N = %d must be a multiple of 16 and K = %d of 128", N, K);
     SPY_REQUIRE(epi >= 0 && epi <= 2, "spy_gemm_decode: unknown epilogue %d", epi);
     SPY_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)Wt % 16) == 0, "spy_gemm_decode: operands must be 16-byte aligned");

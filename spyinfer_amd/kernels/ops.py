@@ -171,7 +171,10 @@ _LIBRARY_F32_OUT = True      # torch.mm(..., out_dtype=float32) exists in this t
 #: then whole cache lines).  Costs the weights' size again in device memory; the row-major copy stays for the
 #: library product of prefill.
 TILED_WEIGHTS = True
-FUSED_DECODE_MAX_ROWS = 16   # rows of the decode kernel that reads the tiled copies
+#: Most rows of a step whose products run with norms and residual sums folded in, handing their outputs over in operand
+#: order (above: the library product with norm kernels of their own).  Measured on MI355X at the Qwen3-8B shapes: such
+#: products beat the library's by 16 % at 32 rows and lose to it from about 56.
+FUSED_DECODE_MAX_ROWS = 48
 
 
 def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
@@ -205,7 +208,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     if M == 0:
         return torch.empty((0, N), dtype=out_dtype, device=x.device)
     all_bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-    if all_bf16 and tiled is not None and M <= FUSED_DECODE_MAX_ROWS:
+    if all_bf16 and tiled is not None and M <= SKINNY_MAX_ROWS:
         _check(tiled.shape == w.shape, "linear: the tiled copy does not fit the matrix")
         return decode_linear(x, tiled, out_dtype)
     global _LIBRARY_F32_OUT
@@ -237,7 +240,7 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, tiled: Optional[torc
            "linear_swiglu: x [M, K] and w [2 I, K] expected")
     M, K = x.shape
     I = w_gate_up.shape[0] // 2
-    if x.dtype == torch.bfloat16 and tiled is not None and 0 < M <= FUSED_DECODE_MAX_ROWS and I % 16 == 0:
+    if x.dtype == torch.bfloat16 and tiled is not None and 0 < M <= SKINNY_MAX_ROWS and I % 16 == 0:
         _check(tiled.shape == w_gate_up.shape, "linear_swiglu: the tiled copy does not fit")
         return decode_linear_swiglu(x, tiled)
     if x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 \
@@ -252,28 +255,35 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, tiled: Optional[torc
 # --------------------------------------------------------------------------
 # Decode-time products with the norm and the residual sum folded in
 class OperandRows:
-    """At most 16 rows of bfloat16 [M, K] in the order the MFMA operand wants them: ``data`` is [K/32 steps, 64 lanes,
-    8] with lane 16 g + r of step s holding x[r][32 s + 8 g ..]; rows M..15 hold anything.  The decode products write
-    their outputs for each other this way (an operand is then one load of 1 KiB in one piece)."""
+    """Rows of bfloat16 [M, K], M <= 64, in the order the MFMA operand wants them: ``data`` is [K/32 steps, MT row
+    tiles, 64 lanes, 8] with lane 16 g + r of row tile t and step s holding x[16 t + r][32 s + 8 g ..]; MT = ceil(M / 16);
+    rows M.. of the last tile hold anything.  The decode products write their outputs for each other this way (an
+    operand is then one load of 1 KiB in one piece)."""
     __slots__ = ("data", "rows", "width")
 
     def __init__(self, data: torch.Tensor, rows: int, width: int):
         self.data, self.rows, self.width = data, rows, width
 
+    @property
+    def tiles(self) -> int:
+        return -(-self.rows // 16)
+
     @staticmethod
     def empty(rows: int, width: int, device) -> "OperandRows":
-        _check(0 < rows <= 16 and width % 32 == 0, "operand order takes 1..16 rows of a width that is a multiple of 32")
-        return OperandRows(torch.empty((width // 32, 64, 8), dtype=torch.bfloat16, device=device), rows, width)
+        _check(0 < rows <= FUSED_DECODE_MAX_ROWS and width % 32 == 0,
+               "operand order takes 1..%d rows of a width that is a multiple of 32" % FUSED_DECODE_MAX_ROWS)
+        return OperandRows(torch.empty((width // 32, -(-rows // 16), 64, 8), dtype=torch.bfloat16, device=device), rows, width)
 
     def to_rows(self) -> torch.Tensor:
         """The same values as an ordinary [M, K] tensor (for tests; not used by the engine)."""
-        return self.data.view(self.width // 32, 4, 16, 8).permute(2, 0, 1, 3).reshape(16, self.width)[:self.rows].contiguous()
+        mt = self.tiles
+        return self.data.view(self.width // 32, mt, 4, 16, 8).permute(1, 3, 0, 2, 4).reshape(16 * mt, self.width)[:self.rows].contiguous()
 
 
 class ScaledInput:
     """The input of a product as 'the RMS norm of the residual stream' with the scale still to come:
-    ``xw`` = bfloat16(h * w_norm), as [M, K] or as OperandRows, and the parts ``ss_parts [n, 16]`` of every row's sum
-    of squares (row r of the stream in column r; their sum over n is sum(h[r]^2)).  ``decode_linear`` and
+    ``xw`` = bfloat16(h * w_norm), as [M, K] or as OperandRows, and the parts ``ss_parts [n, MP]`` of every row's sum
+    of squares (row r of the stream in column r; their sum over n is sum(h[r]^2); MP = M rounded up to 16).  ``decode_linear`` and
     ``decode_linear_swiglu`` multiply their result by rsqrt(sum / K + eps), which equals the product with the
     normed rows.  ``norm`` is the norm part this was prepared for."""
     __slots__ = ("xw", "ss_parts", "eps", "norm")
@@ -290,7 +300,7 @@ OPERAND_ORDER = True
 
 def fused_decode_ok(rows: int, act_dtype, *tiled_weights) -> bool:
     """True if products of ``rows`` rows with these tiled matrices can run with the norm's scale and the residual
-    sum folded in: bfloat16 activations, at most 16 rows, tiled bfloat16 weights."""
+    sum folded in: bfloat16 activations, few rows, tiled bfloat16 weights."""
     if not FUSED_DECODE or _impl is not None or act_dtype != torch.bfloat16 or not 0 < rows <= FUSED_DECODE_MAX_ROWS:
         return False
     return all(t is not None and t.dtype == torch.bfloat16 and t.shape[0] % 16 == 0 and t.shape[1] % 128 == 0
@@ -302,22 +312,25 @@ def _gemm_decode(x, tiled: torch.Tensor, epi: int, n_out: int, out, resid, xw_ou
     K = tiled.shape[1]
     if isinstance(x, ScaledInput):
         xs, ss, eps = x.xw, x.ss_parts, x.eps
-        _check(ss.dtype == torch.float32 and ss.dim() == 2 and ss.shape[1] == 16 and ss.shape[0] > 0,
-               "decode product: the parts of the sums of squares must be float32 [n, 16]")
+        _check(ss.dtype == torch.float32 and ss.dim() == 2 and ss.shape[0] > 0,
+               "decode product: the parts of the sums of squares must be float32 [n, rows rounded up to 16]")
     else:
         xs, ss, eps = x, None, 0.0
     x_tiled = isinstance(xs, OperandRows)
     if x_tiled:
-        _check(xs.width == K and tuple(xs.data.shape) == (K // 32, 64, 8) and xs.data.dtype == torch.bfloat16,
-               "decode product: x in operand order must be bfloat16 [%d / 32, 64, 8]" % K)
+        _check(xs.width == K and tuple(xs.data.shape) == (K // 32, xs.tiles, 64, 8) and xs.data.dtype == torch.bfloat16,
+               "decode product: x in operand order must be bfloat16 [%d / 32, row tiles, 64, 8]" % K)
         M, xs = xs.rows, xs.data
     else:
         _check(xs.dtype == torch.bfloat16 and xs.dim() == 2 and xs.shape[1] == K, "decode product: x must be bfloat16 [M, %d]" % K)
         M = xs.shape[0]
     out_tiled = isinstance(out, OperandRows) or isinstance(xw_out, OperandRows)
+    mp = -(-M // 16) * 16
+    _check(ss is None or ss.shape[1] == mp, "decode product: the parts of the sums of squares must have %d columns" % mp)
+    _check(ss_out is None or tuple(ss_out.shape) == (n_out // 16, mp), "decode product: the new parts must be [N / 16, %d]" % mp)
     for o in (out, xw_out):
         if isinstance(o, OperandRows):
-            _check(o.rows == M and o.width == n_out and tuple(o.data.shape) == (n_out // 32, 64, 8),
+            _check(o.rows == M and o.width == n_out and tuple(o.data.shape) == (n_out // 32, o.tiles, 64, 8),
                    "decode product: the output in operand order does not fit")
     out_t = out.data if isinstance(out, OperandRows) else out
     xw_t = xw_out.data if isinstance(xw_out, OperandRows) else xw_out
@@ -369,7 +382,7 @@ def decode_linear_residual(x, tiled: torch.Tensor, resid: torch.Tensor, next_nor
            "decode_linear_residual: the stream must be float32 [M, %d]" % N)
     _check(next_norm_weight.dtype == torch.bfloat16 and next_norm_weight.shape == (N,),
            "decode_linear_residual: the next norm's weight must be bfloat16 [%d]" % N)
-    ss = torch.empty((N // 16, 16), dtype=torch.float32, device=resid.device)
+    ss = torch.empty((N // 16, -(-M // 16) * 16), dtype=torch.float32, device=resid.device)
     if _operand_order_ok(N):
         xw = OperandRows.empty(M, N, resid.device)
     else:
@@ -379,16 +392,17 @@ def decode_linear_residual(x, tiled: torch.Tensor, resid: torch.Tensor, next_nor
 
 
 def embedding_scaled(ids: torch.Tensor, table: torch.Tensor, norm_weight: torch.Tensor, eps: float, norm=None):
-    """embedding() for at most 16 tokens -> (stream, ScaledInput of the first norm)."""
+    """embedding() for few tokens -> (stream, ScaledInput of the first norm)."""
     _dev(ids, table, norm_weight)
-    _check(ids.dtype == torch.int32 and ids.dim() == 1 and 0 < ids.shape[0] <= 16, "embedding_scaled: ids must be int32 [1..16]")
+    _check(ids.dtype == torch.int32 and ids.dim() == 1 and 0 < ids.shape[0] <= FUSED_DECODE_MAX_ROWS,
+           "embedding_scaled: ids must be int32 [1..%d]" % FUSED_DECODE_MAX_ROWS)
     _check(table.dim() == 2, "embedding: table must be [V, H]")
     T, (V, H) = ids.shape[0], table.shape
     _check(norm_weight.dtype == torch.bfloat16 and norm_weight.shape == (H,), "embedding_scaled: the norm weight must be bfloat16 [H]")
     out = torch.empty((T, H), dtype=torch.float32, device=table.device)
     tiled = _operand_order_ok(H)
     xw = OperandRows.empty(T, H, table.device) if tiled else torch.empty((T, H), dtype=torch.bfloat16, device=table.device)
-    ss = torch.empty((1, 16), dtype=torch.float32, device=table.device)
+    ss = torch.empty((1, -(-T // 16) * 16), dtype=torch.float32, device=table.device)
     hip().call("spy_embedding_sumsq", _ptr(out), _ptr(xw.data if tiled else xw), _ptr(ss), _ptr(table), _code(table, "embedding table"),
                _ptr(norm_weight), _ptr(ids), ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(V), ctypes.c_int(1 if tiled else 0),
                _Hip.stream())

@@ -48,7 +48,8 @@ class LMHead(Part):
         self.weight_tiled = ops.tile_weight(self.weight)
 
     def can_fold(self, batch):
-        return ops.fused_decode_ok(batch.T, batch.act_dtype, self.weight_tiled)
+        # above 16 rows the library's product (after a norm kernel) is faster for a matrix of this size
+        return batch.T <= ops.SKINNY_MAX_ROWS and ops.fused_decode_ok(batch.T, batch.act_dtype, self.weight_tiled)
 
     def forward(self, normed):
         if isinstance(normed, ops.ScaledInput):
