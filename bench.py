@@ -6,7 +6,7 @@ Default: the Qwen3-8B shape of BASELINE.json configs[2] (36 layers, hidden 4096,
 bfloat16 weights; 8 requests with 1024-token random prompts decode through the engine's own step
 (scheduler, step function, cache, kernels, device sampling).  A "step" is one decode step.
 Prints ONE JSON line: decoded tokens per second, plus the prefill of 2048 tokens, the decode
-step's HBM roofline, and decode at batch 1 and 64.
+step's HBM roofline, and decode at batch 1, 32 and 64.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--dtype bfloat16|float32]
 """
@@ -35,7 +35,7 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096, help="max_model_len")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--points", default="1,64", help="further decode batch sizes to report (empty: none)")
+    ap.add_argument("--points", default="1,32,64", help="further decode batch sizes to report (empty: none)")
     ap.add_argument("--enforce-eager", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
