@@ -115,7 +115,7 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, bf16_t* kc, bf16_t* vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
-    int n_q, int n_kv, int d, float scale, int window, int splits, float* __restrict__ ws, FusedQKV fz) {
+    int n_q, int n_kv, int d, float scale, int window, int splits, float* __restrict__ ws, FusedQKV fz, int out_tiles) {
     constexpr int KK = DMAX / 32;   // 32-wide chunks of the head dim for Q.K
     constexpr int DT = DMAX / 16;   // 16-row tiles of the head dim for P.V
     extern __shared__ float lds[];   // (AW - 1) * (DT * 4 + 2) * 64 floats: the other waves' O, m, l
@@ -378,7 +378,9 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
                 uint2 w;
                 w.x = pack_bf16x2(acc[dt][0] * inv, acc[dt][1] * inv);
                 w.y = pack_bf16x2(acc[dt][2] * inv, acc[dt][3] * inv);
-                *reinterpret_cast<uint2*>(op + dd) = w;
+                // (four columns from a multiple of 4 never cross a group of 8: one store either way)
+                if (out_tiles) *reinterpret_cast<uint2*>(out + attention_out_operand_order(q0 + tq, head * d + dd, out_tiles)) = w;
+                else *reinterpret_cast<uint2*>(op + dd) = w;
             }
         }
         return;
@@ -403,6 +405,8 @@ extern "C" int64_t spy_attention_mfma_workspace(int num_tiles, int n_kv, int d, 
     return (int64_t)num_tiles * n_kv * splits * 16 * (dmax_of(d) + 2);
 }
 
+// out_tiles > 0: the output [T, n_q d] goes out in MFMA operand order for that many row tiles (attention_merge.h), for a
+// decode product that reads it next.
 // qkv != null: the fused variant (see the top of the file).  Then q is not read, every entry must be a single token
 // (T == S), head_dim 64, 128 or 256 with the whole head rotated (or no rotation: cos_t == null), and the new keys and
 // values are written to kc and vc by this call (store != 0).
@@ -410,7 +414,8 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
                                   const int* pos0, const int* kv_len, const int* block_table, int max_blocks, const int* tile_entry,
                                   const int* tile_row0, int num_tiles, int S, int T, int n_q, int n_kv, int d, float scale,
                                   int window, int splits, float* ws, const void* qkv, const void* qw, const void* kw, int w_dtype,
-                                  float eps, const float* cos_t, const float* sin_t, int max_pos, int store, hipStream_t st) {
+                                  float eps, const float* cos_t, const float* sin_t, int max_pos, int store, int out_tiles,
+                                  hipStream_t st) {
     SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
                 "spy_attention_mfma: empty operand");
     SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 256, "spy_attention_mfma: head_dim %d is not a multiple of 16 in 16..256", d);
@@ -419,6 +424,8 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
     SPY_REQUIRE(splits >= 1 && splits <= 64, "spy_attention_mfma: %d parts (1..64 allowed)", splits);
     SPY_REQUIRE(splits == 1 || ws, "spy_attention_mfma: parts without a workspace");
     SPY_REQUIRE(n_kv <= 65535, "spy_attention_mfma: too many kv heads");
+    SPY_REQUIRE(out_tiles >= 0 && out_tiles <= 4 && (!out_tiles || (T <= 16 * out_tiles && (n_q * d) % 32 == 0 && d % 8 == 0)),
+                "spy_attention_mfma: operand order is for at most 64 rows (%d here) of a width that is a multiple of 32", T);
     FusedQKV fz = {(const bf16_t*)qkv, qw, kw, w_dtype, eps, cos_t, sin_t, max_pos, store};
     if (qkv) {
         SPY_REQUIRE(T == S && num_tiles == S, "spy_attention_mfma: the fused variant takes single tokens only (%d tokens of %d entries)", T, S);
@@ -435,11 +442,11 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
 #define ATT_LAUNCH(DM, FZ)                                                                                                    \
     attention_mfma_kernel<DM, FZ><<<grid, AW * 64, (AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>(                \
         (bf16_t*)out, (const bf16_t*)q, (bf16_t*)kc, (bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,  \
-        tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz)
+        tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz, out_tiles)
 #define ATT_CASE(DM)                                                                                                          \
     if (qkv) ATT_LAUNCH(DM, true); else ATT_LAUNCH(DM, false);                                                                \
     if (splits > 1)                                                                                                           \
-        attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits, 1);
+        attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits, 1, out_tiles);
     switch (dmax_of(d)) {
         case 64: ATT_CASE(64) break;
         case 128: ATT_CASE(128) break;

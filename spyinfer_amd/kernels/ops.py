@@ -533,10 +533,13 @@ def fused_attention_ok(dtype, meta: AttentionMeta, n_q: int, n_kv: int, d: int, 
 
 
 def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: torch.Tensor, page_size: int, meta: AttentionMeta,
-                    n_q: int, n_kv: int, d: int, scale: float, window: Optional[int], raw: Optional[RawQKV] = None) -> torch.Tensor:
+                    n_q: int, n_kv: int, d: int, scale: float, window: Optional[int], raw: Optional[RawQKV] = None,
+                    for_product: bool = False):
     """Causal grouped-query attention of the step's query tokens over the paged cache
     (which already holds this step's keys and values, or gets them from ``raw`` in this call).  Query at position p
-    reads keys max(0, p - window + 1) .. p.  Scores, softmax and the weighted sum are float32."""
+    reads keys max(0, p - window + 1) .. p.  Scores, softmax and the weighted sum are float32.
+    ``for_product``: the result goes into a decode product only and may come as OperandRows (it does when all of the
+    step runs through the 16-row-tile kernel and has few rows)."""
     if _impl is not None:
         return _impl.paged_attention(q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window)
     T, S = meta.T, meta.S
@@ -572,6 +575,11 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
     if T == 0:
         return out
     group = n_q // n_kv
+    operand = None
+    if for_product and _operand_order_ok(n_q * d) and T <= FUSED_DECODE_MAX_ROWS and d % 8 == 0 and meta.tiles is not None \
+            and meta.tiles_group == group and meta.tiles["big"][2] == 0 and mfma_attention_ok(q.dtype, d, page_size):
+        operand = OperandRows.empty(T, n_q * d, q.device)
+        out = operand.data
     if mfma_attention_ok(q.dtype, d, page_size) and meta.tiles is not None and meta.tiles_group == group:
         small_entry, small_row0, n_small = meta.tiles["small"]
         big_entry, big_row0, n_big = meta.tiles["big"]
@@ -613,8 +621,8 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
                          ctypes.c_int(0), ctypes.c_int(0))
             hip().call("spy_attention_mfma", _ptr(out), _ptr(None if raw is not None else q), _ptr(k_cache), _ptr(v_cache), *common,
                        _ptr(small_entry), _ptr(small_row0), ctypes.c_int(n_small), *sizes, ctypes.c_int(splits), _ptr(ws), *fused,
-                       _Hip.stream())
-        return out
+                       ctypes.c_int(operand.tiles if operand is not None else 0), _Hip.stream())
+        return operand if operand is not None else out
     hip().call("spy_attention_generic", _ptr(out), _ptr(q), _code(q, "q"), _ptr(k_cache), _ptr(v_cache),
                ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(meta.kv_len), _ptr(meta.block_table),
                ctypes.c_int(meta.max_blocks), _ptr(meta.token_entry), _ptr(meta.positions), ctypes.c_int(S), ctypes.c_int(T),

@@ -68,7 +68,7 @@ class PagedAttention(Mixer):
     def can_fold(self, batch):
         return ops.fused_decode_ok(batch.T, batch.act_dtype, self.w_qkv_tiled, self.w_o_tiled)
 
-    def _attend(self, x, batch, cache, store):
+    def _attend(self, x, batch, cache, store, for_product=False):
         nq, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
         if isinstance(x, ops.ScaledInput):
             qkv = ops.decode_linear(x, self.w_qkv_tiled)
@@ -81,15 +81,18 @@ class PagedAttention(Mixer):
         if ops.fused_attention_ok(qkv.dtype, meta, nq, nkv, d, cache.page_size, rdim, self.q_norm, self.k_norm):
             # single tokens only: the attention kernel norms, rotates and stores by itself
             raw = ops.RawQKV(qkv, self.q_norm, self.k_norm, eps, cos if rdim else None, sin if rdim else None, store)
-            return ops.paged_attention(None, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window, raw)
+            return ops.paged_attention(None, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window, raw,
+                                       for_product=for_product)
         slots = batch.slot_mapping(cache.group) if store else None
         q = ops.qk_norm_rope_store(qkv, nq, nkv, d, self.q_norm, self.k_norm, eps,
                                    cos, sin, rdim, batch.positions, cache.k, cache.v, cache.page_size, slots)
-        return ops.paged_attention(q, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window)
+        return ops.paged_attention(q, cache.k, cache.v, cache.page_size, meta, nq, nkv, d, self.scale, self.window,
+                                   for_product=for_product)
 
     def forward(self, x, batch, cache, store=True):
         return ops.linear(self._attend(x, batch, cache, store), self.w_o, tiled=self.w_o_tiled)
 
     def forward_into(self, x, batch, cache, store, resid, next_norm):
         weight, eps = next_norm.foldable(batch.act_dtype)
-        return ops.decode_linear_residual(self._attend(x, batch, cache, store), self.w_o_tiled, resid, weight, eps, next_norm)
+        return ops.decode_linear_residual(self._attend(x, batch, cache, store, for_product=True), self.w_o_tiled, resid, weight, eps,
+                                          next_norm)

@@ -492,12 +492,34 @@ def test_attention_taking_the_raw_product(case, wdtype, keys_per_part, monkeypat
         new[bt[s][a // P], :, a % P] = True
     assert same(kc_dev[~new.to(dev)], kc_ref[~new]), "keys of other positions must stay as they were"
     close(kc_dev[new.to(dev)], kc_ref[new], dtype, scale=8.0, what="stored keys")
+    # the same result in operand order, for the product that reads it next
+    if T <= ops.FUSED_DECODE_MAX_ROWS:
+        kc3, vc3 = kc_ref.to(dev), vc_ref.to(dev)
+        o3 = ops.paged_attention(None, kc3, vc3, P, meta, n_q, n_kv, d, scale, window, raw, for_product=True)
+        assert isinstance(o3, ops.OperandRows) and torch.equal(o3.to_rows(), out)
     # store = False: nothing is written and the new position is not read (the cache of another call)
     kc2, vc2 = kc_ref.to(dev), vc_ref.to(dev)
     raw.store = False
     out2 = ops.paged_attention(None, kc2, vc2, P, meta, n_q, n_kv, d, scale, window, raw)
     close(out2, ref, dtype, scale=3.0, what="fused attention without store, case %d" % case)
     assert same(kc2, kc_ref) and same(vc2, vc_ref)
+
+
+@pytest.mark.parametrize("case", [1, 3, 8, 9])
+def test_attention_output_in_operand_order(case):
+    """Steps of few rows without 128-row tiles can hand the attention's output over in MFMA operand order: the values
+    are those of the ordinary output, element for element (portions and single tokens, one and several key parts)."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    n_q, n_kv, d, P, entries, window = ATT_CASES[case]
+    q, kc, vc, bt, te, ps, meta = make_attention_case(torch.bfloat16, dev, n_q, n_kv, d, P, entries, seed=case, window=window)
+    scale = 1.0 / math.sqrt(d)
+    rows = ops.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), P, meta, n_q, n_kv, d, scale, window)
+    got = ops.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), P, meta, n_q, n_kv, d, scale, window, for_product=True)
+    if meta.tiles["big"][2] == 0 and meta.T <= ops.FUSED_DECODE_MAX_ROWS and (n_q * d) % 32 == 0:
+        assert isinstance(got, ops.OperandRows) and got.rows == meta.T and torch.equal(got.to_rows(), rows)
+    else:
+        assert torch.equal(got, rows)
 
 
 def test_attention_without_rotation_is_library_sdpa():
