@@ -79,6 +79,52 @@ def test_requests_ending_while_a_step_is_in_flight(folder_a, eager):
     assert eng.runner.manager.num_free_pages() == [11]
 
 
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_arrivals_endings_and_removals(folder_a, seed):
+    """A random serving day in float32 with graphs: requests arrive while others decode, end at an end token, by count
+    or by removal, the pool is small enough for preemption.  Every request's tokens are the plain implementation's."""
+    import random
+    from collections import Counter
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    require_gpu()
+    rng = random.Random(seed)
+    lengths = [rng.randint(1, 50) for _ in range(18)]
+    ps = prompts(256, lengths, 20 + seed)
+    plain = PlainQwen3(folder_a)
+    news = [rng.randint(1, 16) for _ in ps]
+    full = [plain.greedy(p, n) for p, n in zip(ps, news)]
+    eos = Counter(t for g in full for t in g[1:]).most_common(1)[0][0]
+    use_eos = [rng.random() < 0.6 for _ in ps]
+    want = [g[:g.index(eos) + 1] if (u and eos in g) else g for g, u in zip(full, use_eos)]
+    eng = LLMEngine(folder_a, dtype="float32", max_model_len=128, num_kvcache_blocks=13, max_num_seqs=4,
+                    max_num_batched_tokens=48)
+    eng.eos_token_id = eos
+    arrival = sorted((rng.randint(0, 60), i) for i in range(len(ps)))
+    removed_at = {i: rng.randint(2, 8) for i in rng.sample(range(len(ps)), 3)}     # steps after arrival
+    ids, born, gone, step = {}, {}, {}, 0
+    while arrival or eng.has_unfinished_requests():
+        while arrival and arrival[0][0] <= step:
+            _, i = arrival.pop(0)
+            ids[i] = eng.add_request(ps[i], SamplingParams(max_new_tokens=news[i], ignore_eos=not use_eos[i]))
+            born[i] = step
+        for i, after in removed_at.items():
+            if i in ids and i not in gone and step == born[i] + after:
+                gone[i] = eng.get_generated_tokens(ids[i])
+                eng.remove_request(ids[i])
+        eng.step()
+        step += 1
+        assert step < 2000
+    for i in range(len(ps)):
+        if i in gone:
+            assert gone[i] == want[i][:len(gone[i])], "request %d, removed early, had other tokens" % i
+        else:
+            assert eng.get_generated_tokens(ids[i]) == want[i], "request %d" % i
+    eng.runner.manager.check()
+    assert eng.runner.manager.num_free_pages() == [13]
+    assert eng.runner.graph_replays > 0
+
+
 def test_greedy_bfloat16_follows_plain(folder_a):
     """bfloat16 may leave the plain tokens only where the plain logits nearly tie."""
     from spyinfer_amd.engine.llm_engine import LLMEngine
