@@ -66,7 +66,11 @@ class ModelRunner:
         self.use_graphs = (not enforce_eager) and self.device.type == "cuda"
         limit = max_model_len or model.max_positions or num_pages * page_size
         self.fixed_max_blocks = min(-(-limit // page_size), max(1, num_pages))
+        #: captured steps by shape.  Each holds its step's activations and logits, so at most ``max_graphs`` are
+        #: captured; further shapes run kernel by kernel.  A captured step is kept as long as the runner: none
+        #: is destroyed between steps, while others may be in flight.
         self._graphs = {}
+        self.max_graphs = 256
         self._seen = {}
         self._pinned = None
         self._copied = None
@@ -169,8 +173,9 @@ class ModelRunner:
             graph.replay()
             self.graph_replays += 1
             return logits
-        if self._seen.get(key, 0) < 1:
-            # first step of this shape: run it kernel by kernel (this also warms the library up)
+        if self._seen.get(key, 0) < 1 or len(self._graphs) >= self.max_graphs:
+            # first step of this shape: run it kernel by kernel (this also warms the library up); so do shapes
+            # beyond the number of graphs that are kept
             self._seen[key] = 1
             self._upload(batch, None)
             if token_source is not None:

@@ -125,6 +125,26 @@ def test_random_arrivals_endings_and_removals(folder_a, seed):
     assert eng.runner.graph_replays > 0
 
 
+def test_number_of_graphs_is_bounded(folder_a):
+    """The runner captures a bounded number of step shapes (each captured step holds its activations); with room for
+    two, a run whose batch shrinks from four requests to one runs its later shapes kernel by kernel and still gives
+    the plain implementation's tokens."""
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    require_gpu()
+    ps = prompts(256, [5, 17, 33, 9], 12)
+    plain = PlainQwen3(folder_a)
+    news = [30, 22, 14, 6]
+    eng = LLMEngine(folder_a, dtype="float32", max_model_len=128, num_kvcache_blocks=40, max_num_seqs=4)
+    eng.runner.max_graphs = 2
+    ids = [eng.add_request(p, SamplingParams(max_new_tokens=n, ignore_eos=True)) for p, n in zip(ps, news)]
+    while eng.has_unfinished_requests():
+        eng.step()
+    assert len(eng.runner._graphs) == 2
+    assert [eng.get_generated_tokens(i) for i in ids] == [plain.greedy(p, n) for p, n in zip(ps, news)]
+    assert 5 < eng.runner.graph_replays < eng.runner.steps_run
+
+
 def test_greedy_bfloat16_follows_plain(folder_a):
     """bfloat16 may leave the plain tokens only where the plain logits nearly tie."""
     from spyinfer_amd.engine.llm_engine import LLMEngine
