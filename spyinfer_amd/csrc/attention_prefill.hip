@@ -173,6 +173,9 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, RT == 1 ? 1 : 2) void attention_p
 
     const int per_part = (nblk + splits - 1) / splits;
     const int b_first = part * per_part, b_last = min(nblk, b_first + per_part);
+    // The query rows are waited for here, once.  Left pending into the loop, they make the compiler wait for every
+    // outstanding load (vmcnt(0)) ahead of each round's first product, the round's own prefetch included.
+    __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0); the other counters stay as they are
     if (b_first < b_last) {
         PF_PAGES(lo + PF_KEYS * b_first)
         PF_PREFETCH(lo + PF_KEYS * b_first)
