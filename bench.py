@@ -9,6 +9,11 @@ Prints ONE JSON line: decoded tokens per second, plus the prefill of 2048 tokens
 step's HBM roofline, and decode at batch 1, 32 and 64.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--dtype bfloat16|float32]
+
+Other workloads of BASELINE.json, each again one JSON line:
+
+    python bench.py --shape 14b --serve 64                 # configs[3]: 64 requests at once until all have ended
+    python bench.py --shape 32b --batch 64 --prompt-len 4096 --context 4608 --points "" --steps 32 --warmup 4   # configs[4]
 """
 import argparse
 import json
@@ -22,6 +27,12 @@ MODEL_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_a
                 num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936,
                 rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960,
                 bos_token_id=151643, eos_token_id=151645)
+# the larger shapes of BASELINE.json (configs[3] and configs[4]); the default stays the 8B shape
+SHAPES = {
+    "8b": ("Qwen3-8B shape", MODEL_8B),
+    "14b": ("Qwen3-14B shape", dict(MODEL_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)),
+    "32b": ("Qwen3-32B shape", dict(MODEL_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)),
+}
 
 
 def main() -> int:
@@ -38,6 +49,10 @@ def main() -> int:
     ap.add_argument("--points", default="1,32,64", help="further decode batch sizes to report (empty: none)")
     ap.add_argument("--enforce-eager", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes: BASELINE.json configs[2] (8b), [3] (14b), [4] (32b)")
+    ap.add_argument("--serve", type=int, default=0, metavar="N",
+                    help="instead of the decode steps: N requests arriving at once, prompts of 128..2048 and outputs of 64..512 "
+                         "tokens (uniform), run until all have ended; the value is generated tokens per second of the whole run")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
@@ -55,7 +70,8 @@ def main() -> int:
 
     ops.hip()
     dev = torch.device("cuda:0")
-    raw = dict(MODEL_8B)
+    shape_name, shape = SHAPES[args.shape]
+    raw = dict(shape)
     model_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
@@ -69,7 +85,7 @@ def main() -> int:
     torch.cuda.empty_cache()
 
     points = [int(x) for x in args.points.split(",") if x.strip()]
-    max_batch = max([args.batch] + points)
+    max_batch = max([args.batch, args.serve] + points)
     page = 16
     pages_per_req = -(-args.context // page)
     eng = LLMEngine.__new__(LLMEngine)
@@ -125,6 +141,38 @@ def main() -> int:
             best = dt if best is None else min(best, dt)       # the first run also warms the library up
         return best
 
+    def serve_run(n):
+        """n requests at once through the scheduler until all have ended: (generated tokens/s, seconds, steps, mean number
+        of requests in a step, preemptions, prompt tokens, generated tokens)."""
+        lens = torch.randint(128, 2049, (n,), generator=g).tolist()
+        outs = torch.randint(64, 513, (n,), generator=g).tolist()
+        for length, new in zip(lens, outs):
+            eng.add_request(prompts(1, length)[0], SamplingParams(temperature=0.0, max_new_tokens=new, ignore_eos=True))
+        steps = rows = 0
+        before = eng.scheduler.num_preemptions
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while eng.has_unfinished_requests():
+            rows += len(eng.step())
+            steps += 1
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        return sum(outs) / dt, dt, steps, rows / max(1, steps), eng.scheduler.num_preemptions - before, sum(lens), sum(outs)
+
+    if args.serve:
+        serve_run(min(args.serve, 4))                                        # warms the library and the graphs up
+        v, dt, steps, mean_rows, pre, n_prompt, n_out = serve_run(args.serve)
+        print(json.dumps({
+            "metric": "generated tok/s, %d requests at once (%s, prompts 128..2048, outputs 64..512)" % (args.serve, shape_name),
+            "value": round(v, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": 0, "ms_per_step": round(dt / steps * 1e3, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic (random weights, uniform-random token ids and lengths)",
+            "config": {"model": shape_name, "layers": cfg.num_hidden_layers, "layers_of_model": model_layers, "hidden": cfg.hidden_size,
+                       "q_heads": nq, "kv_heads": nkv, "head_dim": d, "intermediate": I, "vocab": V, "global_batch": args.serve,
+                       "seq_len": args.context, "prompt_tokens": n_prompt, "generated_tokens": n_out, "seconds": round(dt, 3),
+                       "mean_rows_per_step": round(mean_rows, 2), "preemptions": pre, "page_size": page, "parallelism": "single GPU"}}))
+        return 0
+
     value, ms, ctx = decode_run(args.batch, args.steps, args.warmup)
     step_bytes = weight_bytes + args.batch * ctx * kv_bytes_per_token
     achieved = step_bytes / (ms * 1e-3) / 1e9
@@ -138,11 +186,11 @@ def main() -> int:
         v, _, _ = decode_run(b, max(8, args.steps // 2), max(4, args.warmup // 2))
         extra["decode_b%d" % b] = round(v, 1)
     line = {
-        "metric": "decode tok/s at batch %d (Qwen3-8B shape, %d-token prompts)" % (args.batch, args.prompt_len),
+        "metric": "decode tok/s at batch %d (%s, %d-token prompts)" % (args.batch, shape_name, args.prompt_len),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, uniform-random token ids)",
-        "config": {"model": "Qwen3-8B shape", "layers": L, "layers_of_model": model_layers, "hidden": H, "q_heads": nq,
+        "config": {"model": shape_name, "layers": L, "layers_of_model": model_layers, "hidden": H, "q_heads": nq,
                    "kv_heads": nkv, "head_dim": d, "intermediate": I, "vocab": V, "global_batch": args.batch,
                    "seq_len": args.context, "prompt_len": args.prompt_len, "mean_context": round(ctx, 1), "page_size": page,
                    "graphs": not args.enforce_eager, "run_ahead": bool(eng.run_ahead), "parallelism": "single GPU"},

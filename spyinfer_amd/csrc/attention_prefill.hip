@@ -270,12 +270,29 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, RT == 1 ? 1 : 2) void attention_p
                     for (int dt = 0; dt < DT; ++dt) acc[t][dt] *= alpha[t];
                 }
             }
+            if (DFULL) {
+                // the value fragments are read two products ahead of their use; the scheduling barriers keep the compiler
+                // from moving every read down to its product (it did, to save registers: 8 LDS round trips in a row)
+                const bf16_t* vrow = vs + r16 * VLD + 32 * half + 8 * g;
+                bf16x8_t vt[3];
+                vt[0] = *reinterpret_cast<const bf16x8_t*>(vrow);
+                vt[1] = *reinterpret_cast<const bf16x8_t*>(vrow + 16 * VLD);
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                if (DFULL || dt * 16 < d) {
-                    const bf16x8_t vt = *reinterpret_cast<const bf16x8_t*>(vs + (dt * 16 + r16) * VLD + 32 * half + 8 * g);
+                for (int dt = 0; dt < DT; ++dt) {
+                    if (dt + 2 < DT) vt[(dt + 2) % 3] = *reinterpret_cast<const bf16x8_t*>(vrow + (dt + 2) * 16 * VLD);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int t = 0; t < RT; ++t) acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pb[t], acc[t][dt], 0, 0, 0);
+                    for (int t = 0; t < RT; ++t) acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt % 3], pb[t], acc[t][dt], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    if (dt * 16 < d) {
+                        const bf16x8_t vt = *reinterpret_cast<const bf16x8_t*>(vs + (dt * 16 + r16) * VLD + 32 * half + 8 * g);
+#pragma unroll
+                        for (int t = 0; t < RT; ++t) acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pb[t], acc[t][dt], 0, 0, 0);
+                    }
                 }
             }
         }
