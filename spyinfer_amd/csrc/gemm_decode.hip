@@ -183,18 +183,19 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
 // The same for 17 to 64 rows: MT row tiles of X per tile of W, one chunk per round (the operands of MT row tiles take
 // the registers that a second chunk would).  X and the outputs in operand order have MT row tiles per step; the parts
 // of sum(h^2) have 16 MT rows each: ss[n][16 MT].
-template <int EPI, bool SCALED, typename TC, int MT, int GD_WAVES, bool XT, bool OT>
+// CT: column tiles of 16 per block.  Every block reads all of X, from L2, and with MT row tiles that is MT times the
+// bytes of its W tile: with two column tiles the X fragments in registers serve both, and X's traffic halves.
+template <int EPI, bool SCALED, typename TC, int MT, int CT, int GD_WAVES, bool XT, bool OT>
 __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, float* __restrict__ resid_out,
     bf16_t* __restrict__ xw_out, const bf16_t* __restrict__ w_next, float* __restrict__ ss_out, const float* __restrict__ ss_in,
     int n_parts, float eps, int M, int N, int K) {
-    constexpr int NT = EPI == EPI_GATED ? 2 : 1;
+    constexpr int NT = (EPI == EPI_GATED ? 2 : 1) * CT;      // W tiles per block: [gate tiles | up tiles] for the gated product
     constexpr int MP = 16 * MT;
     __shared__ float red[(GD_WAVES - 1) * NT * MT * 64 * 4];
     __shared__ float ss_red[GD_WAVES * 4 * MP];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int r = lane & 15, g = lane >> 4;
-    const int n_base = blockIdx.x * 16;
 
     if (SCALED) {
         float part[MT];
@@ -212,12 +213,12 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    const size_t chunk_stride = (size_t)(NT * N / 16) * 4096;
-    const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)blockIdx.x * 4096;
+    const size_t chunk_stride = (size_t)((EPI == EPI_GATED ? 2 : 1) * N / 16) * 4096;
+    const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)blockIdx.x * (CT * 4096);
     unsigned woff[NT], xoff[MT];
     bool x_ok[MT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) woff[nt] = (unsigned)(nt * N / 16) * 4096u + 16u * lane;
+    for (int nt = 0; nt < NT; ++nt) woff[nt] = (unsigned)((nt / CT) * (N / 16) + nt % CT) * 4096u + 16u * lane;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         x_ok[mt] = 16 * mt + r < M;
@@ -269,45 +270,53 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
                 for (int i = 0; i < 4; ++i) acc[nt][mt][i] += red[((((w - 1) * NT + nt) * MT + mt) * 4 + i) * 64 + lane];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        const int m = 16 * mt + r, n = n_base + 4 * g;
+        const int m = 16 * mt + r;
+        float scale = 1.f;
         if (SCALED) {
             float s = 0.f;
             for (int i = 0; i < GD_WAVES * 4; ++i) s += ss_red[i * MP + m];
-            const float scale = 1.0f / sqrtf(s / (float)K + eps);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[nt][mt][i] *= scale;
+            scale = 1.0f / sqrtf(s / (float)K + eps);
         }
-        if (EPI == EPI_RESID) {
-            float s = 0.f;
-            if (m < M) {
-                float* hp = resid_out + (size_t)m * N + n;
-                f32x4_t h = *reinterpret_cast<const f32x4_t*>(hp);
-                const uint2 wn = *reinterpret_cast<const uint2*>(w_next + n);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) { h[i] += acc[0][mt][i]; s += h[i] * h[i]; }
-                *reinterpret_cast<f32x4_t*>(hp) = h;
-                uint2 o;
-                o.x = pack_bf16x2(h[0] * __uint_as_float(wn.x << 16), h[1] * __uint_as_float(wn.x & 0xffff0000u));
-                o.y = pack_bf16x2(h[2] * __uint_as_float(wn.y << 16), h[3] * __uint_as_float(wn.y & 0xffff0000u));
-                *reinterpret_cast<uint2*>(xw_out + (OT ? operand_order(m, n, MT) : (size_t)m * N + n)) = o;
+        for (int ct = 0; ct < CT; ++ct) {
+            const int tile = blockIdx.x * CT + ct, n = tile * 16 + 4 * g;
+            if (SCALED) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { acc[ct][mt][i] *= scale; if (EPI == EPI_GATED) acc[CT + ct][mt][i] *= scale; }
             }
-            s += __shfl_xor(s, 16, 64);
-            s += __shfl_xor(s, 32, 64);
-            if (g == 0) ss_out[blockIdx.x * MP + m] = s;      // rows beyond M: 0
-            continue;
-        }
-        if (m >= M) continue;
-        TC* out = C + (OT ? operand_order(m, n, MT) : (size_t)m * N + n);
+            if (EPI == EPI_RESID) {
+                float s = 0.f;
+                if (m < M) {
+                    float* hp = resid_out + (size_t)m * N + n;
+                    f32x4_t h = *reinterpret_cast<const f32x4_t*>(hp);
+                    const uint2 wn = *reinterpret_cast<const uint2*>(w_next + n);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float v = acc[0][mt][i];
-            if (EPI == EPI_GATED) { const float up = acc[NT - 1][mt][i]; v = (v / (1.0f + expf(-v))) * up; }
-            out[i] = from_f32<TC>(v);
+                    for (int i = 0; i < 4; ++i) { h[i] += acc[ct][mt][i]; s += h[i] * h[i]; }
+                    *reinterpret_cast<f32x4_t*>(hp) = h;
+                    uint2 o;
+                    o.x = pack_bf16x2(h[0] * __uint_as_float(wn.x << 16), h[1] * __uint_as_float(wn.x & 0xffff0000u));
+                    o.y = pack_bf16x2(h[2] * __uint_as_float(wn.y << 16), h[3] * __uint_as_float(wn.y & 0xffff0000u));
+                    *reinterpret_cast<uint2*>(xw_out + (OT ? operand_order(m, n, MT) : (size_t)m * N + n)) = o;
+                }
+                s += __shfl_xor(s, 16, 64);
+                s += __shfl_xor(s, 32, 64);
+                if (g == 0) ss_out[tile * MP + m] = s;      // rows beyond M: 0
+                continue;
+            }
+            if (m >= M) continue;
+            TC* out = C + (OT ? operand_order(m, n, MT) : (size_t)m * N + n);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float v = acc[ct][mt][i];
+                if (EPI == EPI_GATED) { const float up = acc[CT + ct][mt][i]; v = (v / (1.0f + expf(-v))) * up; }
+                out[i] = from_f32<TC>(v);
+            }
         }
     }
 }
+
+static int g_rows_two_tiles = 1;
+extern "C" void spy_gemm_decode_rows_two_tiles(int on) { g_rows_two_tiles = on; }    // for measurements
 
 struct GdArgs {
     const bf16_t* x; const bf16_t* w; void* c; float* resid; bf16_t* xw_out; const bf16_t* w_next; float* ss_out; const float* ss_in;
@@ -320,10 +329,17 @@ template <int EPI, bool SCALED, typename TC, bool XT, bool OT>
 static void gd_launch2(const GdArgs& a) {
     constexpr int W = EPI == EPI_GATED ? GD_WAVES_GATED : 8;
 #define GD_ARGS a.x, a.w, (TC*)a.c, a.resid, a.xw_out, a.w_next, a.ss_out, a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K
+    // Two column tiles per block where that leaves enough blocks (measured, 64 rows: qkv of 6144 columns 26.8 -> 20.5
+    // us; with 4096 columns, 128 blocks, 15.4 -> 19.4 us; the gated product 53 -> 61 us: its block has one wave per SIMD then)
+    const bool two = g_rows_two_tiles && EPI == EPI_STORE && a.N % 32 == 0 && a.N / 32 >= 192;
     if (a.M <= 16) gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
-    else if (a.M <= 32) gemm_decode_rows_kernel<EPI, SCALED, TC, 2, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
-    else if (a.M <= 48) gemm_decode_rows_kernel<EPI, SCALED, TC, 3, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
-    else gemm_decode_rows_kernel<EPI, SCALED, TC, 4, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
+#define GD_ROWS(MT)                                                                                                  \
+    if (two) gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 2, W, XT, OT><<<a.N / 32, W * 64, 0, a.st>>>(GD_ARGS);       \
+    else gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 1, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS)
+    else if (a.M <= 32) { GD_ROWS(2); }
+    else if (a.M <= 48) { GD_ROWS(3); }
+    else { GD_ROWS(4); }
+#undef GD_ROWS
 #undef GD_ARGS
 }
 

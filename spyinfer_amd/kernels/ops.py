@@ -173,8 +173,9 @@ _LIBRARY_F32_OUT = True      # torch.mm(..., out_dtype=float32) exists in this t
 TILED_WEIGHTS = True
 #: Most rows of a step whose products run with norms and residual sums folded in, handing their outputs over in operand
 #: order (above: the library product with norm kernels of their own).  Measured on MI355X at the Qwen3-8B shapes: such
-#: products beat the library's by 16 % at 32 rows and lose to it from about 56.
-FUSED_DECODE_MAX_ROWS = 48
+#: products beat the library's by 16 % at 32 rows and are level with it at 64 (where the step still gains 1.5 % from
+#: the norm and SwiGLU kernels it does not run).
+FUSED_DECODE_MAX_ROWS = 64
 
 
 def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:

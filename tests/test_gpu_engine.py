@@ -260,6 +260,55 @@ def test_folded_decode_steps(tmp_path_factory):
     assert torch.allclose(mixed[1:3], ref4[[1, 4]], **TOL["bfloat16"])
 
 
+@pytest.mark.parametrize("requests", [19, 37, 57, 64])
+def test_folded_decode_steps_of_many_requests(tmp_path_factory, requests):
+    """Decode steps of 17 to 64 requests take the folded products with two to four row tiles; their logits equal, up to
+    bfloat16 rounding, those of the same steps with the norms as kernels of their own, from graphs as well, and the last
+    step's equal the plain implementation's."""
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.runner import ModelRunner, load_model
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.weights import write_random_model
+    dev = require_gpu()
+    folder = write_random_model(str(tmp_path_factory.mktemp("eng_many")), TINY_D, 64, torch.bfloat16, **INIT)
+    plain = PlainQwen3(folder)
+    model = load_model(folder, "bfloat16", dev)
+    ps = prompts(400, [3 + (7 * i) % 23 for i in range(requests)], 5)
+    runs, calls = [], []
+    real = ops.decode_linear_residual
+    for folded, eager in ((True, True), (True, False), (False, True)):
+        ops.FUSED_DECODE = folded
+        n = [0]
+        ops.decode_linear_residual = lambda *a, **k: (n.__setitem__(0, n[0] + 1), real(*a, **k))[1]
+        try:
+            runner = ModelRunner(model, "bfloat16", dev, 16, 4 * requests, requests, enforce_eager=eager, max_model_len=64)
+            caches = [runner.manager.admit(i) for i in range(requests)]
+            for c, p in zip(caches, ps):
+                runner.manager.reserve(c, len(p))
+            runner.step([StepEntry(c, p, []) for c, p in zip(caches, ps)])
+            g = torch.Generator().manual_seed(6)
+            outs, seqs = [], [list(p) for p in ps]
+            for i in range(5):
+                toks = torch.randint(0, 400, (requests,), generator=g).tolist()
+                for c in caches:
+                    runner.manager.reserve(c, 1)
+                for q, t in zip(seqs, toks):
+                    q.append(t)
+                outs.append(runner.step([StepEntry(c, [t], [0]) for c, t in zip(caches, toks)]).cpu().clone())
+            runs.append(outs)
+            calls.append(n[0])
+        finally:
+            ops.FUSED_DECODE = True
+            ops.decode_linear_residual = real
+    assert calls[0] >= 5 * 2 * 3 and calls[2] == 0
+    for i, (a, b, c) in enumerate(zip(*runs)):
+        for x, what in ((b, "graphs"), (c, "plain norms")):
+            assert a.shape == x.shape and torch.allclose(a, x, **TOL["bfloat16"]), "step %d: folded and %s differ by %g" % (
+                i, what, (a - x).abs().max())
+    ref = torch.stack([plain.forward(q)[-1] for q in seqs])
+    assert torch.allclose(runs[0][-1], ref, **TOL["bfloat16"]), (runs[0][-1] - ref).abs().max()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_and_first_tokens(folder_c, dtype, tmp_path):
     require_gpu()
