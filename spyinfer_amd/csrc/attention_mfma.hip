@@ -28,6 +28,7 @@
 #include "common.h"
 #include "attention_merge.h"
 #include <math.h>
+#include <type_traits>
 
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
@@ -110,7 +111,10 @@ __device__ __forceinline__ void norm_rotate(bf16x8_t (&x)[KK], bool normed, cons
     }
 }
 
-template <int DMAX, bool FUSED>
+// FULL: head_dim == DMAX.  The loads of keys and values then have no conditions (a page that does not exist is read as
+// page 0 and what was read is masked: scores by position, values by the count of keys that exist), so the compiler knows
+// how many loads are in flight and a wait is for the oldest only.
+template <int DMAX, bool FUSED, bool FULL>
 __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void attention_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, bf16_t* kc, bf16_t* vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
@@ -209,42 +213,66 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         }
     }
 
-    // Pages are looked up one block ahead, both lookups together, and a block's K and V loads are
-    // all issued before its first product: a block costs one memory round trip, not four.
-    int kpage = -1, vpage = -1;
-    {
-        const int c0 = lo + 32 * (b_begin + wave);
-        const int key_a = c0 + 8 * (r16 >> 2) + (r16 & 3), key_v = c0 + 8 * g;
-        if (b_begin + wave < b_end) {
-            if (key_a < kvl) kpage = bt[key_a / P];
-            if (key_v < kvl) vpage = bt[key_v / P];
-        }
+    // A wave's loop is a chain of memory round trips, so they are overlapped: pages are looked up two blocks ahead (both
+    // lookups together); the keys of the next block are asked for as soon as this block's S^T products have read the
+    // key registers, and arrive while the softmax and the second product run; the values are asked for at the top of
+    // their block and arrive behind the first product.
+    int kpage = -1, vpage = -1, kpage_n = -1, vpage_n = -1;
+#define AM_LOOKUP(B, KP, VP)                                                                                  \
+    {                                                                                                         \
+        KP = -1;                                                                                              \
+        VP = -1;                                                                                              \
+        if ((B) < b_end) {                                                                                    \
+            const int c0_ = lo + 32 * (B);                                                                    \
+            const int ka_ = c0_ + 8 * (r16 >> 2) + (r16 & 3), kv_ = c0_ + 8 * g;                              \
+            if (ka_ < kvl) KP = bt[ka_ / P];                                                                  \
+            if (kv_ < kvl) VP = bt[kv_ / P];                                                                  \
+        }                                                                                                     \
     }
-    for (int b = b_begin + wave; b < b_end; b += AW) {
+    bf16x8_t ka[KK], kb[KK];
+    // tile a of block B has this lane's key lo + 32 B + 8 (r16 / 4) + r16 % 4; tile b is 4 keys on (same page: P % 8 == 0)
+#define AM_LOAD_K(B, KP)                                                                                      \
+    {                                                                                                         \
+        const int key_ = lo + 32 * (B) + 8 * (r16 >> 2) + (r16 & 3);                                          \
+        const bool ok_ = (KP) >= 0 && (KP) < num_pages;                                                       \
+        const bf16_t* kp_ = kc + (((size_t)(ok_ ? (KP) : 0) * n_kv + hk) * P + key_ % P) * d;                 \
+        _Pragma("unroll") for (int kk = 0; kk < KK; ++kk) {                                                   \
+            const int dofs = kk * 32 + 8 * g;                                                                 \
+            if (FULL) {                                                                                       \
+                ka[kk] = *reinterpret_cast<const bf16x8_t*>(kp_ + dofs);                                      \
+                kb[kk] = *reinterpret_cast<const bf16x8_t*>(kp_ + 4 * d + dofs);                              \
+            } else {                                                                                          \
+                ka[kk] = zero8();                                                                             \
+                kb[kk] = zero8();                                                                             \
+                if (ok_ && dofs < d) {                                                                        \
+                    ka[kk] = *reinterpret_cast<const bf16x8_t*>(kp_ + dofs);                                  \
+                    if (key_ + 4 < kvl) kb[kk] = *reinterpret_cast<const bf16x8_t*>(kp_ + 4 * d + dofs);      \
+                }                                                                                             \
+            }                                                                                                 \
+        }                                                                                                     \
+    }
+    AM_LOOKUP(b_begin + wave, kpage, vpage)
+    AM_LOOKUP(b_begin + wave + AW, kpage_n, vpage_n)
+    if (b_begin + wave < b_end) AM_LOAD_K(b_begin + wave, kpage)
+    // One block of 32 keys.  LAST: the wave's last block, which alone can hold keys beyond the request's and the step's
+    // new key, and after which no keys are asked for; the blocks before it have no condition around their loads.
+    auto block = [&](const int b, auto last_block) {
+        constexpr bool LAST = decltype(last_block)::value;
         const int c0 = lo + 32 * b;
-        const int key_a = c0 + 8 * (r16 >> 2) + (r16 & 3);      // tile a; tile b is key_a + 4 (same page: P % 8 == 0)
+        const int key_a = c0 + 8 * (r16 >> 2) + (r16 & 3);      // tile a; tile b is key_a + 4
         const int key_v = c0 + 8 * g;                             // this lane's 8 keys of V
-        const bool k_ok = kpage >= 0 && kpage < num_pages;
         const bool v_ok = vpage >= 0 && vpage < num_pages;
-        const bf16_t* kp = kc + (((size_t)(k_ok ? kpage : 0) * n_kv + hk) * P + key_a % P) * d;
         const bf16_t* vp = vc + (((size_t)(v_ok ? vpage : 0) * n_kv + hk) * d) * P + key_v % P;
-        bf16x8_t ka[KK], kb[KK], vt[DT];
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            const int dofs = kk * 32 + 8 * g;
-            ka[kk] = zero8();
-            kb[kk] = zero8();
-            if (k_ok && dofs < d) {
-                ka[kk] = *reinterpret_cast<const bf16x8_t*>(kp + dofs);
-                if (key_a + 4 < kvl) kb[kk] = *reinterpret_cast<const bf16x8_t*>(kp + 4 * d + dofs);
-            }
-        }
+        bf16x8_t vt[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             const int dd = dt * 16 + r16;
-            vt[dt] = (v_ok && dd < d) ? *reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P) : zero8();
+            if (FULL) vt[dt] = *reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P);
+            else vt[dt] = (v_ok && dd < d) ? *reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P) : zero8();
         }
-        if (FUSED && has_new && newpos >= c0 && newpos < c0 + 32) {
+        int kpage_nn, vpage_nn;
+        AM_LOOKUP(b + 2 * AW, kpage_nn, vpage_nn)
+        if (FUSED && LAST && has_new && newpos >= c0 && newpos < c0 + 32) {
             // the new key: the four lanes of its row take the prepared pieces; the lanes with r16 % 16 == its row store it
             const bool mine_a = key_a == newpos, mine_b = key_a + 4 == newpos;
 #pragma unroll
@@ -270,24 +298,22 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
             }
         }
         const int v_valid = min(8, kvl - key_v);                  // keys of the group that exist (slots beyond hold anything)
-        // the next block's pages
-        kpage = -1;
-        vpage = -1;
-        if (b + AW < b_end) {
-            const int na = key_a + 32 * AW, nv = key_v + 32 * AW;
-            if (na < kvl) kpage = bt[na / P];
-            if (nv < kvl) vpage = bt[nv / P];
-        }
         // ---- S^T = K . Q^T ------------------------------------------------------------------
         f32x4_t sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
-            if (kk * 32 < d) {
+            if (FULL || kk * 32 < d) {
                 sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[kk], bq[kk], sa, 0, 0, 0);
                 sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[kk], bq[kk], sb, 0, 0, 0);
             }
         }
-        if (v_ok && v_valid < 8) {
+        // the key registers are free: the next block's keys
+        if (!LAST) AM_LOAD_K(b + AW, kpage_n)
+        kpage = kpage_n;
+        vpage = vpage_n;
+        kpage_n = kpage_nn;
+        vpage_n = vpage_nn;
+        if ((LAST || !FULL) && (FULL || v_ok) && v_valid < 8) {
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -325,12 +351,19 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         // ---- O^T = O^T * alpha + V^T . P^T -----------------------------------------------------
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            if (dt * 16 < d) {
+            if (FULL || dt * 16 < d) {
                 acc[dt] *= alpha;
                 acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt], pb, acc[dt], 0, 0, 0);
             }
         }
+    };
+    {
+        int b = b_begin + wave;
+        for (; b + AW < b_end; b += AW) block(b, std::false_type{});
+        if (b < b_end) block(b, std::true_type{});
     }
+#undef AM_LOOKUP
+#undef AM_LOAD_K
     // the four lanes of a row hold partial sums of l
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
@@ -439,12 +472,12 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
     }
     const dim3 grid(num_tiles, n_kv, splits);
     const dim3 mgrid(num_tiles, n_kv);
-#define ATT_LAUNCH(DM, FZ)                                                                                                    \
-    attention_mfma_kernel<DM, FZ><<<grid, AW * 64, (AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>(                \
+#define ATT_LAUNCH(DM, FZ, FL)                                                                                                \
+    attention_mfma_kernel<DM, FZ, FL><<<grid, AW * 64, (AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>(                \
         (bf16_t*)out, (const bf16_t*)q, (bf16_t*)kc, (bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,  \
         tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz, out_tiles)
 #define ATT_CASE(DM)                                                                                                          \
-    if (qkv) ATT_LAUNCH(DM, true); else ATT_LAUNCH(DM, false);                                                                \
+    if (qkv) ATT_LAUNCH(DM, true, true); else if (d == DM) ATT_LAUNCH(DM, false, true); else ATT_LAUNCH(DM, false, false);       \
     if (splits > 1)                                                                                                           \
         attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits, 1, out_tiles);
     switch (dmax_of(d)) {
