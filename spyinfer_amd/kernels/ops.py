@@ -176,6 +176,12 @@ TILED_WEIGHTS = True
 #: products beat the library's by 16 % at 32 rows and are level with it at 64 (where the step still gains 1.5 % from
 #: the norm and SwiGLU kernels it does not run).
 FUSED_DECODE_MAX_ROWS = 64
+#: With four row tiles (49 to 64 rows) the products themselves are 8-12 % slower than the library's (every block reads
+#: all of X) and the step gains only by the norm and SwiGLU kernels it does not run, a fixed time per layer: at the
+#: Qwen3-8B shape (151 M elements in a layer's feed-forward) the step at 64 rows gains 1.5 %, at the 32B shape
+#: (393 M) it loses 5 %.  So parts whose matrices hold more than this many elements fold up to 48 rows only.
+FUSED_DECODE_WIDE_ROWS = 48
+FUSED_DECODE_WIDE_MAX_ELEMS = 1 << 28
 
 
 def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
@@ -303,6 +309,8 @@ def fused_decode_ok(rows: int, act_dtype, *tiled_weights) -> bool:
     """True if products of ``rows`` rows with these tiled matrices can run with the norm's scale and the residual
     sum folded in: bfloat16 activations, few rows, tiled bfloat16 weights."""
     if not FUSED_DECODE or _impl is not None or act_dtype != torch.bfloat16 or not 0 < rows <= FUSED_DECODE_MAX_ROWS:
+        return False
+    if rows > FUSED_DECODE_WIDE_ROWS and sum(t.numel() for t in tiled_weights if t is not None) > FUSED_DECODE_WIDE_MAX_ELEMS:
         return False
     return all(t is not None and t.dtype == torch.bfloat16 and t.shape[0] % 16 == 0 and t.shape[1] % 128 == 0
                for t in tiled_weights)
