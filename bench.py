@@ -90,7 +90,7 @@ def main() -> int:
     pages_per_req = -(-args.context // page)
     eng = LLMEngine.__new__(LLMEngine)
     eng._init_with_model(model, dev, dtype=args.dtype, max_model_len=args.context, kvcache_block_size=page,
-                         num_kvcache_blocks=pages_per_req * max_batch + 8, max_num_seqs=max_batch,
+                         num_kvcache_blocks=max(pages_per_req * max_batch, -(-args.prefill_tokens // page)) + 8, max_num_seqs=max_batch,
                          max_num_batched_tokens=max(16384, args.prefill_tokens), enforce_eager=args.enforce_eager, seed=args.seed)
     g = torch.Generator().manual_seed(args.seed)
 
