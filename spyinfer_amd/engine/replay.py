@@ -76,8 +76,8 @@ def run(argv=None, stdin=None, stdout=None) -> int:
                 rc = live[rid] = runner.manager.admit(rid)
             runner.manager.reserve(rc, len(tokens))
             entries.append(StepEntry(rc, tokens, [int(w) for w in ent.get("want", [])]))
-        logits = runner.step(entries)
-        if logits.shape[0] > 0:
+        logits = runner.step(entries) if entries else None        # a line may only end requests
+        if logits is not None and logits.shape[0] > 0:
             data = logits.detach().to("cpu", torch.float32).contiguous().numpy().astype("<f4", copy=False)
             tmp = os.path.join(args.out, "%s.f32.tmp" % step)
             data.tofile(tmp)

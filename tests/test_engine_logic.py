@@ -1,5 +1,6 @@
 """The engine's logic (batch metadata, cache pages, block tables, every way of cutting) on the
 CPU stand-in for the kernels, compared with the plain implementation."""
+import numpy as np
 import pytest
 import torch
 
@@ -36,3 +37,24 @@ def test_cuts_match_plain(name, mode, folders, tmp_path, emu_ops):
     if mode != "mixed":
         assert len(got) == sum(lengths)
     rc.compare(got, ref, atol=2e-4, rtol=2e-4, what="%s/%s" % (name, mode))
+
+
+def test_replay_lines_without_tokens_and_names_used_again(folders, tmp_path, emu_ops):
+    """A line may bring no tokens at all (it only ends requests), a request may be left out of steps, and a name that
+    has ended may be used again for a new request, which starts from an empty cache."""
+    cfg = TINY_A
+    reqs = rc.random_requests(cfg["vocab_size"], [21, 9], seed=5)
+    a, b = reqs["r0"], reqs["r1"]
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": a[:10], "want": [9]}], "end": []},
+             {"step": 1, "entries": [{"id": "y", "tokens": b, "want": [8]}], "end": []},
+             {"step": 2, "entries": [{"id": "x", "tokens": a[10:], "want": [10]}, {"id": "y", "tokens": [], "want": []}], "end": []},
+             {"step": 3, "entries": [], "end": ["x", "y"]},
+             {"step": 4, "entries": [{"id": "x", "tokens": b, "want": [0, 8]}], "end": ["x"]}]
+    rc.run_replay_inprocess(folders["A"], "float32", str(tmp_path), steps, 128, ["--device", "cpu"])
+    plain = PlainQwen3(folders["A"])
+    ra, rb = plain.forward(a), plain.forward(b)
+    V = cfg["vocab_size"]
+    read = lambda i, n: torch.from_numpy(np.fromfile(str(tmp_path / ("%d.f32" % i)), dtype="<f4").reshape(n, V).copy())
+    assert not (tmp_path / "3.f32").exists()
+    for got, ref in ((read(0, 1), ra[[9]]), (read(1, 1), rb[[8]]), (read(2, 1), ra[[20]]), (read(4, 2), rb[[0, 8]])):
+        assert torch.allclose(got, ref, atol=2e-4, rtol=2e-4)
