@@ -315,9 +315,6 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
     }
 }
 
-static int g_rows_two_tiles = 1;
-extern "C" void spy_gemm_decode_rows_two_tiles(int on) { g_rows_two_tiles = on; }    // for measurements
-
 struct GdArgs {
     const bf16_t* x; const bf16_t* w; void* c; float* resid; bf16_t* xw_out; const bf16_t* w_next; float* ss_out; const float* ss_in;
     int n_parts; float eps; int M, N, K; bool xt, ot; hipStream_t st;
@@ -331,11 +328,13 @@ static void gd_launch2(const GdArgs& a) {
 #define GD_ARGS a.x, a.w, (TC*)a.c, a.resid, a.xw_out, a.w_next, a.ss_out, a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K
     // Two column tiles per block where that leaves enough blocks (measured, 64 rows: qkv of 6144 columns 26.8 -> 20.5
     // us; with 4096 columns, 128 blocks, 15.4 -> 19.4 us; the gated product 53 -> 61 us: its block has one wave per SIMD then)
-    const bool two = g_rows_two_tiles && EPI == EPI_STORE && a.N % 32 == 0 && a.N / 32 >= 192;
+    const bool two = EPI == EPI_STORE && a.N % 32 == 0 && a.N / 32 >= 192;
     if (a.M <= 16) gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
 #define GD_ROWS(MT)                                                                                                  \
-    if (two) gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 2, W, XT, OT><<<a.N / 32, W * 64, 0, a.st>>>(GD_ARGS);       \
-    else gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 1, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS)
+    if constexpr (EPI == EPI_STORE) {                                                                                \
+        if (two) gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 2, W, XT, OT><<<a.N / 32, W * 64, 0, a.st>>>(GD_ARGS);   \
+        else gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 1, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);      \
+    } else gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 1, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS)
     else if (a.M <= 32) { GD_ROWS(2); }
     else if (a.M <= 48) { GD_ROWS(3); }
     else { GD_ROWS(4); }
