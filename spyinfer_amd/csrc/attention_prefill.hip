@@ -338,9 +338,18 @@ extern "C" int64_t spy_attention_prefill_workspace(int num_tiles, int n_kv, int 
     return (int64_t)num_tiles * (PF_ROWS / 16) * n_kv * splits * 16 * ((d <= 64 ? 64 : 128) + 2);
 }
 
-// Grids of up to this many blocks (a CU count and a half) take the 8-wave shape.  Measured on MI355X, 32 query heads
-// of 128: 2048 tokens (256 blocks) 104 -> 78 us with it, 4096 tokens (512 blocks) 238 -> 274 us.
-static const long long g_thin_below = 384;
+// Grids of at most one block per CU take the 8-wave shape: a block of 4 waves would leave every SIMD with a single
+// wave.  Measured on MI355X (256 CUs), 32 query heads of 128, 8-wave against 4-wave blocks: 2048 tokens (256 blocks)
+// 65 against 85 us; 2304 tokens (288 blocks) 130 against 116 us; 4096 tokens (512 blocks) 217 against 193 us.
+static long long thin_below() {
+    static long long cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus = n;
+    }
+    return cus;
+}
 
 extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, const void* vc, int P, int num_pages, const int* cu_q,
                                      const int* pos0, const int* kv_len, const int* block_table, int max_blocks,
@@ -358,7 +367,7 @@ extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, c
     SPY_REQUIRE(splits == 1 || ws, "spy_attention_prefill: key parts without a workspace");
     const dim3 grid(splits > 1 ? num_tiles : (num_tiles + 1) / 2, n_kv, splits);
     const dim3 mgrid(num_tiles * (PF_ROWS / 16), n_kv);
-    bool thin = (long long)grid.x * grid.y * grid.z <= g_thin_below;     // (only for head sizes 64 and 128: the others need too many registers)
+    bool thin = (long long)grid.x * grid.y * grid.z <= thin_below();     // (only for head sizes 64 and 128: the others need too many registers)
 #define PF_LAUNCH(DM, FULL)                                                                                                      \
     if (thin) attention_prefill_kernel<DM, FULL, 1><<<grid, PF_ROWS * 4, 0, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, \
                                                                  P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,      \
