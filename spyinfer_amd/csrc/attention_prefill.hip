@@ -1,9 +1,9 @@
-// Paged attention on MFMA for entries with many query rows (prompt portions): a block of 4 waves
-// works on 128 rows of one entry and one kv head, 32 rows (two 16-row MFMA tiles) per wave.  Rows
-// are (token, query head of the group) pairs as in attention_mfma.hip.  Keys and values of 64 keys
-// at a time are gathered through the block table into LDS once per block (prefetched into
-// registers while the previous 64 keys are worked on) and shared by the 8 row tiles; every K and V
-// fragment that a wave reads from LDS serves both of its row tiles.
+// Paged attention on MFMA for entries with many query rows (prompt portions): a block works on 128 rows of one entry
+// and one kv head, as 8 waves of one 16-row MFMA tile each (head sizes 64 and 128) or 4 waves of two tiles each (the
+// other head sizes).  Rows are (token, query head of the group) pairs as in attention_mfma.hip.  Keys and values of
+// 64 keys at a time are gathered through the block table into LDS once per block (prefetched into registers while
+// the previous 64 keys are worked on) and shared by the 8 row tiles; with two row tiles per wave every K and V
+// fragment that a wave reads from LDS serves both.
 //
 // MFMA arrangement as in attention_mfma.hip: S^T = K . Q^T in two tiles whose key order leaves
 // lane (q row, g) with the scores of 8 consecutive keys, which are exactly the 8 k-values that
@@ -25,11 +25,13 @@ __device__ __forceinline__ bf16x8_t pf_zero8() { return bf16x8_t{0, 0, 0, 0, 0, 
 
 // DFULL: head_dim == DMAX, so no part of the head-dim loops is conditional and the compiler may move the LDS reads of
 // a whole 32-key half ahead of its products.
-// RT: 16-row tiles per wave.  2 (4 waves per block): every K and V fragment read from LDS serves two row tiles.  1 (8
-// waves per block): for grids with one block per CU only, where 4 waves would leave every SIMD with a single wave and
-// nothing to run while that wave waits (measured at 2048 tokens: 60 % of the cycles were such waits).
-template <int DMAX, bool DFULL, int RT>
-__global__ __launch_bounds__(PF_ROWS / RT * 4, RT == 1 ? 1 : 2) void attention_prefill_kernel(
+// RT: 16-row tiles per wave.  2 (4 waves per block): every K and V fragment read from LDS serves two row tiles, but a
+// SIMD has one wave per block and little to run while it waits.  1 (8 waves per block): two waves per SIMD and block.
+// MINW: waves per SIMD that the registers must allow.  The 8-wave shape with 4 (128 registers, two blocks per CU) is
+// the fastest shape for grids of more than one block per CU; with one block per CU it is 6 % faster with the
+// registers of 2.
+template <int DMAX, bool DFULL, int RT, int MINW>
+__global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
@@ -338,10 +340,11 @@ extern "C" int64_t spy_attention_prefill_workspace(int num_tiles, int n_kv, int 
     return (int64_t)num_tiles * (PF_ROWS / 16) * n_kv * splits * 16 * ((d <= 64 ? 64 : 128) + 2);
 }
 
-// Grids of at most one block per CU take the 8-wave shape: a block of 4 waves would leave every SIMD with a single
-// wave.  Measured on MI355X (256 CUs), 32 query heads of 128, 8-wave against 4-wave blocks: 2048 tokens (256 blocks)
-// 65 against 85 us; 2304 tokens (288 blocks) 130 against 116 us; 4096 tokens (512 blocks) 217 against 193 us.
-static long long thin_below() {
+// Measured on MI355X (256 CUs), 32 query heads of 128, microseconds per call for 2048 / 2304 / 3072 / 4096 / 8192
+// tokens of one prompt (256 / 288 / 384 / 512 / 1024 blocks): 4 waves of two row tiles 85 / 115 / 148 / 193 / 717;
+// 8 waves of one row tile with registers for one block per CU 65 / 130 / 165 / 217 / 807, with 128 registers (two
+// blocks per CU) 69 / 98 / 129 / 185 / 677.  So: 8 waves always (full head sizes), the registers by the grid.
+static long long cu_count() {
     static long long cus = 0;
     if (cus == 0) {
         int dev = 0, n = 0;
@@ -367,24 +370,21 @@ extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, c
     SPY_REQUIRE(splits == 1 || ws, "spy_attention_prefill: key parts without a workspace");
     const dim3 grid(splits > 1 ? num_tiles : (num_tiles + 1) / 2, n_kv, splits);
     const dim3 mgrid(num_tiles * (PF_ROWS / 16), n_kv);
-    bool thin = (long long)grid.x * grid.y * grid.z <= thin_below();     // (only for head sizes 64 and 128: the others need too many registers)
-#define PF_LAUNCH(DM, FULL)                                                                                                      \
-    if (thin) attention_prefill_kernel<DM, FULL, 1><<<grid, PF_ROWS * 4, 0, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, \
-                                                                 P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,      \
-                                                                 tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p,      \
-                                                                 num_tiles, splits, ws);                                         \
-    else attention_prefill_kernel<DM, FULL, 2><<<grid, PF_ROWS * 2, 0, st>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, \
-                                                                 P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,      \
-                                                                 tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p,      \
-                                                                 num_tiles, splits, ws)
+    const bool one_per_cu = (long long)grid.x * grid.y * grid.z <= cu_count();
+#define PF_ARGS (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table,   \
+                max_blocks, tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p, num_tiles, splits, ws
+    // (head sizes other than 64 and 128 keep the 4-wave shape: with conditions in the head-dim loops the other needs too many registers)
 #define PF_CASE(DM)                                                                                                              \
-    if (d == DM) { PF_LAUNCH(DM, true); } else { thin = false; PF_LAUNCH(DM, false); }                                           \
+    if (d == DM) {                                                                                                               \
+        if (one_per_cu) attention_prefill_kernel<DM, true, 1, 2><<<grid, PF_ROWS * 4, 0, st>>>(PF_ARGS);                         \
+        else attention_prefill_kernel<DM, true, 1, 4><<<grid, PF_ROWS * 4, 0, st>>>(PF_ARGS);                                    \
+    } else attention_prefill_kernel<DM, false, 2, 2><<<grid, PF_ROWS * 2, 0, st>>>(PF_ARGS);                                     \
     if (splits > 1)                                                                                                              \
         attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits,    \
                                                           PF_ROWS / 16);
     if (d <= 64) { PF_CASE(64) } else { PF_CASE(128) }
-#undef PF_LAUNCH
 #undef PF_CASE
+#undef PF_ARGS
     SPY_CHECK_LAUNCH("spy_attention_prefill");
     return 0;
 }
