@@ -233,9 +233,13 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kern
 #pragma unroll
                 for (int j = 0; j < 8; ++j) sc[j] = j < 4 ? sa[t][j] : sb[t][j - 4];
                 if (!unmasked) {
+                    // (the empty statement keeps the masks' index arithmetic inside this branch: the compiler had moved
+                    // it ahead of the branch, into the path of every block of keys)
+                    int key0 = h0 + 8 * g;
+                    asm volatile("" : "+v"(key0));
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
-                        const int key = h0 + 8 * g + j;
+                        const int key = key0 + j;
                         const bool ok = row_ok[t] && key <= pos[t] && key >= lo_row[t] && key < kvl;
                         sc[j] = ok ? sc[j] : -INFINITY;
                     }
