@@ -94,7 +94,7 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
         const char* xb_ = xbase + (size_t)(CHUNK) * (XT ? 4096 : GD_CHUNK * 2) + xoff;                   \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                  \
             _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                            \
-                A[nt][j] = *reinterpret_cast<const bf16x8_t*>(wb_ + woff[nt] + 1024 * j);                \
+                A[nt][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wb_ + woff[nt] + 1024 * j));                \
             B[j] = x_ok ? *reinterpret_cast<const bf16x8_t*>(xb_ + (XT ? 1024 : 64) * j) : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; \
         }                                                                                                \
     }
@@ -232,7 +232,7 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
         const char* xb = xbase + (size_t)(CHUNK) * (XT ? 4 * MT * 1024 : GD_CHUNK * 2);                              \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                              \
             _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                        \
-                A[nt][j] = *reinterpret_cast<const bf16x8_t*>(wb + woff[nt] + 1024 * j);                             \
+                A[nt][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wb + woff[nt] + 1024 * j));                             \
             _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                        \
                 B[mt][j] = x_ok[mt] ? *reinterpret_cast<const bf16x8_t*>(xb + xoff[mt] + (XT ? MT * 1024 : 64) * j)  \
                                     : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};                                              \
