@@ -239,14 +239,14 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         _Pragma("unroll") for (int kk = 0; kk < KK; ++kk) {                                                   \
             const int dofs = kk * 32 + 8 * g;                                                                 \
             if (FULL) {                                                                                       \
-                ka[kk] = *reinterpret_cast<const bf16x8_t*>(kp_ + dofs);                                      \
-                kb[kk] = *reinterpret_cast<const bf16x8_t*>(kp_ + 4 * d + dofs);                              \
+                ka[kk] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(kp_ + dofs));                                      \
+                kb[kk] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(kp_ + 4 * d + dofs));                              \
             } else {                                                                                          \
                 ka[kk] = zero8();                                                                             \
                 kb[kk] = zero8();                                                                             \
                 if (ok_ && dofs < d) {                                                                        \
-                    ka[kk] = *reinterpret_cast<const bf16x8_t*>(kp_ + dofs);                                  \
-                    if (key_ + 4 < kvl) kb[kk] = *reinterpret_cast<const bf16x8_t*>(kp_ + 4 * d + dofs);      \
+                    ka[kk] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(kp_ + dofs));                                  \
+                    if (key_ + 4 < kvl) kb[kk] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(kp_ + 4 * d + dofs));      \
                 }                                                                                             \
             }                                                                                                 \
         }                                                                                                     \
@@ -267,7 +267,7 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             const int dd = dt * 16 + r16;
-            if (FULL) vt[dt] = *reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P);
+            if (FULL) vt[dt] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P));
             else vt[dt] = (v_ok && dd < d) ? *reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P) : zero8();
         }
         int kpage_nn, vpage_nn;
