@@ -260,9 +260,9 @@ def test_folded_decode_steps(tmp_path_factory):
     assert torch.allclose(mixed[1:3], ref4[[1, 4]], **TOL["bfloat16"])
 
 
-@pytest.mark.parametrize("requests", [19, 37, 57, 64])
+@pytest.mark.parametrize("requests", [19, 37, 57, 64, 70])
 def test_folded_decode_steps_of_many_requests(tmp_path_factory, requests):
-    """Decode steps of 17 to 64 requests take the folded products with two to four row tiles; their logits equal, up to
+    """Decode steps of 17 to 64 requests take the folded products with two to four row tiles (70 requests: the library's); their logits equal, up to
     bfloat16 rounding, those of the same steps with the norms as kernels of their own, from graphs as well, and the last
     step's equal the plain implementation's.  Parts with large matrices fold up to 48 rows only (the limit is made tiny
     here): the embedding then still prepares the first norm's input, which the unfolded block does not use."""
@@ -302,7 +302,10 @@ def test_folded_decode_steps_of_many_requests(tmp_path_factory, requests):
         finally:
             ops.FUSED_DECODE, ops.FUSED_DECODE_WIDE_MAX_ELEMS = True, wide
             ops.decode_linear_residual = real
-    assert calls[0] >= 5 * 2 * 3 and calls[2] == 0 and (calls[3] == 0) == (requests > ops.FUSED_DECODE_WIDE_ROWS)
+    if requests <= ops.FUSED_DECODE_MAX_ROWS:
+        assert calls[0] >= 5 * 2 * 3 and calls[2] == 0 and (calls[3] == 0) == (requests > ops.FUSED_DECODE_WIDE_ROWS)
+    else:
+        assert calls == [0, 0, 0, 0]          # more rows than the folded products take: the library's, with norm kernels
     for i, (a, b, c, e) in enumerate(zip(*runs)):
         for x, what in ((b, "graphs"), (c, "plain norms"), (e, "large matrices")):
             assert a.shape == x.shape and torch.allclose(a, x, **TOL["bfloat16"]), "step %d: folded and %s differ by %g" % (
