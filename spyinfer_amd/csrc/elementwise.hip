@@ -42,6 +42,38 @@ __global__ __launch_bounds__(256) void embedding_sumsq_kernel(float* __restrict_
     const TW* row = table + (size_t)(id < 0 || id >= V ? 0 : id) * H;
     const bool known = id >= 0 && id < V;
     float s = 0.f;
+    if (H % 8 == 0 && ((uintptr_t)table % 16) == 0 && ((uintptr_t)w_norm % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)xw % 16) == 0) {
+        // 8 values per thread and step: one or two 16-byte loads of the row, one of the weight, two 16-byte stores of
+        // the stream and one of the product's input (8 consecutive columns are one piece in operand order too)
+        typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+        typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f4_t;
+        for (int i = threadIdx.x * 8; i < H; i += blockDim.x * 8) {
+            float v[8];
+            if (sizeof(TW) == 2) {
+                const u32x4_t r4 = *reinterpret_cast<const u32x4_t*>(row + i);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { v[2 * e] = __uint_as_float(r4[e] << 16); v[2 * e + 1] = __uint_as_float(r4[e] & 0xffff0000u); }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = to_f32<TW>(row[i + e]);
+            }
+            const u32x4_t w4 = *reinterpret_cast<const u32x4_t*>(w_norm + i);
+            u32x4_t y;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (!known) { v[2 * e] = 0.f; v[2 * e + 1] = 0.f; }
+                y[e] = pack_bf16x2(v[2 * e] * __uint_as_float(w4[e] << 16), v[2 * e + 1] * __uint_as_float(w4[e] & 0xffff0000u));
+                s += v[2 * e] * v[2 * e] + v[2 * e + 1] * v[2 * e + 1];
+            }
+            *reinterpret_cast<f4_t*>(o + i) = f4_t{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<f4_t*>(o + i + 4) = f4_t{v[4], v[5], v[6], v[7]};
+            bf16_t* dst = tiled ? xw + (((size_t)(i >> 5) * (gridDim.x >> 4) + (t >> 4)) * 64 + ((i & 31) >> 3) * 16 + (t & 15)) * 8 : x + i;
+            *reinterpret_cast<u32x4_t*>(dst) = y;
+        }
+        s = block_sum(s, red);
+        if (threadIdx.x == 0) ss[t] = s;
+        return;
+    }
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
         const float v = known ? to_f32<TW>(row[i]) : 0.f;
         o[i] = v;
