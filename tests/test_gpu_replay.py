@@ -21,7 +21,7 @@ CASES = {"A": (TINY_A, [5, 17, 33, 60], 16), "B": (TINY_B, [1, 40, 130], 8), "C"
          "D": (TINY_D, [9, 50, 190, 77, 300], 16), "E": (TINY_E, [2, 130, 425, 61], 16)}
 # float32: only the order of sums differs.  bfloat16: activations are rounded to 8 bits between
 # kernels; with these weights the CPU model of that rounding differs from float32 by up to 0.04
-# on logits of standard deviation 0.7 ("tolerances").
+# on logits of standard deviation 0.7, hence twice that as the absolute tolerance.
 TOL = {"float32": dict(atol=1e-4, rtol=1e-4), "bfloat16": dict(atol=8e-2, rtol=2e-2)}
 
 
