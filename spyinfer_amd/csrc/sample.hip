@@ -5,7 +5,9 @@
 // (2) one wave per row merges the chunks in id order, finds the chunk that holds u * total and
 // walks it.  All sums run over ascending ids, so the choice is a function of (logits, T, u) alone.
 #include "common.h"
+#include "no_alloc.h"
 #include <math.h>
+#include <mutex>
 
 #define SM_CHUNKS 64
 #define SM_THREADS 256
@@ -131,16 +133,64 @@ __global__ __launch_bounds__(64) void sample_pick_kernel(const float* __restrict
 
 extern "C" int64_t spy_sample_workspace(int R) { return (int64_t)R * SM_CHUNKS * 3; }
 
-extern "C" int spy_sample(const float* logits, const float* temperature, const float* uniform, int* out, int R, int V, float* ws,
-                          hipStream_t st) {
-    SPY_REQUIRE(R > 0 && V > 0, "spy_sample: empty operand");
-    SPY_REQUIRE(R <= 65535, "spy_sample: too many rows");
-    SPY_REQUIRE(ws, "spy_sample: no workspace");
+// Both kernels; ``ws`` holds spy_sample_workspace(R) floats of device memory.
+static int launch_sample(const char* name, const float* logits, const float* temperature, const float* uniform, int* out, int R, int V,
+                         float* ws, hipStream_t st) {
     float* pmax = ws;
     int* pidx = reinterpret_cast<int*>(ws + (size_t)R * SM_CHUNKS);
     float* psum = ws + (size_t)2 * R * SM_CHUNKS;
     sample_chunks_kernel<<<dim3(SM_CHUNKS, R), SM_THREADS, 0, st>>>(logits, temperature, pmax, pidx, psum, V);
     sample_pick_kernel<<<R, 64, 0, st>>>(logits, temperature, uniform, pmax, pidx, psum, out, V);
-    SPY_CHECK_LAUNCH("spy_sample");
+    SPY_CHECK_LAUNCH(name);
     return 0;
+}
+
+extern "C" int spy_sample(const float* logits, const float* temperature, const float* uniform, int* out, int R, int V, float* ws,
+                          hipStream_t st) {
+    SPY_REQUIRE(R > 0 && V > 0, "spy_sample: empty operand");
+    SPY_REQUIRE(R <= 65535, "spy_sample: too many rows");
+    SPY_REQUIRE(ws, "spy_sample: no workspace");
+    return launch_sample("spy_sample", logits, temperature, uniform, out, R, V, ws, st);
+}
+
+// ---- the variant that allocates nothing (no_alloc.h) ------------------------------------------------------------
+// The workspace of the two kernels as an array of the library: every GPU that runs the library has its own copy at
+// its own address.  In host code the array's name is only a handle for hipGetSymbolAddress, never a device pointer.
+static __device__ __align__(256) float scratch[(size_t)SPY_SAMPLE_STATIC_MAX_ROWS * SM_CHUNKS * 3];
+
+#define SPY_MAX_DEVICES 64
+static std::mutex g_scratch_lock;
+static float* g_scratch_ptr[SPY_MAX_DEVICES];      // the array's address on each device, asked for once per device
+
+// The current device's copy of ``scratch``; nullptr (and the error recorded) if it cannot be had.
+static float* scratch_of_current_device() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= SPY_MAX_DEVICES) {
+        spy_fail("spy_sample_static: no current device (%s)", e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        float* ptr = nullptr;
+        e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            spy_fail("spy_sample_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
+extern "C" int spy_sample_static(const float* logits, const float* temperature, const float* uniform, int* out, int R, int V,
+                                 hipStream_t st) {
+    SPY_REQUIRE(R > 0 && V > 0, "spy_sample_static: empty operand");
+    SPY_REQUIRE(R <= SPY_SAMPLE_STATIC_MAX_ROWS, "spy_sample_static: %d rows, the library's scratch array holds %d at most", R,
+                SPY_SAMPLE_STATIC_MAX_ROWS);
+    SPY_REQUIRE(logits && temperature && uniform && out, "spy_sample_static: null operand");
+    float* ws = scratch_of_current_device();
+    if (!ws) return 1;
+    // nothing to clear: sample_chunks_kernel writes all 3 * R * SM_CHUNKS elements that sample_pick_kernel reads
+    return launch_sample("spy_sample_static", logits, temperature, uniform, out, R, V, ws, st);
 }

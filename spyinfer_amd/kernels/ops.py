@@ -75,7 +75,7 @@ class _Hip:
                      "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_prefill",
                      "spy_attention_prefill_workspace", "spy_swiglu",
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
-                     "spy_gemm_decode", "spy_embedding_sumsq"):
+                     "spy_gemm_decode", "spy_embedding_sumsq", "spy_sample_static"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: rebuild it (python -c 'import __graft_entry__ as g; g.build()')"
                                   % (self.lib._name, name))
