@@ -60,7 +60,6 @@ def main() -> int:
 
     import torch
 
-    from spyinfer_amd.cache.spec import PagedKV
     from spyinfer_amd.config.registry import architecture_of
     from spyinfer_amd.engine.batch import StepEntry
     from spyinfer_amd.engine.llm_engine import LLMEngine
@@ -102,7 +101,7 @@ def main() -> int:
     nq, nkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
     layer_params = H * (nq + 2 * nkv) * d + nq * d * H + 3 * H * I + 2 * H + 2 * d
     weight_bytes = (L * layer_params + H + V * H) * act_bytes              # every weight a decode step uses, once
-    kv_bytes_per_token = sum(2 * s.num_kv_heads * s.head_dim * act_bytes for s in model.cache_specs() if isinstance(s, PagedKV))
+    kv_bytes_per_token = sum(s.page_bytes(1, run_dtype) for s in model.cache_specs() if s is not None and s.paged)
 
     def decode_run(batch, steps, warmup):
         """tokens/s, ms/step, mean context over the timed steps."""

@@ -25,6 +25,7 @@ def main(argv=None) -> int:
     ap.add_argument("-b", dest="backend_type", default="hip", help="backend; available: " + ", ".join(BACKENDS))
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--max-num-batched-tokens", type=int, default=16384)
+    ap.add_argument("--prefill-chunk", type=int, default=2048, help="most tokens of one request in one step")
     ap.add_argument("--max-num-seqs", type=int, default=512)
     ap.add_argument("--max-model-len", type=int, default=4096)
     ap.add_argument("--gpu-memory-utilization", type=float, default=0.9)
@@ -59,7 +60,8 @@ def main(argv=None) -> int:
     from .sampling import SamplingParams
 
     engine = LLMEngine(args.model_path, dtype=args.dtype, max_num_batched_tokens=args.max_num_batched_tokens,
-                       max_num_seqs=args.max_num_seqs, max_model_len=args.max_model_len,
+                       prefill_chunk=args.prefill_chunk, max_num_seqs=args.max_num_seqs, max_model_len=args.max_model_len,
+                       keep_finished_cache=not args.prompt_ids,       # the conversation's further turns compute their new tokens only
                        gpu_memory_utilization=args.gpu_memory_utilization, enforce_eager=args.enforce_eager,
                        kvcache_block_size=args.kvcache_block_size, num_kvcache_blocks=args.num_kvcache_blocks, seed=args.seed)
     params = SamplingParams(temperature=args.temperature, max_new_tokens=args.max_new_tokens, ignore_eos=args.ignore_eos)

@@ -1,3 +1,3 @@
 from .manager import CacheManager, OutOfSlots, PageGroup, RequestCache, SlotPool, StateGroup
 from .pages import OutOfPages, PagePool
-from .spec import FixedState, PagedKV
+from .spec import CacheKind, FixedState, PagedKV, PagedKVLayer, StateLayer

@@ -14,7 +14,7 @@ import dataclasses
 from typing import Dict, List, Optional, Sequence
 
 from .pages import OutOfPages, PagePool
-from .spec import FixedState, PagedKV
+from .spec import CacheKind
 
 
 class OutOfSlots(RuntimeError):
@@ -55,7 +55,7 @@ class PageGroup:
     """Layer caches with one need: they share page numbers and block tables."""
 
     index: int
-    spec: PagedKV
+    spec: CacheKind
     cache_ids: List[int]
     page_size: int
     pool: PagePool
@@ -71,7 +71,7 @@ class PageGroup:
 @dataclasses.dataclass
 class StateGroup:
     index: int
-    spec: FixedState
+    spec: CacheKind
     cache_ids: List[int]
 
 
@@ -106,22 +106,21 @@ class CacheManager:
         for cid, spec in enumerate(cache_specs):
             if spec is None:
                 continue
-            if isinstance(spec, PagedKV):
+            if not isinstance(spec, CacheKind):
+                raise TypeError("cache need %r of layer cache %d is no CacheKind" % (spec, cid))
+            # equal kinds share a group: one pool of pages (or the slots) and one block table per request
+            if spec.paged:
                 grp = next((g for g in self.page_groups if g.spec == spec), None)
                 if grp is None:
                     grp = PageGroup(len(self.page_groups), spec, [], page_size, PagePool(num_pages))
                     self.page_groups.append(grp)
-                self.location[cid] = ("paged", grp.index, len(grp.cache_ids))
-                grp.cache_ids.append(cid)
-            elif isinstance(spec, FixedState):
+            else:
                 grp = next((g for g in self.state_groups if g.spec == spec), None)
                 if grp is None:
                     grp = StateGroup(len(self.state_groups), spec, [])
                     self.state_groups.append(grp)
-                self.location[cid] = ("state", grp.index, len(grp.cache_ids))
-                grp.cache_ids.append(cid)
-            else:
-                raise TypeError("cache spec %r of layer cache %d is neither PagedKV nor FixedState" % (spec, cid))
+            self.location[cid] = ("paged" if spec.paged else "state", grp.index, len(grp.cache_ids))
+            grp.cache_ids.append(cid)
         self.slots = SlotPool(max_num_seqs)
         self.requests: Dict[object, RequestCache] = {}
 

@@ -1,14 +1,9 @@
 """Device memory behind the cache manager's page and slot numbers.
 
-Per page group, for its ``n`` layer caches:
-  keys    ``[n, num_pages, num_kv_heads, page_size, head_dim]``
-  values  ``[n, num_pages, num_kv_heads, head_dim, page_size]``  (transposed in the page)
-A page number addresses the same page in every layer of the group, as in the
-reference (src/engine/model_runner.cpp:35-40, layout ``[L, NB, P, n_kv*d]``
-there).  Here one head's part of a page is contiguous, so that a wave reads it
-with full-width loads, and values lie with the key index innermost, which is
-the operand order of the MFMA product P.V.
-Per state group: ``[n, num_slots, *shape]``.
+Every group's kind (``cache.spec.CacheKind``) allocates the tensors of its
+layers and says what one layer sees of them.  A page number addresses the same
+page in every layer of a group, as in the reference
+(src/engine/model_runner.cpp:35-40, layout ``[L, NB, P, n_kv*d]`` there).
 """
 from __future__ import annotations
 
@@ -17,23 +12,7 @@ from typing import Dict, List
 import torch
 
 from .manager import CacheManager
-
-
-class PagedKVLayer:
-    """The part of a page group's memory that one layer cache owns."""
-
-    def __init__(self, group: int, k: torch.Tensor, v: torch.Tensor, page_size: int):
-        self.group = group
-        self.k = k
-        self.v = v
-        self.page_size = page_size
-        self.num_pages = k.shape[0]
-
-
-class StateLayer:
-    def __init__(self, group: int, state: torch.Tensor):
-        self.group = group
-        self.state = state      # [num_slots, *shape]
+from .spec import PagedKVLayer, StateLayer  # noqa: F401  (the layer views' home was here)
 
 
 class CacheStorage:
@@ -41,19 +20,13 @@ class CacheStorage:
         self.manager = manager
         self.layers: Dict[int, object] = {}
         self.tensors: List[torch.Tensor] = []
-        for g in manager.page_groups:
-            n, s = len(g.cache_ids), g.spec
-            k = torch.zeros((n, g.pool.num_pages, s.num_kv_heads, g.page_size, s.head_dim), dtype=act_dtype, device=device)
-            v = torch.zeros((n, g.pool.num_pages, s.num_kv_heads, s.head_dim, g.page_size), dtype=act_dtype, device=device)
-            self.tensors += [k, v]
-            for i, cid in enumerate(g.cache_ids):
-                self.layers[cid] = PagedKVLayer(g.index, k[i], v[i], g.page_size)
-        for g in manager.state_groups:
-            dt = torch.float32 if g.spec.dtype == "float32" else act_dtype
-            st = torch.zeros((len(g.cache_ids), manager.slots.num_slots) + tuple(g.spec.shape), dtype=dt, device=device)
-            self.tensors.append(st)
-            for i, cid in enumerate(g.cache_ids):
-                self.layers[cid] = StateLayer(g.index, st[i])
+        for groups, count_of in ((manager.page_groups, lambda g: g.pool.num_pages),
+                                 (manager.state_groups, lambda g: manager.slots.num_slots)):
+            for g in groups:
+                tensors = g.spec.allocate(len(g.cache_ids), count_of(g), manager.page_size, act_dtype, device)
+                self.tensors += tensors
+                for i, cid in enumerate(g.cache_ids):
+                    self.layers[cid] = g.spec.layer_view(g.index, tensors, i, manager.page_size)
 
     def layer(self, cache_id: int):
         return self.layers.get(cache_id)
@@ -61,10 +34,14 @@ class CacheStorage:
     def num_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.tensors)
 
+    def fill(self, value: float) -> None:
+        """Every element of every cache tensor := value (tests poison the pool with NaN this way: a slot is
+        always written before it is read, so a correct engine never shows it)."""
+        for t in self.tensors:
+            if t.is_floating_point():
+                t.fill_(value)
+
     @staticmethod
-    def bytes_per_page(manager_specs, page_size: int, act_bytes: int) -> int:
-        """Bytes that one more page costs, summed over all page groups."""
-        total = 0
-        for spec, n_layers in manager_specs:
-            total += 2 * n_layers * spec.num_kv_heads * spec.head_dim * page_size * act_bytes
-        return total
+    def bytes_per_page(cache_specs, page_size: int, act_dtype: torch.dtype) -> int:
+        """Bytes that one more page in every page group costs, over all layer caches."""
+        return sum(s.page_bytes(page_size, act_dtype) for s in cache_specs if s is not None and s.paged)

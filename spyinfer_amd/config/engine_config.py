@@ -14,6 +14,9 @@ class EngineConfig:
     dtype: str = "bfloat16"
     #: most tokens in one step, prompt portions and decoded tokens together (config.hpp:19)
     max_num_batched_tokens: int = 16384
+    #: most tokens of ONE request in one step: longer prompts are cut into portions of this size, so that the requests
+    #: decoding beside them get a token every step (the reference runs every prompt whole, scheduler.cpp:59-71)
+    prefill_chunk: int = 2048
     #: most requests running at once (config.hpp:20)
     max_num_seqs: int = 512
     #: most tokens of one request, clamped to max_position_embeddings (config.hpp:12, 21)
@@ -29,11 +32,14 @@ class EngineConfig:
     num_kvcache_blocks: Optional[int] = None
     #: base seed of temperature sampling
     seed: int = 0
+    #: True: a finished request keeps its pages and slot for a further turn (append_to_request), as the reference's do
+    #: until they are removed (llm_engine.cpp:40-73); they are the first to go when pages or slots are short
+    keep_finished_cache: bool = False
 
     def validate(self) -> None:
         if self.dtype not in ("bfloat16", "float32"):
             raise ValueError("dtype must be 'bfloat16' or 'float32', got %r" % (self.dtype,))
-        for name in ("max_num_batched_tokens", "max_num_seqs", "max_model_len", "kvcache_block_size"):
+        for name in ("max_num_batched_tokens", "prefill_chunk", "max_num_seqs", "max_model_len", "kvcache_block_size"):
             if getattr(self, name) <= 0:
                 raise ValueError("%s must be positive" % name)
         if self.num_kvcache_blocks is not None and self.num_kvcache_blocks <= 0:

@@ -11,7 +11,7 @@ from __future__ import annotations
 import dataclasses
 import json
 import os
-from typing import Any, ClassVar, Dict, List
+from typing import Any, ClassVar, Dict, List, Optional
 
 
 class ConfigError(ValueError):
@@ -65,6 +65,17 @@ class ModelConfig:
     def validate(self) -> None:
         pass
 
+    # What the engine itself asks of any architecture's configuration, whatever its config.json keys are called.
+    @property
+    def position_limit(self) -> Optional[int]:
+        """Most tokens a request may reach (the architecture's positions end there); None = no limit."""
+        return None
+
+    @property
+    def end_token_id(self) -> Optional[int]:
+        """The token at which generation ends; None = the architecture names none."""
+        return None
+
 
 def _coerce(name, value, type_name):
     t = str(type_name)
@@ -113,6 +124,14 @@ class Qwen3Config(ModelConfig):
     vocab_size: int = -1
 
     required: ClassVar[tuple] = ("model_type", "hidden_act")
+
+    @property
+    def position_limit(self):
+        return self.max_position_embeddings
+
+    @property
+    def end_token_id(self):
+        return self.eos_token_id if self.eos_token_id >= 0 else None
 
     def fill_defaults(self) -> None:
         if self.head_dim == -1 and self.num_attention_heads > 0:

@@ -16,11 +16,6 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, RequestCache
-from ..kernels.ops import AttentionMeta, key_parts_for
-
-ROWS_PER_TILE = 16        # rows of (token, head-in-group) pairs in a small attention tile
-ROWS_PER_BIG_TILE = 128   # rows in a tile of the prefill attention kernel
-BIG_MIN_ROWS = 64         # entries with at least this many rows go to the prefill kernel
 
 
 class StepEntry:
@@ -61,7 +56,9 @@ class StepBatch:
         self.fixed_shape = fixed_max_blocks > 0
         self._arrays: Dict[str, np.ndarray] = {}
         self._dev: Dict[str, torch.Tensor] = {}
-        self._tiles: Dict[int, int] = {}
+        #: host-side notes of the parts for this step (what one layer planned, the next need not plan again)
+        self.shared: Dict[object, object] = {}
+        self._graph_extra: Dict[str, object] = {}
         seen = set()
         lens = np.empty(S, dtype=np.int32)
         pos0 = np.empty(S, dtype=np.int32)
@@ -130,31 +127,15 @@ class StepBatch:
             raise RuntimeError("the batch is already on the device")
         self._arrays[name] = np.asarray(values, dtype=np.int32).reshape(-1)
 
-    def add_attention_tiles(self, group_size: int, big_tiles: bool = True) -> None:
-        """Tiles over each entry's rows (token-major, head-in-group minor) for a query-head group of
-        ``group_size``: entries with at least BIG_MIN_ROWS rows are cut into 128-row tiles (the
-        LDS-sharing prefill kernel), the others into 16-row tiles (one block of waves each)."""
-        if group_size in self._tiles:
-            return
-        rows = self.lens.astype(np.int64) * group_size
-        big = (rows >= BIG_MIN_ROWS) & bool(big_tiles)
-        counts = {}
-        for kind, size, mask in (("small", ROWS_PER_TILE, ~big), ("big", ROWS_PER_BIG_TILE, big)):
-            ntiles = np.where(mask, (rows + size - 1) // size, 0)
-            tile_entry = np.repeat(np.arange(self.S, dtype=np.int32), ntiles)
-            first = np.zeros(self.S + 1, dtype=np.int64)
-            np.cumsum(ntiles, out=first[1:])
-            tile_row0 = ((np.arange(int(first[-1]), dtype=np.int64) - first[:-1][tile_entry]) * size).astype(np.int32)
-            if kind == "big" and tile_entry.shape[0] > 2:
-                # the prefill kernel gives a block the tiles b and n - 1 - b: sorted by the keys they read, blocks are even
-                pos0 = self._arrays["pos0"][tile_entry].astype(np.int64)
-                last_tok = np.minimum(self.lens[tile_entry].astype(np.int64), (tile_row0.astype(np.int64) + size + group_size - 1) // group_size)
-                order = np.argsort(-(pos0 + last_tok), kind="stable")
-                tile_entry, tile_row0 = tile_entry[order], tile_row0[order]
-            counts[kind] = int(first[-1])
-            self.add_array("tile_entry_%s_%d" % (kind, group_size), tile_entry)
-            self.add_array("tile_row0_%s_%d" % (kind, group_size), tile_row0)
-        self._tiles[group_size] = counts
+    def has_array(self, name: str) -> bool:
+        return name in self._arrays
+
+    def add_graph_key(self, name: str, value) -> None:
+        """A part's ``plan`` says what, beside the arrays' lengths, the shape of its launches takes from this step
+        (a number of blocks that follows the requests' lengths, say): a captured graph is replayed only for steps
+        with the same values."""
+        self._graph_extra[name] = value
+        self._graph_key = None
 
     # ---- to the device -------------------------------------------------------
     def layout(self):
@@ -171,7 +152,7 @@ class StepBatch:
     def graph_key(self):
         """What a captured graph of this step depends on beside the arrays' contents."""
         if self._graph_key is None:
-            self._graph_key = (self.layout_key(), self.all_rows_wanted, key_parts_for(self.max_kv_len))
+            self._graph_key = (self.layout_key(), self.all_rows_wanted, tuple(sorted(self._graph_extra.items())))
         return self._graph_key
 
     def host_array(self, name: str) -> np.ndarray:
@@ -212,13 +193,3 @@ class StepBatch:
 
     def block_table(self, group: int) -> torch.Tensor:
         return self._dev["block_table_%d" % group].view(self.S, self.max_blocks[group])
-
-    def attention_meta(self, group: int, group_size: int) -> AttentionMeta:
-        tiles = None
-        if group_size in self._tiles:
-            tiles = {}
-            for kind, n in self._tiles[group_size].items():
-                tiles[kind] = (self._dev["tile_entry_%s_%d" % (kind, group_size)], self._dev["tile_row0_%s_%d" % (kind, group_size)], n)
-        return AttentionMeta(self._dev["cu_q"], self._dev["pos0"], self._dev["kv_len"], self.block_table(group),
-                             self._dev["token_entry"], self._dev["positions"], self.S, self.T, self.max_blocks[group],
-                             self.max_kv_len, self.max_q_len, tiles, group_size, fixed_shape=self.fixed_shape)

@@ -40,6 +40,25 @@ class _Flight(NamedTuple):
         return [int(x) for x in self.host.tolist()]
 
 
+def pages_for_memory(free_bytes: int, config: EngineConfig, model) -> int:
+    """Pages of the cache pool when ``free_bytes`` of device memory are free (num_kvcache_blocks not given): the share
+    ``gpu_memory_utilization`` of what is left after the memory that captured decode steps will hold over the run
+    (``ModelRunner.graph_memory_bound``; nothing with enforce_eager), less a tenth for the activations of one full
+    step; never more than max_num_seqs requests of max_model_len tokens need."""
+    page = config.kvcache_block_size
+    per_page = ModelRunner.bytes_per_page(model, page, config.dtype)
+    if per_page == 0:
+        return 1
+    blocks = -(-config.max_model_len // page)
+    graphs = 0
+    if not config.enforce_eager:
+        groups = len({s for s in model.cache_specs() if s is not None and s.paged})
+        graphs = ModelRunner.graph_logits_bytes(config.max_num_seqs, model.vocab_size) \
+            + ModelRunner.MAX_GRAPHS * ModelRunner.graph_metadata_bytes(config.max_num_seqs, groups, blocks)
+    pages = int(max(0, free_bytes - graphs) * config.gpu_memory_utilization * 0.9) // per_page
+    return max(1, min(pages, blocks * config.max_num_seqs))
+
+
 class LLMEngine:
     def __init__(self, model_path: str, device="cuda:0", **params):
         known = {f for f in EngineConfig.__dataclass_fields__}
@@ -60,7 +79,9 @@ class LLMEngine:
         self.model = model
         mc = self.model.config
         # as the reference: a request never outgrows the model's positions (src/config.hpp:12)
-        self.config.max_model_len = min(self.config.max_model_len, getattr(mc, "max_position_embeddings", 1 << 30))
+        limit = self.model.max_positions or mc.position_limit
+        if limit:
+            self.config.max_model_len = min(self.config.max_model_len, limit)
         num_pages = self.config.num_kvcache_blocks
         if num_pages is None:
             num_pages = self._pages_from_free_memory()
@@ -68,9 +89,9 @@ class LLMEngine:
                                   self.config.max_num_seqs, self.config.max_num_batched_tokens,
                                   enforce_eager=self.config.enforce_eager, max_model_len=self.config.max_model_len)
         self.scheduler = Scheduler(self.runner.manager, self.config.max_num_batched_tokens, self.config.max_num_seqs,
-                                   self.config.max_model_len)
+                                   self.config.max_model_len, self.config.prefill_chunk)
         self.sampler = Sampler(self.device)
-        self.eos_token_id = getattr(mc, "eos_token_id", -1)
+        self.eos_token_id = -1 if mc.end_token_id is None else mc.end_token_id
         self._sequences: Dict[int, Sequence] = {}
         self._next_id = 0
         self.stats = dict(steps=0, prefill_tokens=0, decode_tokens=0)
@@ -79,17 +100,11 @@ class LLMEngine:
         self.run_ahead = True
 
     def _pages_from_free_memory(self) -> int:
-        per_page = ModelRunner.bytes_per_page(self.model, self.config.kvcache_block_size, self.config.dtype)
-        if per_page == 0:
-            return 1
         if self.device.type == "cuda":
             free, _total = torch.cuda.mem_get_info(self.device)
         else:
             free = 1 << 30
-        # room for the activations of one full step is left beside the pool
-        pages = int(free * self.config.gpu_memory_utilization * 0.9) // per_page
-        cap = -(-self.config.max_model_len // self.config.kvcache_block_size) * self.config.max_num_seqs
-        return max(1, min(pages, cap))
+        return pages_for_memory(free, self.config, self.model)
 
     # ---- requests --------------------------------------------------------
     def add_request(self, prompt_tokens: Seq[int], params: Optional[SamplingParams] = None) -> int:
@@ -106,17 +121,25 @@ class LLMEngine:
         return rid
 
     def append_to_request(self, request_id: int, tokens: Seq[int], params: Optional[SamplingParams] = None) -> None:
-        """A further turn of a finished request (src/engine/llm_engine.cpp:40-73).  The reference keeps the
-        finished request's pages and prefills the new tokens only; here pages went back when it finished,
-        so the history is computed again.  The tokens that come out are the same."""
+        """A further turn of a finished request (src/engine/llm_engine.cpp:40-73).  As in the reference only the new
+        tokens are computed if the request still holds its cache (``keep_finished_cache``); if its pages went back
+        when it finished, or were taken back since, the history is computed again.  The tokens that come out are the
+        same.  A turn that is refused (ValueError) leaves the request as it was."""
         seq = self._sequences[request_id]
         if seq.status is not SequenceStatus.FINISHED:
             raise ValueError("request %d is still running" % request_id)
-        seq.tokens += [int(t) for t in tokens]
-        seq.num_prompt_tokens = len(seq.tokens)
+        new = [int(t) for t in tokens]
+        for t in new:
+            if not (0 <= t < self.model.vocab_size):
+                raise ValueError("token id %d is outside the vocabulary of %d" % (t, self.model.vocab_size))
         if params is not None:
             params.validate()
-            seq.params = params
+        turn = params if params is not None else seq.params
+        self.scheduler.check_admissible(len(seq.tokens) + len(new), turn.max_new_tokens)      # raises before anything changes
+        seq.draws_before += seq.num_generated
+        seq.tokens += new
+        seq.num_prompt_tokens = len(seq.tokens)
+        seq.params = turn
         seq.finish_reason = None
         self.scheduler.add_sequence(seq)
 
@@ -139,7 +162,7 @@ class LLMEngine:
 
     def remove_request(self, request_id: int) -> None:
         seq = self._sequences.pop(request_id)
-        if seq.status is not SequenceStatus.FINISHED:
+        if seq.status is not SequenceStatus.FINISHED or seq.cache is not None:
             self.scheduler.abort(seq)
 
     # ---- one step --------------------------------------------------------
@@ -176,7 +199,7 @@ class LLMEngine:
             elif len(seq) >= self.config.max_model_len:
                 reason = "max_model_len"
             if reason:
-                self.scheduler.finish(seq, reason)
+                self.scheduler.finish(seq, reason, keep=self.config.keep_finished_cache)
             outputs.append(StepOutput(seq.id, tok, reason is not None))
         self._flight = ahead
         return outputs
@@ -201,7 +224,7 @@ class LLMEngine:
         picked = self.sampler.sample_device(
             logits, [s.params.temperature for s in sampling],
             [s.params.seed if s.params.seed is not None else self.config.seed + s.id for s in sampling],
-            [s.num_generated + ahead for s in sampling])
+            [s.num_draws + ahead for s in sampling])
         self.stats["steps"] += 1
         for sc in scheduled:
             self.stats["decode_tokens" if sc.num_tokens == 1 and sc.samples else "prefill_tokens"] += sc.num_tokens

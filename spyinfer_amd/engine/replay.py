@@ -41,6 +41,8 @@ def run(argv=None, stdin=None, stdout=None) -> int:
     ap.add_argument("--kvcache-block-size", type=int, default=16, help="tokens in a cache page")
     ap.add_argument("--max-num-seqs", type=int, default=8, help="most live requests")
     ap.add_argument("--device", default="cuda:0")
+    ap.add_argument("--poison-cache", action="store_true",
+                    help="fill the cache pool with NaN before the first step: a read of a slot that no step wrote shows in the logits")
     args = ap.parse_args(argv)
     stdin = stdin or sys.stdin
     stdout = stdout or sys.stdout
@@ -58,6 +60,8 @@ def run(argv=None, stdin=None, stdout=None) -> int:
     num_pages = page_rounded_tokens(args.max_tokens, args.kvcache_block_size)
     runner = ModelRunner(model, args.dtype, args.device, args.kvcache_block_size, num_pages, args.max_num_seqs,
                          max_num_batched_tokens=1 << 30)
+    if args.poison_cache:
+        runner.storage.fill(float("nan"))
     live = {}
     for line in stdin:
         line = line.strip()

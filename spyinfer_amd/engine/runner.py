@@ -13,7 +13,6 @@ from typing import List, Optional, Sequence
 import torch
 
 from ..cache.manager import CacheManager
-from ..cache.spec import PagedKV
 from ..cache.storage import CacheStorage
 from ..config.registry import load_model_config
 from ..models.base import DecoderModel
@@ -51,6 +50,9 @@ class PreparedStep:
 
 
 class ModelRunner:
+    #: most step shapes that are captured as graphs
+    MAX_GRAPHS = 256
+
     def __init__(self, model: DecoderModel, dtype, device, page_size: int, num_pages: int, max_num_seqs: int,
                  max_num_batched_tokens: int = 16384, enforce_eager: bool = True, max_model_len: Optional[int] = None):
         """``enforce_eager=False``: steps that hold single tokens only (decoding) are captured in
@@ -66,11 +68,17 @@ class ModelRunner:
         self.use_graphs = (not enforce_eager) and self.device.type == "cuda"
         limit = max_model_len or model.max_positions or num_pages * page_size
         self.fixed_max_blocks = min(-(-limit // page_size), max(1, num_pages))
-        #: captured steps by shape.  Each holds its step's activations and logits, so at most ``max_graphs`` are
-        #: captured; further shapes run kernel by kernel.  A captured step is kept as long as the runner: none
-        #: is destroyed between steps, while others may be in flight.
+        #: captured steps by shape; at most ``max_graphs``, further shapes run kernel by kernel.  A captured step is
+        #: kept as long as the runner: none is destroyed between steps, while others may be in flight.  All captures
+        #: allocate from one memory pool and write their logits into one tensor, so what they hold together is the
+        #: activations of the largest step, that tensor and each graph's own copy of the step's metadata
+        #: (``graph_memory_bound``): steps run one after the other on one stream, and a step's logits are read
+        #: (sampled, copied) before the next step is queued.
         self._graphs = {}
-        self.max_graphs = 256
+        self.max_graphs = self.MAX_GRAPHS
+        self.max_num_seqs = max_num_seqs
+        self._graph_pool = None
+        self._graph_logits = None
         self._seen = {}
         self._pinned = None
         self._copied = None
@@ -80,8 +88,26 @@ class ModelRunner:
     @staticmethod
     def bytes_per_page(model: DecoderModel, page_size: int, dtype) -> int:
         """Device bytes that one more page in every page group costs."""
-        act = 2 if resolve_dtype(dtype) == torch.bfloat16 else 4
-        return sum(2 * s.num_kv_heads * s.head_dim * page_size * act for s in model.cache_specs() if isinstance(s, PagedKV))
+        return CacheStorage.bytes_per_page(model.cache_specs(), page_size, resolve_dtype(dtype))
+
+    # ---- what captured steps cost ------------------------------------------------
+    @staticmethod
+    def graph_logits_bytes(max_num_seqs: int, vocab_size: int) -> int:
+        """The one float32 tensor [max_num_seqs, vocab] that every captured step writes its logits into."""
+        return 4 * max_num_seqs * vocab_size
+
+    @staticmethod
+    def graph_metadata_bytes(entries: int, page_groups: int, fixed_max_blocks: int) -> int:
+        """Upper bound of a captured step's own metadata buffer: per entry a row of ``fixed_max_blocks`` page numbers
+        in every page group and 64 further integers (token, position, lengths, slots, tiles; each array padded to 16 B)."""
+        return 4 * (entries * (page_groups * fixed_max_blocks + 64) + 256)
+
+    def graph_memory_bound(self, max_graphs: Optional[int] = None) -> int:
+        """Most device bytes that captured steps hold beside the activations of the largest of them (which any step,
+        captured or not, needs while it runs): the shared logits tensor and ``max_graphs`` metadata buffers."""
+        n = self.max_graphs if max_graphs is None else max_graphs
+        return self.graph_logits_bytes(self.max_num_seqs, self.model.vocab_size) \
+            + n * self.graph_metadata_bytes(self.max_num_seqs, len(self.manager.page_groups), self.fixed_max_blocks)
 
     def prepare(self, entries: Sequence[StepEntry]) -> "PreparedStep":
         """The host work of a step that does not need the device: the batch's arrays, the checks, the parts' plans."""
@@ -186,10 +212,14 @@ class ModelRunner:
         self._upload(batch, dev_buf)
         if token_source is not None:
             batch.token_ids.copy_(token_source)
+        if self._graph_pool is None:
+            self._graph_pool = torch.cuda.graph_pool_handle()
+            self._graph_logits = torch.empty((self.max_num_seqs, self.model.vocab_size), dtype=torch.float32, device=self.device)
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            logits = self.model.forward(batch, self.storage)
+        out = self._graph_logits[:batch.R] if batch.R <= self.max_num_seqs else None
+        with torch.cuda.graph(graph, pool=self._graph_pool):
+            logits = self.model.forward(batch, self.storage, out)
         self._graphs[key] = (graph, dev_buf, logits)
         graph.replay()                          # capture launches nothing: this replay is the step
         self.graph_replays += 1
@@ -205,4 +235,4 @@ class ModelRunner:
         idx = torch.tensor(fresh, dtype=torch.long, device=self.device)
         for g in self.manager.state_groups:
             for cid in g.cache_ids:
-                self.storage.layer(cid).state.index_fill_(0, idx, 0)
+                g.spec.reset(self.storage.layer(cid), idx)

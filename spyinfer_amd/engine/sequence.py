@@ -25,6 +25,9 @@ class Sequence:
         self.cache: Optional[RequestCache] = None
         self.finish_reason: Optional[str] = None
         self.num_preemptions = 0
+        #: draws of the sampler made in earlier turns of this request (a further turn goes on in the same stream of
+        #: uniform numbers instead of starting it again)
+        self.draws_before = 0
         self.admit_order = -1
 
     def __len__(self) -> int:
@@ -38,6 +41,11 @@ class Sequence:
     @property
     def num_generated(self) -> int:
         return len(self.tokens) - self.num_prompt_tokens
+
+    @property
+    def num_draws(self) -> int:
+        """Index of the request's next draw of the sampler."""
+        return self.draws_before + self.num_generated
 
     @property
     def is_prefill(self) -> bool:

@@ -171,17 +171,19 @@ _LIBRARY_F32_OUT = True      # torch.mm(..., out_dtype=float32) exists in this t
 #: then whole cache lines).  Costs the weights' size again in device memory; the row-major copy stays for the
 #: library product of prefill.
 TILED_WEIGHTS = True
-#: Most rows of a step whose products run with norms and residual sums folded in, handing their outputs over in operand
-#: order (above: the library product with norm kernels of their own).  Measured on MI355X at the Qwen3-8B shapes: such
-#: products beat the library's by 16 % at 32 rows and are level with it at 64 (where the step still gains 1.5 % from
-#: the norm and SwiGLU kernels it does not run).
+#: Most rows that the decode products (``decode_linear`` and its kin) take.
 FUSED_DECODE_MAX_ROWS = 64
-#: With four row tiles (49 to 64 rows) the products themselves are 8-12 % slower than the library's (every block reads
-#: all of X) and the step gains only by the norm and SwiGLU kernels it does not run, a fixed time per layer: at the
-#: Qwen3-8B shape (151 M elements in a layer's feed-forward) the step at 64 rows gains 1.5 %, at the 32B shape
-#: (393 M) it loses 5 %.  So parts whose matrices hold more than this many elements fold up to 48 rows only.
-FUSED_DECODE_WIDE_ROWS = 48
-FUSED_DECODE_WIDE_MAX_ELEMS = 1 << 28
+
+
+def default_fold_rows(weight_elements: int) -> int:
+    """Most rows of a step for which a part with ``weight_elements`` matrix elements should run its products with the
+    norms and residual sums folded in (above: the library product with norm kernels of their own), where the part's
+    builder names no limit.  Measured on MI355X: such products beat the library's by 16 % at 32 rows and are level with
+    it at 64 rows; with four row tiles (49 to 64 rows) the products themselves are 8-12 % slower than the library's (every
+    block reads all of X) and the step gains only by the norm and SwiGLU kernels it does not run, a fixed time per layer.
+    With 151 M elements in a feed-forward the step at 64 rows gains 1.5 %, with 393 M it loses 5 %: parts with more than
+    2^28 elements fold up to 48 rows only."""
+    return 48 if weight_elements > (1 << 28) else FUSED_DECODE_MAX_ROWS
 
 
 def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
@@ -196,15 +198,26 @@ def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
     return w.view(N // 16, 16, K // 128, 4, 4, 8).permute(2, 0, 3, 4, 1, 5).contiguous().view(N, K)
 
 
+def _result(out: Optional[torch.Tensor], M: int, N: int, dtype: torch.dtype, device) -> torch.Tensor:
+    """The [M, N] result tensor of a product: ``out`` if the caller brought one (checked), else a new one."""
+    if out is None:
+        return torch.empty((M, N), dtype=dtype, device=device)
+    _check(tuple(out.shape) == (M, N) and out.dtype == dtype and out.device == device and out.is_contiguous(),
+           "the result tensor brought by the caller must be contiguous %s [%d, %d] on %s" % (dtype, M, N, device))
+    return out
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-           tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
+           tiled: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y = x . w^T with w stored [N, K] (out_features, in_features), float32 accumulation.
     ``tiled``: the same matrix from ``tile_weight``, used when few bfloat16 rows stream it.
+    ``out``: the result is written there (a tensor of the result's shape and dtype) instead of into a new tensor.
 
     float32 anywhere among x and w -> the hand-written true-fp32 kernel.  All bfloat16: the streaming
     MFMA kernel for few rows, the library product for many."""
     if _impl is not None:
-        return _impl.linear(x, w, out_dtype)
+        y = _impl.linear(x, w, out_dtype)
+        return y if out is None else out.copy_(y)
     _dev(x, w)
     _check(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "linear: x [M, K] and w [N, K] expected, got %s and %s"
            % (tuple(x.shape), tuple(w.shape)))
@@ -212,26 +225,25 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     N = w.shape[0]
     out_dtype = out_dtype or x.dtype
     _check(out_dtype in _CODES, "linear: output dtype must be float32 or bfloat16")
+    out = _result(out, M, N, out_dtype, x.device)
     if M == 0:
-        return torch.empty((0, N), dtype=out_dtype, device=x.device)
+        return out
     all_bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
     if all_bf16 and tiled is not None and M <= SKINNY_MAX_ROWS:
         _check(tiled.shape == w.shape, "linear: the tiled copy does not fit the matrix")
-        return decode_linear(x, tiled, out_dtype)
+        return decode_linear(x, tiled, out_dtype, out)
     global _LIBRARY_F32_OUT
     if all_bf16 and out_dtype == torch.float32 and M > SKINNY_MAX_ROWS and _LIBRARY_F32_OUT:
         try:
-            return torch.mm(x, w.t(), out_dtype=torch.float32)      # logits of many rows: the library, float32 result
+            return torch.mm(x, w.t(), out_dtype=torch.float32, out=out)      # logits of many rows: the library, float32 result
         except TypeError:
             _LIBRARY_F32_OUT = False
     if all_bf16 and K % 8 == 0 and M <= (SKINNY_MAX_ROWS_F32_OUT if out_dtype == torch.float32 else SKINNY_MAX_ROWS):
-        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         hip().call("spy_gemm_skinny", _ptr(x), _ptr(w), _ptr(out), _code(out, "out"), ctypes.c_int(M), ctypes.c_int(N),
                    ctypes.c_int(K), _Hip.stream())
         return out
     if all_bf16 and out_dtype == torch.bfloat16 and M > SKINNY_MAX_ROWS:
-        return torch.matmul(x, w.t())
-    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        return torch.matmul(x, w.t(), out=out)
     hip().call("spy_gemm", _ptr(x), _code(x, "x"), _ptr(w), _code(w, "w"), _ptr(out), _code(out, "out"),
                ctypes.c_int(M), ctypes.c_int(N), ctypes.c_int(K), _Hip.stream())
     return out
@@ -305,12 +317,15 @@ FUSED_DECODE = True
 OPERAND_ORDER = True
 
 
-def fused_decode_ok(rows: int, act_dtype, *tiled_weights) -> bool:
+def fused_decode_ok(rows: int, act_dtype, *tiled_weights, max_rows: Optional[int] = None) -> bool:
     """True if products of ``rows`` rows with these tiled matrices can run with the norm's scale and the residual
-    sum folded in: bfloat16 activations, few rows, tiled bfloat16 weights."""
+    sum folded in: bfloat16 activations, at most ``max_rows`` rows (default: ``default_fold_rows`` of the matrices),
+    tiled bfloat16 weights."""
     if not FUSED_DECODE or _impl is not None or act_dtype != torch.bfloat16 or not 0 < rows <= FUSED_DECODE_MAX_ROWS:
         return False
-    if rows > FUSED_DECODE_WIDE_ROWS and sum(t.numel() for t in tiled_weights if t is not None) > FUSED_DECODE_WIDE_MAX_ELEMS:
+    if max_rows is None:
+        max_rows = default_fold_rows(sum(t.numel() for t in tiled_weights if t is not None))
+    if rows > max_rows:
         return False
     return all(t is not None and t.dtype == torch.bfloat16 and t.shape[0] % 16 == 0 and t.shape[1] % 128 == 0
                for t in tiled_weights)
@@ -360,10 +375,11 @@ def _operand_order_ok(width: int) -> bool:
     return OPERAND_ORDER and width % 32 == 0
 
 
-def decode_linear(x, tiled: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
-    """y = x . w^T for at most 16 rows; ``x`` bfloat16 [M, K], OperandRows or a ScaledInput, ``tiled`` from tile_weight."""
+def decode_linear(x, tiled: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y = x . w^T for few rows; ``x`` bfloat16 [M, K], OperandRows or a ScaledInput, ``tiled`` from tile_weight; the
+    result goes into ``out`` if one is brought."""
     N = tiled.shape[0]
-    out = torch.empty((_rows_of(x), N), dtype=out_dtype, device=tiled.device)
+    out = _result(out, _rows_of(x), N, out_dtype, tiled.device)
     _gemm_decode(x, tiled, 0, N, out, None, None, None, None)
     return out
 

@@ -13,7 +13,6 @@ from typing import Dict, List, NamedTuple, Optional, Sequence
 
 import torch
 
-from ..kernels.ops import ScaledInput
 from ..parts.base import Block, Norm, PositionEncoding
 from ..parts.embedding import LMHead, TokenEmbedding
 from ..weights.loader import WeightSpec
@@ -90,9 +89,9 @@ class DecoderModel:
         for call in self.schedule:
             self.layers[call.layer].mixer.plan(batch)
 
-    def forward(self, batch, storage) -> torch.Tensor:
+    def forward(self, batch, storage, logits_out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Runs the batch's tokens through all calls of the run order; float32 logits [R, vocab]
-        at the batch's wanted rows."""
+        at the batch's wanted rows (in ``logits_out`` if the caller brings a tensor of that shape)."""
         calls = self.schedule
         entry = [self.layers[c.layer].entry_norm() for c in calls] + [self.final_norm]
         if self.position is None or type(self.position).on_embeddings is PositionEncoding.on_embeddings:
@@ -103,10 +102,5 @@ class DecoderModel:
             cache = storage.layer(call.cache) if call.cache is not None else None
             resid, pending = self.layers[call.layer].forward(resid, pending, batch, cache, call.store, next_norm=entry[i + 1])
         if batch.R == 0:
-            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=resid.device)
-        if isinstance(pending, ScaledInput):
-            if pending.norm is self.final_norm and batch.all_rows_wanted and self.lm_head.can_fold(batch):
-                return self.lm_head.forward(pending)
-            pending = None                       # the stream is complete
-        normed = self.final_norm.add_norm(resid, pending, batch.act_dtype, batch.logit_rows)
-        return self.lm_head.forward(normed)
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=resid.device) if logits_out is None else logits_out
+        return self.lm_head.logits(resid, pending, self.final_norm, batch, logits_out)

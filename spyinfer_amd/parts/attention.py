@@ -14,6 +14,7 @@ from __future__ import annotations
 import math
 from typing import Optional
 
+import numpy as np
 import torch
 
 from ..cache.spec import PagedKV
@@ -22,10 +23,66 @@ from ..weights.loader import WeightSpec
 from .base import Mixer, PositionEncoding
 
 
+ROWS_PER_TILE = 16        # rows of (token, head-in-group) pairs in a small attention tile
+ROWS_PER_BIG_TILE = 128   # rows in a tile of the prefill attention kernel
+BIG_MIN_ROWS = 64         # entries with at least this many rows go to the prefill kernel
+
+
+def plan_attention_tiles(batch, group_size: int, big_tiles: bool = True) -> None:
+    """Adds to the step's arrays the tiles over each entry's rows (token-major, head-in-group minor) for a query-head
+    group of ``group_size``: entries with at least BIG_MIN_ROWS rows are cut into 128-row tiles (the LDS-sharing
+    prefill kernel), the others into 16-row tiles (one block of waves each).  Once per step and group size."""
+    note = ("attention_tiles", group_size)
+    if note in batch.shared:
+        return
+    S, lens = batch.S, batch.lens
+    rows = lens.astype(np.int64) * group_size
+    big = (rows >= BIG_MIN_ROWS) & bool(big_tiles)
+    counts = {}
+    for kind, size, mask in (("small", ROWS_PER_TILE, ~big), ("big", ROWS_PER_BIG_TILE, big)):
+        ntiles = np.where(mask, (rows + size - 1) // size, 0)
+        tile_entry = np.repeat(np.arange(S, dtype=np.int32), ntiles)
+        first = np.zeros(S + 1, dtype=np.int64)
+        np.cumsum(ntiles, out=first[1:])
+        tile_row0 = ((np.arange(int(first[-1]), dtype=np.int64) - first[:-1][tile_entry]) * size).astype(np.int32)
+        if kind == "big" and tile_entry.shape[0] > 2:
+            # the prefill kernel gives a block the tiles b and n - 1 - b: sorted by the keys they read, blocks are even
+            pos0 = batch.host_array("pos0")[tile_entry].astype(np.int64)
+            last_tok = np.minimum(lens[tile_entry].astype(np.int64), (tile_row0.astype(np.int64) + size + group_size - 1) // group_size)
+            order = np.argsort(-(pos0 + last_tok), kind="stable")
+            tile_entry, tile_row0 = tile_entry[order], tile_row0[order]
+        counts[kind] = int(first[-1])
+        batch.add_array("tile_entry_%s_%d" % (kind, group_size), tile_entry)
+        batch.add_array("tile_row0_%s_%d" % (kind, group_size), tile_row0)
+    batch.shared[note] = counts
+    # the 16-row tiles' keys are split into a number of parts that follows the longest request: a launch shape
+    batch.add_graph_key("attention_key_parts", ops.key_parts_for(batch.max_kv_len))
+
+
+def attention_meta(batch, group: int, group_size: int) -> ops.AttentionMeta:
+    """The step's description for the attention kernels, from the batch's arrays on the device (one object per step,
+    cache group and group size)."""
+    note = ("attention_meta", group, group_size)
+    meta = batch.shared.get(note)
+    if meta is None:
+        tiles = None
+        counts = batch.shared.get(("attention_tiles", group_size))
+        if counts is not None:
+            tiles = {kind: (batch.array("tile_entry_%s_%d" % (kind, group_size)), batch.array("tile_row0_%s_%d" % (kind, group_size)), n)
+                     for kind, n in counts.items()}
+        meta = ops.AttentionMeta(batch.array("cu_q"), batch.array("pos0"), batch.array("kv_len"), batch.block_table(group),
+                                 batch.array("token_entry"), batch.array("positions"), batch.S, batch.T, batch.max_blocks[group],
+                                 batch.max_kv_len, batch.max_q_len, tiles, group_size, fixed_shape=batch.fixed_shape)
+        batch.shared[note] = meta
+    return meta
+
+
 class PagedAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: Optional[PositionEncoding], qk_norm_eps: Optional[float] = None,
-                 window: Optional[int] = None, scale: Optional[float] = None):
+                 window: Optional[int] = None, scale: Optional[float] = None, fold_rows: Optional[int] = None):
+        """``fold_rows``: most rows of a step whose products here run with the norms and the residual sum folded in
+        (None: ``ops.default_fold_rows`` of this part's matrices)."""
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
@@ -33,6 +90,7 @@ class PagedAttention(Mixer):
         self.qk_norm_eps = qk_norm_eps
         self.window = window
         self.scale = 1.0 / math.sqrt(head_dim) if scale is None else float(scale)
+        self.fold_rows = fold_rows
         self.w_qkv = self.w_o = self.q_norm = self.k_norm = self.w_qkv_tiled = self.w_o_tiled = None
 
     # ---- weights ---------------------------------------------------------
@@ -62,11 +120,11 @@ class PagedAttention(Mixer):
         return PagedKV(self.num_kv_heads, self.head_dim, self.window)
 
     def plan(self, batch) -> None:
-        batch.add_attention_tiles(self.num_heads // self.num_kv_heads, ops.prefill_attention_ok(self.head_dim, batch.page_size))
+        plan_attention_tiles(batch, self.num_heads // self.num_kv_heads, ops.prefill_attention_ok(self.head_dim, batch.page_size))
 
     # ---- step ------------------------------------------------------------
     def can_fold(self, batch):
-        return ops.fused_decode_ok(batch.T, batch.act_dtype, self.w_qkv_tiled, self.w_o_tiled)
+        return ops.fused_decode_ok(batch.T, batch.act_dtype, self.w_qkv_tiled, self.w_o_tiled, max_rows=self.fold_rows)
 
     def _attend(self, x, batch, cache, store, for_product=False):
         nq, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
@@ -77,7 +135,7 @@ class PagedAttention(Mixer):
         rot = self.position.rotary() if self.position is not None else None
         cos, sin, rdim = rot if rot is not None else (None, None, 0)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
-        meta = batch.attention_meta(cache.group, nq // nkv)
+        meta = attention_meta(batch, cache.group, nq // nkv)
         if ops.fused_attention_ok(qkv.dtype, meta, nq, nkv, d, cache.page_size, rdim, self.q_norm, self.k_norm):
             # single tokens only: the attention kernel norms, rotates and stores by itself
             raw = ops.RawQKV(qkv, self.q_norm, self.k_norm, eps, cos if rdim else None, sin if rdim else None, store)

@@ -33,8 +33,12 @@ class TokenEmbedding(Part):
 
 
 class LMHead(Part):
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding = None):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding = None, fold_rows: int = 32):
+        """``fold_rows``: most rows for which the head runs as a decode product with the final norm folded in.  Above,
+        the library's product after a norm kernel is faster for a large matrix (measured with 151936 x 4096: 229 / 253 us
+        at 24 / 32 rows against the library's 264 / 269, but 323 against 260 at 48)."""
         self.vocab_size, self.hidden_size, self.tied_to = vocab_size, hidden_size, tied_to
+        self.fold_rows = fold_rows
         self.weight = None
 
     def weight_specs(self, prefix):
@@ -48,11 +52,19 @@ class LMHead(Part):
         self.weight_tiled = ops.tile_weight(self.weight)
 
     def can_fold(self, batch):
-        # above 32 rows the library's product (after a norm kernel) is faster for a matrix of this size (measured with
-        # 151936 x 4096: 229 / 253 us at 24 / 32 rows against the library's 264 / 269, but 323 against 260 at 48)
-        return batch.T <= 32 and ops.fused_decode_ok(batch.T, batch.act_dtype, self.weight_tiled)
+        return ops.fused_decode_ok(batch.T, batch.act_dtype, self.weight_tiled, max_rows=self.fold_rows)
 
-    def forward(self, normed):
+    def logits(self, resid, pending, final_norm, batch, out=None):
+        """The end of a forward pass: ``final_norm`` of the stream (``pending`` as a block leaves it: None, an addend
+        or the prepared input of a norm) at the batch's wanted rows, then the head."""
+        if isinstance(pending, ops.ScaledInput):
+            if pending.norm is final_norm and batch.all_rows_wanted and self.can_fold(batch):
+                return self.forward(pending, out)
+            pending = None                       # the stream is complete
+        return self.forward(final_norm.add_norm(resid, pending, batch.act_dtype, batch.logit_rows), out)
+
+    def forward(self, normed, out=None):
+        """float32 logits [rows, vocab]; written into ``out`` if the caller brings a tensor of that shape."""
         if isinstance(normed, ops.ScaledInput):
-            return ops.decode_linear(normed, self.weight_tiled, torch.float32)
-        return ops.linear(normed, self.weight, torch.float32, tiled=self.weight_tiled)
+            return ops.decode_linear(normed, self.weight_tiled, torch.float32, out)
+        return ops.linear(normed, self.weight, torch.float32, tiled=self.weight_tiled, out=out)

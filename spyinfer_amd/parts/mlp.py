@@ -11,10 +11,13 @@ from .base import FeedForward
 
 
 class GatedMLP(FeedForward):
-    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", fold_rows=None):
+        """``fold_rows``: most rows of a step whose products here run with the norms and the residual sum folded in
+        (None: ``ops.default_fold_rows`` of this part's matrices)."""
         if activation != "silu":
             raise ValueError("GatedMLP: activation %r is not implemented" % activation)
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.fold_rows = fold_rows
         self.w_gate_up = self.w_down = self.w_gate_up_tiled = self.w_down_tiled = None
 
     def weight_specs(self, prefix):
@@ -33,7 +36,7 @@ class GatedMLP(FeedForward):
         self.w_down_tiled = ops.tile_weight(self.w_down)
 
     def can_fold(self, batch):
-        return ops.fused_decode_ok(batch.T, batch.act_dtype, self.w_gate_up_tiled, self.w_down_tiled)
+        return ops.fused_decode_ok(batch.T, batch.act_dtype, self.w_gate_up_tiled, self.w_down_tiled, max_rows=self.fold_rows)
 
     def forward(self, x, batch):
         if isinstance(x, ops.ScaledInput):

@@ -20,3 +20,17 @@ def emu_ops():
     ops.install_test_double(EmuOps())
     yield
     ops.install_test_double(None)
+
+
+@pytest.fixture(autouse=True)
+def poisoned_cache_pool(monkeypatch):
+    """Every cache pool that a test's engine makes is filled with NaN instead of zeros.  A slot is always written
+    before it is read, so a correct engine never shows it; a read of a slot that was never written (a wrong page, a
+    key beyond a request's length that is not masked) turns the logits into NaN instead of passing as a zero."""
+    from spyinfer_amd.cache.storage import CacheStorage
+    real = CacheStorage.__init__
+
+    def init(self, *args, **kwargs):
+        real(self, *args, **kwargs)
+        self.fill(float("nan"))
+    monkeypatch.setattr(CacheStorage, "__init__", init)

@@ -108,9 +108,14 @@ class PlainQwen3:
     """Reads a model folder and runs whole sequences.  Layer order:
     src/models/qwen3.hpp:122-278 (block) and :283-301 (final norm + lm_head)."""
 
-    def __init__(self, folder, compute=torch.float32):
-        with open(os.path.join(folder, "config.json")) as f:
-            c = json.load(f)
+    def __init__(self, folder, compute=torch.float32, config=None, weights=None):
+        """``folder``: a model folder; or None with ``config`` (the config.json keys) and ``weights`` (name -> tensor)
+        given directly, for models that are never written to disk."""
+        if folder is not None:
+            with open(os.path.join(folder, "config.json")) as f:
+                c = json.load(f)
+        else:
+            c = dict(config)
         self.c = c
         self.compute = compute
         self.n_q = c["num_attention_heads"]
@@ -120,7 +125,9 @@ class PlainQwen3:
         self.eps = c.get("rms_norm_eps", 1e-6)
         self.theta = c.get("rope_theta", 1000000.0)
         self.L = c["num_hidden_layers"]
-        self.w = {k: v.to(compute) for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+        if weights is None:
+            weights = load_file(os.path.join(folder, "model.safetensors"))
+        self.w = {k: v.to("cpu", compute) for k, v in weights.items()}
         # src/models/qwen3.hpp:46: a tied model uses the embedding as lm_head
         if c.get("tie_word_embeddings", False):
             self.w["lm_head.weight"] = self.w["model.embed_tokens.weight"]

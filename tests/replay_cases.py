@@ -84,6 +84,34 @@ def mixed(requests, seed=0, max_live=4):
     return steps
 
 
+def trace_properties(steps):
+    """What a trace exercises: (steps that hold a portion of one request beside a single token of a request that has
+    tokens in the cache already, requests admitted after another request ended, most requests live at once)."""
+    fed, ended = {}, 0
+    beside = late = most = 0
+    for st in steps:
+        portion = any(len(e["tokens"]) >= 2 for e in st["entries"])
+        single = any(len(e["tokens"]) == 1 and fed.get(e["id"], 0) > 0 for e in st["entries"])
+        beside += portion and single
+        for e in st["entries"]:
+            if e["id"] not in fed and e["tokens"]:
+                late += ended > 0
+            fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
+        most = max(most, len(fed))
+        for rid in st["end"]:
+            if fed.pop(rid, None) is not None:
+                ended += 1
+    return beside, late, most
+
+
+def assert_mixed(steps, what=""):
+    """A mixed trace must hold what it is for: at least 5 steps with a portion beside a decoded token, requests
+    admitted after others ended (their pages are handed out again), at most four live."""
+    beside, late, most = trace_properties(steps)
+    assert beside >= 5 and late >= 1 and most <= 4, "%s: the mixed trace has %d steps with a portion beside a single token, " \
+        "%d requests admitted after another ended, %d live at once" % (what, beside, late, most)
+
+
 def max_live_tokens(steps, unit=64):
     """Most tokens held at any time, each live request rounded up to a multiple of ``unit``."""
     held, most = {}, 0

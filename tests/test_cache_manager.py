@@ -106,3 +106,45 @@ def test_random_orders_keep_the_invariants(seed):
         m.release(rc)
     m.check()
     assert m.num_free_pages() == [40, 40] and m.slots.num_free == 6
+
+
+def test_a_cache_kind_from_outside_forms_groups_of_its_own():
+    """The manager and the storage ask a kind only what ``CacheKind`` defines: a kind defined here (pages of one float32
+    tensor) is grouped apart from keys and values, gets its own pool and block tables, and its layers get its view."""
+    import dataclasses
+
+    import torch
+
+    from spyinfer_amd.cache import CacheKind
+    from spyinfer_amd.cache.storage import CacheStorage
+
+    @dataclasses.dataclass(frozen=True)
+    class Latent(CacheKind):
+        width: int
+        paged = True
+
+        def page_bytes(self, page_size, act_dtype):
+            return 4 * self.width * page_size
+
+        def allocate(self, num_layers, count, page_size, act_dtype, device):
+            return [torch.zeros((num_layers, count, page_size, self.width), dtype=torch.float32, device=device)]
+
+        def layer_view(self, group, tensors, index, page_size):
+            return ("latent", group, tensors[0][index])
+
+    m = CacheManager([Latent(12), PagedKV(2, 16), Latent(12), FixedState((3,)), Latent(5)], page_size=8, num_pages=6, max_num_seqs=2)
+    assert [g.cache_ids for g in m.page_groups] == [[0, 2], [1], [4]] and [g.cache_ids for g in m.state_groups] == [[3]]
+    st = CacheStorage(m, torch.bfloat16, "cpu")
+    assert [tuple(t.shape) for t in st.tensors] == [(2, 6, 8, 12), (1, 6, 2, 8, 16), (1, 6, 2, 16, 8), (1, 6, 8, 5), (1, 2, 3)]
+    kind, group, view = st.layer(2)
+    assert kind == "latent" and group == 0 and view.data_ptr() == st.tensors[0][1].data_ptr()
+    assert CacheStorage.bytes_per_page([s for s in (Latent(12), PagedKV(2, 16), Latent(12), FixedState((3,)), Latent(5), None)], 8,
+                                       torch.bfloat16) == 4 * 12 * 8 * 2 + 2 * 2 * 16 * 8 * 2 + 4 * 5 * 8
+    rc = m.admit("a")
+    m.reserve(rc, 20)
+    assert [len(t) for t in rc.tables] == [3, 3, 3] and m.num_free_pages() == [3, 3, 3]
+    m.commit(rc, 20)
+    m.release(rc)
+    m.check()
+    with pytest.raises(TypeError, match="CacheKind"):
+        CacheManager([object()], 8, 4, 2)

@@ -159,3 +159,45 @@ def test_steps_run_ahead_change_nothing(folder_a, emu_ops):
     assert used >= 15, "steps of decoded tokens alone must have been launched ahead (%d were)" % used
     assert out_a[0] == g1[:k + 1]                              # the second request ended at its end token
     assert out_a[1] == plain.greedy(ps[2], 7) and out_a[2] == plain.greedy(ps[3], 9)
+
+
+def test_config_b_workload_against_plain_model_and_plain_sampler(folder_b, emu_ops):
+    """Prompts of 1 / 40 / 130 tokens in portions of 32 beside decoding requests, pages of 8: greedy tokens equal the
+    plain implementation's, and tokens sampled at temperature 0.8 equal the plain sampler's on the plain logits (so the
+    index of a draw, run-ahead steps included, and the seed of a request are the stated ones)."""
+    from tests.workloads import run_config_b_workload
+    run_config_b_workload(folder_b, PlainQwen3(folder_b), "cpu", "float32")
+
+
+def test_refused_turn_leaves_the_request_as_it_was_and_draws_go_on(folder_a, emu_ops):
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from tests.workloads import check_sampled_against_plain
+    plain = PlainQwen3(folder_a)
+    p = prompts(256, [12])[0]
+    sp = SamplingParams(temperature=0.9, max_new_tokens=5, ignore_eos=True, seed=77)
+    for keep in (False, True):
+        eng = LLMEngine(folder_a, dtype="float32", device="cpu", max_model_len=40, num_kvcache_blocks=8, keep_finished_cache=keep)
+        rid = eng.add_request(p, sp)
+        while not eng.is_request_finished(rid):
+            eng.step()
+        first = eng.get_generated_tokens(rid)
+        history = eng.get_output_tokens(rid)
+        with pytest.raises(ValueError, match="max_model_len"):
+            eng.append_to_request(rid, [1] * 30)                       # 12 + 5 + 30 > 40
+        with pytest.raises(ValueError, match="vocabulary"):
+            eng.append_to_request(rid, [3, 999])
+        assert eng.is_request_finished(rid) and eng.get_output_tokens(rid) == history and eng.get_generated_tokens(rid) == first
+        prefill_before = eng.stats["prefill_tokens"]
+        eng.append_to_request(rid, [7, 8, 9])
+        while not eng.is_request_finished(rid):
+            eng.step()
+        second = eng.get_generated_tokens(rid)
+        # the second turn computes its new tokens only if the cache was kept, the whole history otherwise
+        assert eng.stats["prefill_tokens"] - prefill_before == (4 if keep else len(history) + 3)
+        # its draws go on where the first turn's ended (indices 5..9 of the same seed), checked with the plain sampler
+        check_sampled_against_plain(plain, [p], [first], 0.9, [77], 1e-4)
+        compared, _ = check_sampled_against_plain(plain, [history + [7, 8, 9]], [second], 0.9, [77], 1e-4, first_draw=5)
+        assert compared >= 4
+        eng.remove_request(rid)
+        eng.runner.manager.check()
+        assert eng.runner.manager.num_free_pages() == [8] and eng.runner.manager.slots.num_free == eng.config.max_num_seqs

@@ -18,7 +18,7 @@ def folders(tmp_path_factory):
     return out
 
 
-CASES = {"A": (TINY_A, [5, 17, 33, 60]), "B": (TINY_B, [1, 40, 130]), "C": (TINY_C, [3, 70, 200, 45, 64, 97])}
+CASES = {"A": (TINY_A, [5, 17, 33, 60, 44, 23, 9, 51]), "B": (TINY_B, [1, 40, 130, 75, 12, 100, 33]), "C": (TINY_C, [3, 70, 200, 45, 64, 97])}
 
 
 @pytest.mark.parametrize("name", ["A", "B", "C"])
@@ -27,6 +27,8 @@ def test_cuts_match_plain(name, mode, folders, tmp_path, emu_ops):
     cfg, lengths = CASES[name]
     reqs = rc.random_requests(cfg["vocab_size"], lengths, seed=3)
     steps = getattr(rc, mode)(reqs)
+    if mode == "mixed":
+        rc.assert_mixed(steps, name)
     max_tokens = rc.max_live_tokens(steps)
     page = {"A": 16, "B": 8, "C": 16}[name]
     rc.run_replay_inprocess(folders[name], "float32", str(tmp_path), steps, max_tokens,
@@ -58,3 +60,49 @@ def test_replay_lines_without_tokens_and_names_used_again(folders, tmp_path, emu
     assert not (tmp_path / "3.f32").exists()
     for got, ref in ((read(0, 1), ra[[9]]), (read(1, 1), rb[[8]]), (read(2, 1), ra[[20]]), (read(4, 2), rb[[0, 8]])):
         assert torch.allclose(got, ref, atol=2e-4, rtol=2e-4)
+
+
+def test_cache_pool_is_sized_after_the_memory_of_captured_steps():
+    """With graphs the pool is sized from what is left after the one logits tensor [max_num_seqs, vocab] and the
+    metadata buffers of every captured step; with enforce_eager from all the free memory; never beyond what
+    max_num_seqs requests of max_model_len tokens need."""
+    from spyinfer_amd.config.engine_config import EngineConfig
+    from spyinfer_amd.config.registry import architecture_of
+    from spyinfer_amd.engine.llm_engine import pages_for_memory
+    from spyinfer_amd.engine.runner import ModelRunner
+    arch = architecture_of(TINY_B)
+    model = arch.build(arch.config_cls.from_dict(TINY_B))
+    per_page = 3 * 2 * 2 * 32 * 8 * 2                                     # layers, K and V, kv heads, head_dim, page, bfloat16
+    assert ModelRunner.bytes_per_page(model, 8, "bfloat16") == per_page
+    assert ModelRunner.bytes_per_page(model, 8, "float32") == 2 * per_page
+    cfg = EngineConfig(max_num_seqs=64, max_model_len=512, kvcache_block_size=8, gpu_memory_utilization=0.5, enforce_eager=True)
+    free = 40 << 20
+    assert pages_for_memory(free, cfg, model) == int(free * 0.5 * 0.9) // per_page
+    cfg.enforce_eager = False
+    logits = 4 * 64 * 384
+    meta = ModelRunner.MAX_GRAPHS * 4 * (64 * (1 * 64 + 64) + 256)        # one page group, 512 / 8 = 64 pages per request
+    assert ModelRunner.graph_logits_bytes(64, 384) == logits
+    assert ModelRunner.MAX_GRAPHS * ModelRunner.graph_metadata_bytes(64, 1, 64) == meta
+    assert pages_for_memory(free, cfg, model) == int((free - logits - meta) * 0.5 * 0.9) // per_page
+    assert pages_for_memory(1 << 20, cfg, model) == 1                       # less free memory than the graphs take: one page, no negative count
+    cfg.gpu_memory_utilization = 1.0
+    assert pages_for_memory(1 << 40, cfg, model) == 64 * 64                 # the cap
+
+
+def test_a_step_metadata_fits_the_bound_used_for_captured_steps(folders, emu_ops):
+    """The per-entry bound of a captured step's metadata (a row of page numbers per page group and 64 further integers)
+    holds for real decode batches with fixed-width block tables."""
+    from spyinfer_amd.engine.batch import StepBatch, StepEntry
+    from spyinfer_amd.engine.runner import ModelRunner, load_model
+    model = load_model(folders["B"], "float32", "cpu")
+    runner = ModelRunner(model, "float32", "cpu", 8, 64, 6, max_model_len=128)
+    caches = [runner.manager.admit(i) for i in range(6)]
+    for n, c in enumerate(caches):
+        runner.manager.reserve(c, 3 + 7 * n)
+        runner.manager.commit(c, 3 + 7 * n)
+        runner.manager.reserve(c, 1)
+    for live in (1, 3, 6):
+        batch = StepBatch([StepEntry(c, [5], [0]) for c in caches[:live]], runner.manager, torch.float32, "cpu", 384, runner.fixed_max_blocks)
+        model.plan(batch)
+        _layout, total = batch.layout()
+        assert 4 * total <= ModelRunner.graph_metadata_bytes(live, 1, runner.fixed_max_blocks)

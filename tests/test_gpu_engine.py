@@ -125,6 +125,77 @@ def test_random_arrivals_endings_and_removals(folder_a, seed):
     assert eng.runner.graph_replays > 0
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("eager", [True, False])
+def test_config_b_workload(tmp_path_factory, dtype, eager):
+    """The second tiny configuration's workload through the entry point on the GPU: prompts of 1 / 40 / 130 tokens in
+    portions of 32 beside decoding requests, pages of 8, 24 tokens each; greedy tokens against the plain implementation,
+    sampled tokens against the plain sampler on the plain logits."""
+    from spyinfer_amd.weights import write_random_model
+    from tests.workloads import run_config_b_workload
+    require_gpu()
+    folder = write_random_model(str(tmp_path_factory.mktemp("eng_b")), TINY_B, 32, torch.bfloat16, **INIT)
+    run_config_b_workload(folder, PlainQwen3(folder), "cuda:0", dtype, enforce_eager=eager)
+
+
+def test_captured_steps_share_their_memory():
+    """Decode steps of 40 and more shapes (batch sizes times numbers of key parts) at a real width and vocabulary are
+    captured as graphs into one memory pool with one logits tensor: the memory that torch holds grows by the metadata
+    buffers and the activations of the largest step, not by a pool and a logits tensor per graph."""
+    from spyinfer_amd.config.registry import architecture_of
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.runner import ModelRunner
+    from spyinfer_amd.weights.random_init import random_tensors_on_device
+    dev = require_gpu()
+    V = 151936
+    raw = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_act="silu", num_hidden_layers=2, hidden_size=4096,
+               num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=V,
+               rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=4096)
+    arch = architecture_of(raw)
+    model = arch.build(arch.config_cls.from_dict(raw))
+    model.bind(random_tensors_on_device(model.weight_specs(), 3, torch.bfloat16, dev), dev)
+    per, targets = 24, (100, 300, 550, 800)               # four groups of requests: 1, 2, 3 and 4 key parts
+    R = per * len(targets)
+    runner = ModelRunner(model, "bfloat16", dev, 16, 3000, R, enforce_eager=False, max_model_len=2048)
+    eager = ModelRunner(model, "bfloat16", dev, 16, 3000, R, enforce_eager=True, max_model_len=2048)
+    g = torch.Generator().manual_seed(1)
+    caches = {r: [r.manager.admit(i) for i in range(R)] for r in (runner, eager)}
+
+    def step(r, ids, tokens):
+        for i, t in zip(ids, tokens):
+            r.manager.reserve(caches[r][i], len(t))
+        return r.step([StepEntry(caches[r][i], t, [len(t) - 1]) for i, t in zip(ids, tokens)])
+
+    for k, target in enumerate(targets):                   # all prompts first, 12 requests a step
+        for half in (0, 1):
+            ids = list(range(k * per + half * 12, k * per + half * 12 + 12))
+            fill = [torch.randint(0, V, (target,), generator=g).tolist() for _ in ids]
+            for r in (runner, eager):
+                step(r, ids, fill)
+    base = None
+    for k, target in enumerate(targets):
+        for live in (1, 2, 3, 5, 8, 9, 12, 16, 17, 20, 24):
+            ids = list(range(k * per, k * per + live))
+            for rep in range(2):                           # a shape is captured at its second step
+                toks = [[int(t)] for t in torch.randint(0, V, (live,), generator=g)]
+                a, b = step(runner, ids, toks), step(eager, ids, toks)
+                assert torch.allclose(a, b, atol=2e-2, rtol=2e-2), "graph and eager logits differ (%d requests near %d tokens)" % (live, target)
+            if base is None:
+                torch.cuda.synchronize()
+                base = torch.cuda.memory_reserved(dev)     # after the first capture: the pool and the logits tensor exist
+    torch.cuda.synchronize()
+    shapes = len(runner._graphs)
+    grown = torch.cuda.memory_reserved(dev) - base
+    assert shapes >= 40 and runner.graph_replays >= 40, (shapes, runner.graph_replays)
+    assert runner._graph_logits.shape == (R, V)
+    # 43 more graphs after the first.  With a pool of its own each would hold its logits (0.6 to 14.6 MB) in allocator
+    # segments of 20 MB at least: more than 860 MB.  Shared, they add their metadata buffers and the activations of the
+    # largest step (24 rows: a few MB), which the allocator rounds up to segments.
+    bound = shapes * ModelRunner.graph_metadata_bytes(per, 1, runner.fixed_max_blocks) + (128 << 20)
+    assert grown <= bound, "captured steps grew torch's memory by %d bytes for %d shapes (bound %d)" % (grown, shapes, bound)
+    assert runner.graph_memory_bound() >= 4 * R * V
+
+
 def test_number_of_graphs_is_bounded(folder_a):
     """The runner captures a bounded number of step shapes (each captured step holds its activations); with room for
     two, a run whose batch shrinks from four requests to one runs its later shapes kernel by kernel and still gives
@@ -264,8 +335,8 @@ def test_folded_decode_steps(tmp_path_factory):
 def test_folded_decode_steps_of_many_requests(tmp_path_factory, requests):
     """Decode steps of 17 to 64 requests take the folded products with two to four row tiles (70 requests: the library's); their logits equal, up to
     bfloat16 rounding, those of the same steps with the norms as kernels of their own, from graphs as well, and the last
-    step's equal the plain implementation's.  Parts with large matrices fold up to 48 rows only (the limit is made tiny
-    here): the embedding then still prepares the first norm's input, which the unfolded block does not use."""
+    step's equal the plain implementation's.  Parts may be built to fold up to fewer rows (48 here, as parts with large
+    matrices are): the embedding then still prepares the first norm's input, which the unfolded block does not use."""
     from spyinfer_amd.engine.batch import StepEntry
     from spyinfer_amd.engine.runner import ModelRunner, load_model
     from spyinfer_amd.kernels import ops
@@ -277,9 +348,11 @@ def test_folded_decode_steps_of_many_requests(tmp_path_factory, requests):
     ps = prompts(400, [3 + (7 * i) % 23 for i in range(requests)], 5)
     runs, calls = [], []
     real = ops.decode_linear_residual
-    wide = ops.FUSED_DECODE_WIDE_MAX_ELEMS
-    for folded, eager, elems in ((True, True, wide), (True, False, wide), (False, True, wide), (True, True, 1000)):
-        ops.FUSED_DECODE, ops.FUSED_DECODE_WIDE_MAX_ELEMS = folded, elems
+    assert ops.default_fold_rows(1 << 20) == 64 and ops.default_fold_rows((1 << 28) + 1) == 48
+    for folded, eager, fold_rows in ((True, True, None), (True, False, None), (False, True, None), (True, True, 48)):
+        ops.FUSED_DECODE = folded
+        for layer in model.layers:
+            layer.mixer.fold_rows = layer.ffn.fold_rows = fold_rows
         n = [0]
         ops.decode_linear_residual = lambda *a, **k: (n.__setitem__(0, n[0] + 1), real(*a, **k))[1]
         try:
@@ -300,14 +373,14 @@ def test_folded_decode_steps_of_many_requests(tmp_path_factory, requests):
             runs.append(outs)
             calls.append(n[0])
         finally:
-            ops.FUSED_DECODE, ops.FUSED_DECODE_WIDE_MAX_ELEMS = True, wide
+            ops.FUSED_DECODE = True
             ops.decode_linear_residual = real
     if requests <= ops.FUSED_DECODE_MAX_ROWS:
-        assert calls[0] >= 5 * 2 * 3 and calls[2] == 0 and (calls[3] == 0) == (requests > ops.FUSED_DECODE_WIDE_ROWS)
+        assert calls[0] >= 5 * 2 * 3 and calls[2] == 0 and (calls[3] == 0) == (requests > 48)
     else:
         assert calls == [0, 0, 0, 0]          # more rows than the folded products take: the library's, with norm kernels
     for i, (a, b, c, e) in enumerate(zip(*runs)):
-        for x, what in ((b, "graphs"), (c, "plain norms"), (e, "large matrices")):
+        for x, what in ((b, "graphs"), (c, "plain norms"), (e, "parts that fold up to 48 rows")):
             assert a.shape == x.shape and torch.allclose(a, x, **TOL["bfloat16"]), "step %d: folded and %s differ by %g" % (
                 i, what, (a - x).abs().max())
     ref = torch.stack([plain.forward(q)[-1] for q in seqs])

@@ -437,6 +437,83 @@ def test_paged_attention(dtype, case, mfma):
     close(out, ref, dtype, scale=2.0, what="attention case %d" % case)
 
 
+def _long_case(dtype, dev, n_q, n_kv, d, P, entries, seed):
+    """As make_attention_case, for thousands of keys: filled and gathered with tensor operations.  Returns also the
+    keys and values of each entry in order, for the reference."""
+    from spyinfer_amd.kernels.ops import AttentionMeta
+    g = torch.Generator().manual_seed(seed)
+    total_pages = sum(-(-(a + n) // P) for a, n in entries) + 5
+    order = torch.randperm(total_pages, generator=g)
+    kc = torch.full((total_pages, n_kv, P, d), float("nan"), dtype=dtype)
+    vc = torch.full((total_pages, n_kv, d, P), float("nan"), dtype=dtype)
+    maxb = max(-(-(a + n) // P) for a, n in entries)
+    bt = torch.full((len(entries), maxb), -1, dtype=torch.int64)
+    cu, used, kept = [0], 0, []
+    for s, (a, n) in enumerate(entries):
+        L, nb = a + n, -(-(a + n) // P)
+        bt[s, :nb] = order[used:used + nb]
+        used += nb
+        K, V = torch.randn(L, n_kv, d, generator=g).to(dtype), torch.randn(L, n_kv, d, generator=g).to(dtype)
+        kept.append((K, V))
+        cu.append(cu[-1] + n)
+    q = torch.randn(cu[-1], n_q * d, generator=g).to(dtype)
+    for s, (a, n) in enumerate(entries):
+        K, V = kept[s]
+        # far keys that the last query of the entry scores high: one near the start, one at a page's first slot deep inside
+        for c in (3, ((a + n) // 2) // P * P):
+            for h in range(n_q):
+                K[c, h * n_kv // n_q] = (q[cu[s + 1] - 1].view(n_q, d)[h].float() * 1.2).to(dtype)
+        c = torch.arange(a + n)
+        kc[bt[s][c // P], :, c % P, :] = K
+        vc[bt[s][c // P], :, :, c % P] = V
+    G = n_q // n_kv
+    i32 = lambda x: torch.as_tensor(x, dtype=torch.int32).to(dev)
+    tiles = {}
+    for kind, size in (("small", 16), ("big", 128)):
+        te, tr = [], []
+        for s, (a, n) in enumerate(entries):
+            if (n * G >= 64) == (kind == "big"):
+                te += [s] * len(range(0, n * G, size)); tr += list(range(0, n * G, size))
+        if kind == "big":                       # sorted by the keys read, most first, as the engine does
+            keys = [entries[s][0] + min(entries[s][1], (r0 + size + G - 1) // G) for s, r0 in zip(te, tr)]
+            idx = sorted(range(len(te)), key=lambda i: -keys[i])
+            te, tr = [te[i] for i in idx], [tr[i] for i in idx]
+        tiles[kind] = (i32(te), i32(tr), len(te))
+    token_entry = [s for s, (a, n) in enumerate(entries) for _ in range(n)]
+    positions = [a + i for a, n in entries for i in range(n)]
+    meta = AttentionMeta(i32(cu), i32([a for a, n in entries]), i32([a + n for a, n in entries]), i32(bt), i32(token_entry),
+                         i32(positions), len(entries), cu[-1], maxb, max(a + n for a, n in entries), max(n for _, n in entries), tiles, G)
+    return q, kc, vc, kept, cu, meta
+
+
+@pytest.mark.parametrize("case", [(32, 8, 128, 16, [(9000, 1), (8191, 1), (4000, 1)]),        # 16 key parts and the merge
+                                  (8, 2, 128, 16, [(8800, 200), (0, 300)]),                   # few 128-row tiles far into a request: key parts
+                                  (16, 2, 64, 32, [(9100, 70), (5000, 1)])])                   # both kernels in one step
+def test_paged_attention_over_9000_keys(case):
+    """The lengths that the benchmarks run (15 000-key decode steps, portions late in 16 000-token prompts): block tables
+    of hundreds of pages, the most key parts, tiles sorted by work.  Reference: float64 softmax over the entry's keys."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    n_q, n_kv, d, P, entries = case
+    dtype = torch.bfloat16
+    q, kc, vc, kept, cu, meta = _long_case(dtype, dev, n_q, n_kv, d, P, entries, seed=len(entries) + n_q)
+    assert ops.key_parts_for(meta.max_kv_len) == 16
+    scale = 1.0 / math.sqrt(d)
+    out = ops.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), P, meta, n_q, n_kv, d, scale, None).cpu().double()
+    for s, (a, n) in enumerate(entries):
+        K, V = (x.double() for x in kept[s])
+        qs = q[cu[s]:cu[s + 1]].double().view(n, n_q, d)
+        kv_of = torch.arange(n_q) * n_kv // n_q
+        scores = torch.einsum("thd,chd->thc", qs, K[:, kv_of]) * scale
+        masked = torch.arange(a + n)[None, :] > (a + torch.arange(n))[:, None]
+        pr = torch.softmax(scores.masked_fill(masked[:, None, :], float("-inf")), dim=-1)
+        ref = torch.einsum("thc,chd->thd", pr, V[:, kv_of]).reshape(n, n_q * d)
+        # the far keys carry weight: for the last query head of a group (whose query the keys were made from) the
+        # largest probability of the entry's last token lies on one of them
+        assert int(pr[-1, n_q // n_kv - 1].argmax()) in (3, ((a + n) // 2) // P * P)
+        close(out[cu[s]:cu[s + 1]], ref, dtype, scale=2.0, what="entry %d of %r" % (s, entries))
+
+
 FUSED_CASES = [
     # n_q, n_kv, d, P, cached tokens of each single-token entry, window, norm, rotation
     (32, 8, 128, 16, [1151, 70, 2000, 0, 15, 16, 31, 32], None, True, True),

@@ -17,8 +17,11 @@ from tests.plain.qwen3_plain import PlainQwen3
 
 pytestmark = pytest.mark.gpu
 
-CASES = {"A": (TINY_A, [5, 17, 33, 60], 16), "B": (TINY_B, [1, 40, 130], 8), "C": (TINY_C, [3, 70, 200, 45, 64, 97, 333], 16),
-         "D": (TINY_D, [9, 50, 190, 77, 300], 16), "E": (TINY_E, [2, 130, 425, 61], 16)}
+# the first requests of A and B are the workloads of those configurations; the further ones are there so that the mixed
+# trace admits requests after others have ended (four are live at most)
+CASES = {"A": (TINY_A, [5, 17, 33, 60, 44, 23, 9, 51], 16), "B": (TINY_B, [1, 40, 130, 75, 12, 100, 33], 8),
+         "C": (TINY_C, [3, 70, 200, 45, 64, 97, 333], 16), "D": (TINY_D, [9, 50, 190, 77, 300, 21], 16),
+         "E": (TINY_E, [2, 130, 425, 61, 90, 17], 16)}
 # float32: only the order of sums differs.  bfloat16: activations are rounded to 8 bits between
 # kernels; with these weights the CPU model of that rounding differs from float32 by up to 0.04
 # on logits of standard deviation 0.7, hence twice that as the absolute tolerance.
@@ -49,11 +52,52 @@ def test_replay_matches_plain(dtype, name, mode, models, tmp_path, monkeypatch):
     cfg, lengths, page = CASES[name]
     folder, reqs, ref = models[name]
     steps = getattr(rc, mode)(reqs)
+    handed_out = _count_pages_handed_out(monkeypatch)
+    if mode == "mixed":
+        rc.assert_mixed(steps, name)         # portions beside decoded tokens, requests admitted after others ended
     rc.run_replay_inprocess(folder, dtype, str(tmp_path), steps, rc.max_live_tokens(steps), ["--kvcache-block-size", str(page)])
     got = rc.collect(str(tmp_path), steps, cfg["vocab_size"])
     rc.compare(got, ref, what="%s/%s/%s" % (name, mode, dtype), **TOL[dtype])
+    if mode != "whole" or len(lengths) > 1:
+        assert max(handed_out.values()) >= 2, "no page of the pool was handed out a second time"
     # configurations D and E in bfloat16 are there for the decode products with folded norms: they must have run
     assert bool(folded) == (name in "DE" and dtype == "bfloat16")
+
+
+def _count_pages_handed_out(monkeypatch):
+    """{page: times it was handed out} over all pools made from now on."""
+    from spyinfer_amd.cache.pages import PagePool
+    count = {}
+    real = PagePool.allocate
+
+    def allocate(self):
+        page = real(self)
+        count[page] = count.get(page, 0) + 1
+        return page
+    monkeypatch.setattr(PagePool, "allocate", allocate)
+    return count
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "E"])
+def test_page_numbering_does_not_matter(dtype, name, models, tmp_path, monkeypatch):
+    """The mixed trace on a pool whose free list was shuffled: requests get pages in no order at all, pages handed out
+    again come back in another order, and the logits are those of the plain implementation all the same."""
+    import random
+    require_gpu()
+    from spyinfer_amd.cache.pages import PagePool
+    real = PagePool.__init__
+
+    def shuffled(self, num_pages):
+        real(self, num_pages)
+        random.Random(num_pages).shuffle(self._free)
+    monkeypatch.setattr(PagePool, "__init__", shuffled)
+    cfg, lengths, page = CASES[name]
+    folder, reqs, ref = models[name]
+    steps = rc.mixed(reqs, seed=3)
+    rc.assert_mixed(steps, name)
+    rc.run_replay_inprocess(folder, dtype, str(tmp_path), steps, rc.max_live_tokens(steps), ["--kvcache-block-size", str(page)])
+    rc.compare(rc.collect(str(tmp_path), steps, cfg["vocab_size"]), ref, what="shuffled/%s/%s" % (name, dtype), **TOL[dtype])
 
 
 @pytest.fixture(scope="module")
@@ -107,9 +151,10 @@ def test_trace_run_program(dtype, models, tmp_path):
     cfg, lengths, page = CASES["B"]
     folder, reqs, ref = models["B"]
     steps = rc.mixed(reqs, seed=7)
+    rc.assert_mixed(steps, "B")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out",
-                        str(tmp_path), "--max-tokens", str(rc.max_live_tokens(steps))],
+                        str(tmp_path), "--max-tokens", str(rc.max_live_tokens(steps)), "--poison-cache"],
                        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
     assert p.returncode == 0, p.stderr[-2000:]
     assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done %d" % s["step"] for s in steps]

@@ -199,3 +199,138 @@ def test_toy_parts_and_shared_cache(dtype, tmp_path):
         assert not torch.allclose(shifted[5:], shifted[:5], atol=1e-2)
     finally:
         unregister_architecture("ToyRoutedLM")
+
+
+# ---------------------------------------------------------------------------------------------
+# A third kind of cache, defined here: one float32 tensor per group, a token's vector per page slot
+# (another layout, another dtype, one tensor instead of two), and a mixer that reads it through the
+# request's block table.
+
+def _toy_latent():
+    from spyinfer_amd.cache import CacheKind
+    from spyinfer_amd.config import ModelConfig
+    from spyinfer_amd.models import DecoderModel
+    from spyinfer_amd.parts import GatedMLP, LMHead, PagedAttention, PreNormBlock, RMSNorm, RotaryEmbedding, TokenEmbedding
+    from spyinfer_amd.parts.base import Mixer
+    from spyinfer_amd.weights import WeightSpec
+
+    class LatentLayer:
+        def __init__(self, group, rows, page_size):
+            self.group, self.rows, self.page_size = group, rows, page_size     # rows: [pages * page, width] float32
+
+    @dataclasses.dataclass(frozen=True)
+    class PagedLatent(CacheKind):
+        """One float32 vector of ``width`` per token, in pages: ``[layers, pages, page, width]``."""
+        width: int
+        paged = True
+
+        def page_bytes(self, page_size, act_dtype):
+            return 4 * self.width * page_size
+
+        def allocate(self, num_layers, count, page_size, act_dtype, device):
+            return [torch.zeros((num_layers, count, page_size, self.width), dtype=torch.float32, device=device)]
+
+        def layer_view(self, group, tensors, index, page_size):
+            return LatentLayer(group, tensors[0][index].view(-1, self.width), page_size)
+
+    class PagedMean(Mixer):
+        """out[t] = gain * mean of the request's inputs at positions 0..t, every input kept in the paged cache."""
+
+        def __init__(self, hidden):
+            self.hidden = hidden
+
+        def weight_specs(self, prefix):
+            return [WeightSpec(prefix + ".gain", (self.hidden,), "norm")]
+
+        def bind(self, prefix, weights):
+            self.gain = weights[prefix + ".gain"]
+
+        def cache_spec(self):
+            return PagedLatent(self.hidden)
+
+        def forward(self, x, batch, cache, store=True):
+            if store:
+                cache.rows[batch.slot_mapping(cache.group).long()] = x.float()
+            table = batch.block_table(cache.group).long()                      # [S, max_blocks]
+            P = cache.page_size
+            out = torch.empty_like(x)
+            lens, pos0 = batch.lens, batch.host_array("pos0")
+            t0 = 0
+            for s in range(batch.S):
+                n, first = int(lens[s]), int(pos0[s])
+                pos = torch.arange(first + n, device=x.device)
+                rows = cache.rows[table[s][pos // P] * P + pos % P]            # every input of the request so far
+                sums = torch.cumsum(rows, 0)[first:]
+                out[t0:t0 + n] = (sums / (pos[first:] + 1).float()[:, None] * self.gain.float()).to(x.dtype)
+                t0 += n
+            return out
+
+    @dataclasses.dataclass
+    class ToyConfig(ModelConfig):
+        hidden_size: int = 0
+        vocab_size: int = 0
+        intermediate_size: int = 0
+
+    def build(cfg):
+        H = cfg.hidden_size
+        emb, rope = TokenEmbedding(cfg.vocab_size, H), RotaryEmbedding(16, 10000.0)
+        mixers = [PagedMean(H), PagedAttention(H, 4, 2, 16, rope), PagedMean(H)]
+        layers = [PreNormBlock(RMSNorm(H, 1e-5), m, RMSNorm(H, 1e-5), GatedMLP(H, cfg.intermediate_size)) for m in mixers]
+        return DecoderModel(cfg, emb, rope, layers, RMSNorm(H, 1e-5), LMHead(cfg.vocab_size, H, tied_to=emb), max_positions=256)
+
+    return ToyConfig, build, PagedLatent
+
+
+def plain_latent_forward(folder, tokens):
+    cfg = json.load(open(os.path.join(folder, "config.json")))
+    w = {k: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    T = len(tokens)
+    cos, sin = P.rope_tables(T, 16, 10000.0)
+    pos = torch.arange(T)
+    h = P.embedding(torch.tensor(tokens), w["model.embed_tokens.weight"])
+    for i in range(3):
+        p = "model.layers.%d." % i
+        n1 = P.rms_norm(h, w[p + "input_layernorm.weight"], 1e-5)
+        if i == 1:
+            q = P.rope_apply(P.linear(n1, w[p + "self_attn.q_proj.weight"]).view(T, 4, 16), pos, cos, sin)
+            k = P.rope_apply(P.linear(n1, w[p + "self_attn.k_proj.weight"]).view(T, 2, 16), pos, cos, sin)
+            v = P.linear(n1, w[p + "self_attn.v_proj.weight"]).view(T, 2, 16)
+            a = P.linear(P.attention(q, k, v).reshape(T, -1), w[p + "self_attn.o_proj.weight"])
+        else:
+            a = torch.cumsum(n1, 0) / (pos + 1).float()[:, None] * w[p + "self_attn.gain"]
+        h = h + a
+        n2 = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], 1e-5)
+        h = h + P.linear(P.swiglu(P.linear(n2, w[p + "mlp.gate_proj.weight"]), P.linear(n2, w[p + "mlp.up_proj.weight"])),
+                         w[p + "mlp.down_proj.weight"])
+    return P.linear(P.rms_norm(h, w["model.norm.weight"], 1e-5), w["model.embed_tokens.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_third_kind_of_cache_defined_in_a_test(dtype, tmp_path):
+    """The cache manager groups, the storage allocates and the step hands out a kind of cache that the framework does
+    not know: pages of one float32 tensor, with a pool and block tables apart from the attention layer's keys and values."""
+    from spyinfer_amd.config import register_architecture, unregister_architecture
+    from spyinfer_amd.engine.runner import ModelRunner, load_model
+    from spyinfer_amd.weights import write_random_model
+    dev = require_gpu()
+    ToyConfig, build, PagedLatent = _toy_latent()
+    register_architecture("ToyLatentLM", ToyConfig, build)
+    try:
+        cfg = dict(architectures=["ToyLatentLM"], hidden_size=64, vocab_size=101, intermediate_size=96)
+        folder = write_random_model(str(tmp_path / "toy"), cfg, 91, torch.bfloat16, **INIT)
+        runner = ModelRunner(load_model(folder, dtype, dev), dtype, dev, 16, 8, 2)
+        groups = runner.manager.page_groups
+        assert [g.cache_ids for g in groups] == [[0, 2], [1]] and groups[0].spec == PagedLatent(64)
+        elem = 2 if dtype == "bfloat16" else 4
+        assert ModelRunner.bytes_per_page(runner.model, 16, dtype) == 2 * 4 * 64 * 16 + 2 * 2 * 16 * 16 * elem
+        assert [tuple(t.shape) for t in runner.storage.tensors] == [(2, 8, 16, 64), (1, 8, 2, 16, 16), (1, 8, 2, 16, 16)]
+        assert runner.storage.tensors[0].dtype == torch.float32
+        reqs = rc.random_requests(101, [70, 9, 41, 120, 33], seed=12)
+        ref = {rid: plain_latent_forward(folder, t) for rid, t in reqs.items()}
+        for mode in ("whole", "bulk_tail", "portions", "mixed"):
+            steps = getattr(rc, mode)(reqs)
+            out = str(tmp_path / mode)
+            rc.run_replay_inprocess(folder, dtype, out, steps, rc.max_live_tokens(steps))
+            rc.compare(rc.collect(out, steps, 101), ref, what="latent/%s/%s" % (mode, dtype), **TOL[dtype])
+    finally:
+        unregister_architecture("ToyLatentLM")

@@ -130,3 +130,68 @@ def test_tied_head(tmp_path):
     m = P.PlainQwen3(write_random_model(str(tmp_path / "a"), TINY_A, 42, torch.bfloat16, **INIT))
     assert m.w["lm_head.weight"] is m.w["model.embed_tokens.weight"]
     assert m.forward([3, 4]).shape == (2, 256)
+
+
+# ---- the whole pass against a second, independent transcription ---------------------------------------------------
+@pytest.fixture(scope="module")
+def anchor_folders(tmp_path_factory):
+    from spyinfer_amd.weights import write_random_model
+    from tests.configs import TINY_C
+    return {name: write_random_model(str(tmp_path_factory.mktemp("anchor_" + name)), cfg, seed, torch.bfloat16, **INIT)
+            for name, cfg, seed in (("A", TINY_A, 41), ("B", TINY_B, 42), ("C", TINY_C, 43))}
+
+
+@pytest.mark.parametrize("name,length", [("A", 23), ("B", 37), ("C", 19)])
+def test_whole_pass_equals_the_second_transcription(anchor_folders, name, length):
+    """``qwen3_plain`` (CPU backend's formulas, whole sequences, torch) and ``qwen3_second`` (CUDA backend's formulas,
+    the model's operation list token by token over growing key/value lists, numpy float64) give the same logits at every
+    position.  The installed ``transformers`` package also holds a Qwen3 and would be a third anchor; model code of
+    installed packages is not a source for this project, so it is neither imported nor read."""
+    from tests.plain.qwen3_second import SecondQwen3
+    vocab = {"A": 256, "B": 384, "C": 331}[name]
+    toks = torch.randint(0, vocab, (length,), generator=torch.Generator().manual_seed(3)).tolist()
+    first = P.PlainQwen3(anchor_folders[name], compute=torch.float64).forward(toks).numpy()
+    second = SecondQwen3(anchor_folders[name]).forward(toks)
+    assert first.shape == second.shape
+    # float64 both; the second forms its rotation angles in float32 as the reference's table does, the first (asked for
+    # float64) in float64: 2e-7 on the logits, none at position 0
+    assert abs(first - second).max() < 1e-6, abs(first - second).max()
+    assert abs(first[0] - second[0]).max() < 1e-12
+
+
+def _small_queries(folder, dst, factor):
+    """The model of ``folder`` with its q and k projections scaled down, so that the mean square of a head vector
+    comes near the norms' eps and the eps of the q/k norm shows in the logits."""
+    import json
+    import os
+    import shutil
+
+    from safetensors.torch import load_file
+
+    from spyinfer_amd.weights import write_file
+    os.makedirs(dst, exist_ok=True)
+    shutil.copy(os.path.join(folder, "config.json"), os.path.join(dst, "config.json"))
+    w = {k: v.clone() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    for k in w:
+        if k.endswith("q_proj.weight") or k.endswith("k_proj.weight"):
+            w[k] = (w[k].float() * factor).to(torch.bfloat16)
+    write_file(os.path.join(dst, "model.safetensors"), w)
+    return dst
+
+
+@pytest.mark.parametrize("mutation", [dict(qk_norm_after_rope=True), dict(qk_eps=1e-4), dict(post_norm_before_add=True),
+                                      dict(final_norm=False), dict(embed_scale=96 ** 0.5)])
+def test_the_anchor_sees_a_misplaced_norm(anchor_folders, tmp_path, mutation):
+    """Each plausible misreading of src/models/qwen3.hpp:113-301, made in the second transcription alone, moves the logits
+    by far more than the 1e-4 at which the engine is compared with the plain implementation: the q/k norm after the
+    rotation instead of before it, a q/k norm with an eps of its own instead of rms_norm_eps, the post-attention norm
+    taken before the residual sum, no final norm, embeddings scaled by sqrt(hidden)."""
+    from tests.plain.qwen3_second import SecondQwen3
+    folder = anchor_folders["B"]
+    if "qk_eps" in mutation:
+        folder = _small_queries(folder, str(tmp_path / "small_q"), 2e-3)       # head vectors of mean square ~1e-6
+    toks = torch.randint(0, 384, (29,), generator=torch.Generator().manual_seed(4)).tolist()
+    first = P.PlainQwen3(folder, compute=torch.float64).forward(toks).numpy()
+    assert abs(first - SecondQwen3(folder).forward(toks)).max() < 1e-6
+    moved = abs(first - SecondQwen3(folder, **mutation).forward(toks)).max()
+    assert moved > 5e-3, "the mutation %r moves the logits by only %g" % (mutation, moved)

@@ -112,3 +112,91 @@ def test_requests_that_can_never_fit_are_refused():
     with pytest.raises(ValueError):
         s.add_sequence(Sequence(2, [], SamplingParams()))
     s.add_sequence(seq(3, 4, max_new_tokens=4))
+
+
+def test_prefill_chunk_caps_one_requests_portion():
+    """A long prompt beside decoding requests is cut into portions of ``prefill_chunk``: it takes ceil(200 / 32) steps,
+    the budget is never exceeded, and every decoding request gets its token in every one of them."""
+    m = CacheManager([PagedKV(1, 8)], 8, 64, 8)
+    s = Scheduler(m, 64, 8, 512, prefill_chunk=32)
+    decoders = [seq(i, 5) for i in range(3)]
+    for d in decoders:
+        s.add_sequence(d)
+    run_step(m, s)
+    long = seq(9, 200)
+    s.add_sequence(long)
+    steps = 0
+    while long.num_generated == 0:
+        out = run_step(m, s)
+        steps += 1
+        assert sum(x.num_tokens for x in out) <= 64
+        assert [(x.seq.id, x.num_tokens, x.samples) for x in out[:3]] == [(0, 1, True), (1, 1, True), (2, 1, True)]
+        mine = [x for x in out if x.seq is long]
+        assert len(mine) == 1 and mine[0].num_tokens == (32 if steps < 7 else 8) and mine[0].samples == (steps == 7)
+    assert steps == -(-200 // 32) == 7
+    # two long prompts share a step's budget, each under the cap
+    a, b = seq(20, 100), seq(21, 100)
+    s.add_sequence(a); s.add_sequence(b)
+    out = run_step(m, s)
+    assert [(x.seq.id, x.num_tokens) for x in out[4:]] == [(20, 32), (21, 28)] and sum(x.num_tokens for x in out) == 64
+
+
+@pytest.mark.parametrize("chunk,page", [(2, 4), (4, 4), (8, 8), (3, 8)])
+def test_small_portions_and_portions_that_end_at_a_page_edge(chunk, page):
+    """Portions down to two tokens; with chunk == page every portion ends exactly at a page's edge: pages are taken for
+    exactly the tokens that run, one page per step and never one ahead."""
+    m = CacheManager([PagedKV(1, 8)], page, 16, 2)
+    s = Scheduler(m, 100, 2, 64, prefill_chunk=chunk)
+    a = seq(0, 19)
+    s.add_sequence(a)
+    done = 0
+    while a.num_generated == 0:
+        out = run_step(m, s)
+        assert len(out) == 1 and out[0].num_tokens == min(chunk, 19 - done)
+        done += out[0].num_tokens
+        assert a.cache.num_tokens == done and len(a.cache.tables[0]) == -(-done // page)
+        assert out[0].samples == (done == 19)
+    assert done == 19
+
+
+def test_a_parked_cache_serves_the_next_turn_and_goes_first_when_pages_are_short():
+    m, s = make(num_pages=6, page=4, budget=100, max_seqs=2, max_len=24)
+    a = seq(0, 6)
+    s.add_sequence(a)
+    run_step(m, s); run_step(m, s)                      # 6 prompt tokens, then one decoded: 7 cached, 8 known
+    s.finish(a, "max_new_tokens", keep=True)
+    assert a.status is SequenceStatus.FINISHED and a.cache is not None and a.cache.live and s.parked == [a]
+    assert m.num_free_pages() == [4] and not s.has_unfinished()
+    # a further turn: only what is not cached yet runs (the last sampled token and the new ones)
+    a.tokens += [3, 4, 5]
+    a.num_prompt_tokens = len(a.tokens)
+    s.add_sequence(a)
+    out = run_step(m, s)
+    assert [(x.seq.id, x.num_tokens, x.samples) for x in out] == [(0, 4, True)] and s.parked == []
+    s.finish(a, "eos", keep=True)
+    # another request needs the pages: the parked cache is taken back before anything is preempted or made to wait
+    b = seq(1, 17)
+    s.add_sequence(b)
+    out = run_step(m, s)
+    assert [(x.seq.id, x.num_tokens) for x in out] == [(1, 17)] and a.cache is None and s.parked == [] and s.num_preemptions == 0
+    # the turn after that recomputes the history
+    s.finish(b, "eos")
+    a.tokens += [6]
+    a.num_prompt_tokens = len(a.tokens)
+    s.add_sequence(a)
+    known = len(a.tokens)
+    assert [(x.seq.id, x.num_tokens) for x in run_step(m, s)] == [(0, known)]
+    s.finish(a, "eos", keep=True)
+    s.abort(a)                                           # removing the request gives the parked cache back
+    assert m.num_free_pages() == [6] and m.slots.num_free == 2 and s.parked == []
+
+
+def test_a_parked_cache_gives_its_slot_to_a_new_request():
+    m, s = make(num_pages=16, page=4, budget=100, max_seqs=1, max_len=24)
+    a = seq(0, 3)
+    s.add_sequence(a)
+    run_step(m, s)
+    s.finish(a, "eos", keep=True)
+    b = seq(1, 3)
+    s.add_sequence(b)
+    assert [(x.seq.id) for x in run_step(m, s)] == [1] and a.cache is None
