@@ -1,19 +1,20 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-Default: the Qwen3-8B shape of BASELINE.json configs[2] (36 layers, hidden 4096, 32 query and
+Default: the Qwen3-8B shape (36 layers, hidden 4096, 32 query and
 8 key/value heads of 128, intermediate 12288, vocabulary 151936, untied head) with random
 bfloat16 weights; 8 requests with 1024-token random prompts decode through the engine's own step
 (scheduler, step function, cache, kernels, device sampling).  A "step" is one decode step.
 Prints ONE JSON line: decoded tokens per second, plus the prefill of 2048 tokens, the decode
-step's HBM roofline, and decode at batch 1, 32 and 64.
+step's HBM roofline, and decode at batch 1, 32 and 64 (tokens per second under "points"; their time per step,
+mean context and share of the HBM roofline under "points_detail").
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--dtype bfloat16|float32]
 
-Other workloads of BASELINE.json, each again one JSON line:
+Other workloads, each again one JSON line:
 
-    python bench.py --shape 14b --serve 64                 # configs[3]: 64 requests at once until all have ended
-    python bench.py --shape 32b --batch 64 --prompt-len 4096 --context 4608 --points "" --steps 32 --warmup 4   # configs[4]
+    python bench.py --shape 14b --serve 64                 # Qwen3-14B shape: 64 requests at once until all have ended
+    python bench.py --shape 32b --batch 64 --prompt-len 4096 --context 4608 --points "" --steps 32 --warmup 4   # long keys at the 32B shape
 """
 import argparse
 import json
@@ -27,7 +28,7 @@ MODEL_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_a
                 num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936,
                 rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960,
                 bos_token_id=151643, eos_token_id=151645)
-# the larger shapes of BASELINE.json (configs[3] and configs[4]); the default stays the 8B shape
+# the larger shapes; the default stays the 8B shape
 SHAPES = {
     "8b": ("Qwen3-8B shape", MODEL_8B),
     "14b": ("Qwen3-14B shape", dict(MODEL_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)),
@@ -49,7 +50,7 @@ def main() -> int:
     ap.add_argument("--points", default="1,32,64", help="further decode batch sizes to report (empty: none)")
     ap.add_argument("--enforce-eager", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes: BASELINE.json configs[2] (8b), [3] (14b), [4] (32b)")
+    ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes of the model")
     ap.add_argument("--serve", type=int, default=0, metavar="N",
                     help="instead of the decode steps: N requests arriving at once, prompts of 128..2048 and outputs of 64..512 "
                          "tokens (uniform), run until all have ended; the value is generated tokens per second of the whole run")
@@ -180,10 +181,13 @@ def main() -> int:
     linear_flops = 2 * T * L * (H * (nq + 2 * nkv) * d + nq * d * H + 3 * H * I) + 2 * V * H
     attn_flops = L * 4 * d * nq * T * (T + 1) / 2
     pf_flops = linear_flops + attn_flops
-    extra = {}
+    extra, detail = {}, {}
     for b in points:
-        v, _, _ = decode_run(b, max(8, args.steps // 2), max(4, args.warmup // 2))
+        v, b_ms, b_ctx = decode_run(b, max(20, args.steps // 2), max(4, args.warmup // 2))
         extra["decode_b%d" % b] = round(v, 1)
+        b_gbs = (weight_bytes + b * b_ctx * kv_bytes_per_token) / (b_ms * 1e-3) / 1e9
+        detail["decode_b%d" % b] = {"ms_per_step": round(b_ms, 4), "mean_context": round(b_ctx, 1), "hbm_gbs": round(b_gbs, 1),
+                                    "hbm_frac": round(b_gbs / PEAK_HBM_GBS, 4)}
     line = {
         "metric": "decode tok/s at batch %d (%s, %d-token prompts)" % (args.batch, shape_name, args.prompt_len),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -198,6 +202,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
         "points": extra,
+        "points_detail": detail,
     }
     print(json.dumps(line))
     return 0

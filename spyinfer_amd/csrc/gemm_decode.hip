@@ -315,6 +315,143 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
     }
 }
 
+// For 17 to 64 rows and matrices of many columns (the gated product, the output head): what bounds the kernel above is
+// not the matrix' way from memory but the L2's throughput, through which every block also pulls all of X (with MT row
+// tiles that is MT times the bytes of its tile of W).  Here one block per CU walks a run of neighbouring column tiles,
+// CT at a time, against the same X fragments in registers: X's traffic falls to MT / CT (MT / 2 CT for the gated
+// product, whose gate and up tiles share them as well).  The 8 waves of a block split K as above; operands are loaded
+// half a chunk at a time (the accumulators of CT tiles take the registers of the other half); the waves' sums of one
+// column tile are added through LDS by the wave that owns the tile (tile ct -> wave ct), in the order of the waves, and
+// that wave runs the tile's epilogue.  Store and gated epilogues only.
+template <int EPI, bool SCALED, typename TC, int MT, int CT, bool XT, bool OT>
+__global__ __launch_bounds__(512, 1) void gemm_decode_wide_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, const float* __restrict__ ss_in,
+    int n_parts, float eps, int M, int N, int K) {
+    static_assert(EPI == EPI_STORE || EPI == EPI_GATED, "the wide kernel has no residual epilogue");
+    static_assert(CT <= 8, "a wave owns at most one column tile of a group");
+    constexpr int GW = 8;
+    constexpr int GATES = EPI == EPI_GATED ? 2 : 1;
+    constexpr int NT = GATES * CT;
+    constexpr int MP = 16 * MT;
+    __shared__ float red[(GW - 1) * MT * 64 * 4];
+    __shared__ float ss_red[GW * 4 * MP];
+    __shared__ float row_scale[MP];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+
+    if (SCALED) {
+        float part[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) part[mt] = 0.f;
+        for (int p = wave * 4 + g; p < n_parts; p += GW * 4)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) part[mt] += ss_in[p * MP + 16 * mt + r];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) ss_red[(wave * 4 + g) * MP + 16 * mt + r] = part[mt];
+        __syncthreads();
+        if (threadIdx.x < MP) {
+            float s = 0.f;
+            for (int i = 0; i < GW * 4; ++i) s += ss_red[i * MP + threadIdx.x];
+            row_scale[threadIdx.x] = 1.0f / sqrtf(s / (float)K + eps);
+        }
+        __syncthreads();
+    }
+
+    // this block's run of column tiles: the tiles dealt evenly over the blocks
+    const int tiles = N / 16;
+    const int t_begin = (int)((long long)tiles * blockIdx.x / gridDim.x), t_end = (int)((long long)tiles * (blockIdx.x + 1) / gridDim.x);
+    const size_t chunk_stride = (size_t)(GATES * tiles) * 4096;
+    unsigned xoff[MT];
+    bool x_ok[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        x_ok[mt] = 16 * mt + r < M;
+        xoff[mt] = XT ? (unsigned)mt * 1024u + 16u * lane : (unsigned)min(16 * mt + r, M - 1) * (unsigned)K * 2u + 16u * g;
+    }
+    const char* xbase = reinterpret_cast<const char*>(X);
+    const int nfull = K / GD_CHUNK;
+
+    for (int t0 = t_begin; t0 < t_end; t0 += CT) {
+        const int here = min(CT, t_end - t0);            // tiles of this group (the run's last group may have fewer)
+        f32x4_t acc[NT][MT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)t0 * 4096 + 16u * lane;
+        for (int c = wave; c < nfull; c += GW) {
+            const char* wb = wbase + (size_t)c * chunk_stride;
+            const char* xb = xbase + (size_t)c * (XT ? 4 * MT * 1024 : GD_CHUNK * 2);
+#pragma unroll
+            for (int h = 0; h < 4; h += 2) {
+                bf16x8_t a[NT][2], b[MT][2];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        // a tile that the group does not have reads the group's first tile again (its sums are dropped)
+                        const int ct = nt % CT < here ? nt % CT : 0;
+                        a[nt][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(
+                            wb + (size_t)((nt / CT) * tiles + ct) * 4096 + 1024 * (h + j)));
+                    }
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        b[mt][j] = x_ok[mt] ? *reinterpret_cast<const bf16x8_t*>(xb + xoff[mt] + (XT ? MT * 1024 : 64) * (h + j))
+                                            : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+                }
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt)
+                            acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], b[mt][j], acc[nt][mt], 0, 0, 0);
+            }
+        }
+        // ---- add the waves' sums tile by tile; tile ct (and its up tile) belongs to wave ct ---------------------------
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int owner = nt % CT;
+            if (wave != owner) {
+                const int slot = wave < owner ? wave : wave - 1;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) red[((slot * MT + mt) * 4 + i) * 64 + lane] = acc[nt][mt][i];
+            }
+            __syncthreads();
+            if (wave == owner) {
+#pragma unroll
+                for (int w = 0; w < GW - 1; ++w)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) acc[nt][mt][i] += red[((w * MT + mt) * 4 + i) * 64 + lane];
+            }
+            __syncthreads();
+        }
+        // ---- epilogue of the tile this wave owns ------------------------------------------------------------------------
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            if (wave != ct || ct >= here) continue;
+            const int n = (t0 + ct) * 16 + 4 * g;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const int m = 16 * mt + r;
+                if (m >= M) continue;
+                const float scale = SCALED ? row_scale[m] : 1.f;
+                TC* out = C + (OT ? operand_order(m, n, MT) : (size_t)m * N + n);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float v = acc[ct][mt][i] * scale;
+                    if (EPI == EPI_GATED) { const float up = acc[CT + ct][mt][i] * scale; v = (v / (1.0f + expf(-v))) * up; }
+                    out[i] = from_f32<TC>(v);
+                }
+            }
+        }
+    }
+}
+
 struct GdArgs {
     const bf16_t* x; const bf16_t* w; void* c; float* resid; bf16_t* xw_out; const bf16_t* w_next; float* ss_out; const float* ss_in;
     int n_parts; float eps; int M, N, K; bool xt, ot; hipStream_t st;
@@ -322,9 +459,58 @@ struct GdArgs {
 
 // Blocks of 8 waves, one per 16 columns; the gated product (two tiles per block, usually three blocks per CU)
 // takes blocks of GD_WAVES_GATED waves so that all of them are resident at once.
+// Compute units of the current device (asked for once per device).
+static int compute_units() {
+    static int cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (!cached[dev]) {
+        int n = 0;
+        cached[dev] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
+    }
+    return cached[dev];
+}
+
+#ifndef GD_WIDE
+#define GD_WIDE 1     // 0: the wide kernel is never taken (for measurements)
+#endif
+
+// Column tiles per group of the wide kernel for blocks that walk `per` tiles each with MT row tiles: the CT that moves the
+// fewest bytes through L2, X once per group (MT units per step) and W once per tile (GATES units).
+static int wide_ct(int per, int MT, int gates, int max_ct) {
+    int best = 1, best_cost = 1 << 30;
+    for (int ct = 1; ct <= max_ct; ++ct) {
+        const int cost = ((per + ct - 1) / ct) * MT + per * gates;
+        if (cost < best_cost) { best = ct; best_cost = cost; }
+    }
+    return best;
+}
+
+template <int EPI, bool SCALED, typename TC, int MT, bool XT, bool OT>
+static bool gd_launch_wide(const GdArgs& a) {
+    if constexpr (EPI == EPI_RESID) return false;
+    else {
+        constexpr int GATES = EPI == EPI_GATED ? 2 : 1;
+        constexpr int MAX_CT = EPI == EPI_GATED ? 3 : 4;
+        const int cus = compute_units(), tiles = a.N / 16;
+        if (!GD_WIDE || tiles < 2 * cus) return false;       // fewer than two tiles per CU: one tile per block, two blocks per CU
+        const int ct = wide_ct((tiles + cus - 1) / cus, MT, GATES, MAX_CT);
+#define GD_WIDE_ARGS a.x, a.w, (TC*)a.c, a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K
+        if (ct == 1) return false;
+        if (ct == 2) gemm_decode_wide_kernel<EPI, SCALED, TC, MT, 2, XT, OT><<<cus, 512, 0, a.st>>>(GD_WIDE_ARGS);
+        else if (ct == 3) gemm_decode_wide_kernel<EPI, SCALED, TC, MT, 3, XT, OT><<<cus, 512, 0, a.st>>>(GD_WIDE_ARGS);
+        else gemm_decode_wide_kernel<EPI, SCALED, TC, MT, MAX_CT, XT, OT><<<cus, 512, 0, a.st>>>(GD_WIDE_ARGS);
+#undef GD_WIDE_ARGS
+        return true;
+    }
+}
+
 template <int EPI, bool SCALED, typename TC, bool XT, bool OT>
 static void gd_launch2(const GdArgs& a) {
     constexpr int W = EPI == EPI_GATED ? GD_WAVES_GATED : 8;
+    if (a.M > 48) { if (gd_launch_wide<EPI, SCALED, TC, 4, XT, OT>(a)) return; }
+    else if (a.M > 32) { if (gd_launch_wide<EPI, SCALED, TC, 3, XT, OT>(a)) return; }
+    else if (a.M > 16) { if (gd_launch_wide<EPI, SCALED, TC, 2, XT, OT>(a)) return; }
 #define GD_ARGS a.x, a.w, (TC*)a.c, a.resid, a.xw_out, a.w_next, a.ss_out, a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K
     // Two column tiles per block where that leaves enough blocks (measured, 64 rows: qkv of 6144 columns 26.8 -> 20.5
     // us; with 4096 columns, 128 blocks, 15.4 -> 19.4 us; the gated product 53 -> 61 us: its block has one wave per SIMD then)

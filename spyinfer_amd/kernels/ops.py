@@ -77,8 +77,8 @@ class _Hip:
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
                      "spy_gemm_decode", "spy_embedding_sumsq", "spy_sample_static"):
             if not hasattr(self.lib, name):
-                raise KernelError("the kernel library %s lacks %s: rebuild it (python -c 'import __graft_entry__ as g; g.build()')"
-                                  % (self.lib._name, name))
+                raise KernelError("the kernel library %s lacks %s: it is older than its sources; build it again "
+                                  "(spyinfer_amd.kernels.build.build())" % (self.lib._name, name))
             getattr(self.lib, name).restype = ctypes.c_int64 if name.endswith("_workspace") else ctypes.c_int
 
     def call(self, name, *args):

@@ -115,7 +115,11 @@ def test_linear_with_tiled_weights(M, N, K):
                                             (3, 5120, 128, 64, 1e-2), (17, 256, 128, 96, 1e-6), (32, 1024, 2048, 320, 1e-5),
                                             (41, 128, 384, 400, 1e-6), (64, 256, 128, 6144, 1e-6), (57, 128, 384, 6176, 1e-5),
                                             (33, 256, 128, 6240, 1e-6), (20, 128, 128, 6144, 1e-6), (48, 768, 384, 96, 1e-6), (25, 1280, 128, 64, 1e-5),
-                                            (64, 2048, 384, 128, 1e-6)])
+                                            (64, 2048, 384, 128, 1e-6),
+                                            # many column tiles (two and more per compute unit): blocks that walk a run of
+                                            # tiles, several at a time, the last group of a run with fewer
+                                            (64, 128, 8320, 8208, 1e-6), (37, 256, 8448, 9008, 1e-5), (20, 128, 8192, 16400, 1e-6),
+                                            (48, 128, 128, 151936, 1e-6), (16, 128, 8320, 8208, 1e-6)])
 def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
     """The chain of a decode step's products with the norms folded in: the residual epilogue adds to the stream,
     prepares bf16(h * w) and the parts of sum(h^2); the next products scale their sums by rsqrt(mean(h^2) + eps).
