@@ -478,7 +478,9 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
         tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz, out_tiles)
 #define ATT_CASE(DM)                                                                                                          \
     if (qkv) ATT_LAUNCH(DM, true, true); else if (d == DM) ATT_LAUNCH(DM, false, true); else ATT_LAUNCH(DM, false, false);       \
-    if (splits > 1)                                                                                                           \
+    if (splits > 1 && qkv)                                                                                                    \
+        attention_merge_kernel<DM, true><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits, 1, out_tiles); \
+    else if (splits > 1)                                                                                                      \
         attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits, 1, out_tiles);
     switch (dmax_of(d)) {
         case 64: ATT_CASE(64) break;

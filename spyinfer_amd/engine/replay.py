@@ -54,8 +54,7 @@ def run(argv=None, stdin=None, stdout=None) -> int:
     os.makedirs(args.out, exist_ok=True)
     if args.max_tokens <= 0:
         ap.error("--max-tokens must be positive")
-    if ops._impl is None:
-        ops.hip()   # builds the kernel library at the first call, and fails here if there is no GPU
+    ops.hip()       # builds the kernel library at the first call, and fails here if there is no GPU
     model = load_model(args.model, args.dtype, args.device)
     num_pages = page_rounded_tokens(args.max_tokens, args.kvcache_block_size)
     runner = ModelRunner(model, args.dtype, args.device, args.kvcache_block_size, num_pages, args.max_num_seqs,

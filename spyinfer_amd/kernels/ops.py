@@ -22,19 +22,11 @@ from . import build as _build
 F32, BF16, I32 = 0, 1, 2
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 
-_impl = None          # object with the same functions; installed by tests that emulate the kernels
 _hip = None
 
 
 class KernelError(RuntimeError):
     pass
-
-
-def install_test_double(impl) -> None:
-    """Route all operations to ``impl`` (None restores the HIP library).  For tests of the
-    engine's logic on machines without a GPU; never used by the engine itself."""
-    global _impl
-    _impl = impl
 
 
 def _code(t: torch.Tensor, what: str) -> int:
@@ -105,8 +97,6 @@ def library_path() -> str:
 # --------------------------------------------------------------------------
 def embedding(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     """out[t, :] = table[ids[t], :] widened to float32 (the start of the residual stream)."""
-    if _impl is not None:
-        return _impl.embedding(ids, table)
     _dev(ids, table)
     _check(ids.dtype == torch.int32 and ids.dim() == 1, "embedding: ids must be int32 [T]")
     _check(table.dim() == 2, "embedding: table must be [V, H]")
@@ -124,8 +114,6 @@ def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: tor
 
     Without ``rows``: every row is updated and normalised -> [T, H].  With ``rows``
     (int32 [R]): only those rows are summed and normalised -> [R, H]; resid is left as it is."""
-    if _impl is not None:
-        return _impl.add_rms_norm(resid, delta, weight, eps, out_dtype, rows)
     _dev(resid, delta, weight, rows)
     _check(resid.dtype == torch.float32 and resid.dim() == 2, "add_rms_norm: the residual stream must be float32 [T, H]")
     T, H = resid.shape
@@ -145,8 +133,6 @@ def add_rms_norm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: tor
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """RMS norm over the last dimension, same dtype out as in."""
-    if _impl is not None:
-        return _impl.rms_norm(x, weight, eps)
     _dev(x, weight)
     n = x.shape[-1]
     _check(weight.shape == (n,), "rms_norm: weight must match the last dimension")
@@ -190,7 +176,7 @@ def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
     """``w [N, K]`` in the order the decode kernel reads it: [K/128 chunks][N/16 tiles][4 steps][g = 4][r = 16][8], the
     values of lane 16 g + r being w[16 tile + r][128 chunk + 32 step + 8 g ..].  None if the copy is switched off or
     the shape or dtype does not allow it (then the kernel for row-major matrices stands)."""
-    if not TILED_WEIGHTS or _impl is not None or not w.is_cuda or w.dtype != torch.bfloat16 or w.dim() != 2:
+    if not TILED_WEIGHTS or not w.is_cuda or w.dtype != torch.bfloat16 or w.dim() != 2:
         return None
     N, K = w.shape
     if N % 16 or K % 128 or N * 256 + 8192 >= (1 << 32):
@@ -215,9 +201,6 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
 
     float32 anywhere among x and w -> the hand-written true-fp32 kernel.  All bfloat16: the streaming
     MFMA kernel for few rows, the library product for many."""
-    if _impl is not None:
-        y = _impl.linear(x, w, out_dtype)
-        return y if out is None else out.copy_(y)
     _dev(x, w)
     _check(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "linear: x [M, K] and w [N, K] expected, got %s and %s"
            % (tuple(x.shape), tuple(w.shape)))
@@ -252,8 +235,6 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """silu(x . Wgate^T) * (x . Wup^T) with ``w_gate_up [2 I, K]`` = [Wgate | Wup] -> [M, I].  For few bfloat16 rows
     (decode) one kernel does both products and the SwiGLU; otherwise it is linear() followed by swiglu()."""
-    if _impl is not None:
-        return _impl.swiglu(_impl.linear(x, w_gate_up, None))
     _dev(x, w_gate_up)
     _check(x.dim() == 2 and w_gate_up.dim() == 2 and x.shape[1] == w_gate_up.shape[1] and w_gate_up.shape[0] % 2 == 0,
            "linear_swiglu: x [M, K] and w [2 I, K] expected")
@@ -321,7 +302,7 @@ def fused_decode_ok(rows: int, act_dtype, *tiled_weights, max_rows: Optional[int
     """True if products of ``rows`` rows with these tiled matrices can run with the norm's scale and the residual
     sum folded in: bfloat16 activations, at most ``max_rows`` rows (default: ``default_fold_rows`` of the matrices),
     tiled bfloat16 weights."""
-    if not FUSED_DECODE or _impl is not None or act_dtype != torch.bfloat16 or not 0 < rows <= FUSED_DECODE_MAX_ROWS:
+    if not FUSED_DECODE or act_dtype != torch.bfloat16 or not 0 < rows <= FUSED_DECODE_MAX_ROWS:
         return False
     if max_rows is None:
         max_rows = default_fold_rows(sum(t.numel() for t in tiled_weights if t is not None))
@@ -442,9 +423,6 @@ def qk_norm_rope_store(qkv: torch.Tensor, n_q: int, n_kv: int, d: int, q_norm_w,
     ``cos/sin [positions, rotary_dim/2]`` (if given), q written to the result ``[T, n_q d]``;
     k and v written into the cache pages at ``slots[t] = page * page_size + offset``
     (skipped for slot -1 or when ``slots`` is None)."""
-    if _impl is not None:
-        return _impl.qk_norm_rope_store(qkv, n_q, n_kv, d, q_norm_w, k_norm_w, eps, cos, sin, rotary_dim, positions,
-                                        k_cache, v_cache, page_size, slots)
     _dev(qkv, q_norm_w, k_norm_w, cos, sin, positions, k_cache, v_cache, slots)
     T = qkv.shape[0]
     _check(qkv.dim() == 2 and qkv.shape[1] == (n_q + 2 * n_kv) * d, "qk_norm_rope_store: qkv must be [T, (n_q + 2 n_kv) d]")
@@ -546,7 +524,7 @@ FUSED_ATTENTION = True     # False: the norm, rotation and store always run as a
 def fused_attention_ok(dtype, meta: AttentionMeta, n_q: int, n_kv: int, d: int, page_size: int, rotary_dim: int, q_norm_w, k_norm_w) -> bool:
     """True if this step's attention may take the raw product (``RawQKV``): every entry a single token, bfloat16,
     head_dim 64, 128 or 256 rotated whole or not at all, 16-row tiles built for this group size."""
-    if not FUSED_ATTENTION or _impl is not None or not mfma_attention_ok(dtype, d, page_size):
+    if not FUSED_ATTENTION or not mfma_attention_ok(dtype, d, page_size):
         return False
     if meta.T != meta.S or meta.max_q_len != 1 or meta.tiles is None or meta.tiles_group != n_q // n_kv or n_q // n_kv > 16:
         return False
@@ -565,8 +543,6 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
     reads keys max(0, p - window + 1) .. p.  Scores, softmax and the weighted sum are float32.
     ``for_product``: the result goes into a decode product only and may come as OperandRows (it does when all of the
     step runs through the 16-row-tile kernel and has few rows)."""
-    if _impl is not None:
-        return _impl.paged_attention(q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window)
     T, S = meta.T, meta.S
     if raw is not None:
         _dev(raw.qkv, raw.q_norm_w, raw.k_norm_w, raw.cos, raw.sin)
@@ -657,8 +633,6 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
 
 def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     """``gate_up [T, 2 I]`` = [gate | up]  ->  silu(gate) * up  [T, I], float32 arithmetic."""
-    if _impl is not None:
-        return _impl.swiglu(gate_up)
     _dev(gate_up)
     _check(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "swiglu: [T, 2 I] expected")
     T, I = gate_up.shape[0], gate_up.shape[1] // 2
@@ -673,8 +647,6 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor) -> 
     """Row r: temperature[r] == 0 -> first maximum of logits[r]; else the token whose cumulative
     probability of softmax(logits[r] / temperature[r]), over ascending token ids, first exceeds
     u[r] in [0, 1).  int32 [R]."""
-    if _impl is not None:
-        return _impl.sample(logits, temperature, u)
     _dev(logits, temperature, u)
     _check(logits.dtype == torch.float32 and logits.dim() == 2, "sample: logits must be float32 [R, V]")
     R, V = logits.shape

@@ -103,11 +103,14 @@ class PagedAttention(Mixer):
         return specs
 
     def bind(self, prefix, weights):
-        q, k, v = (weights[prefix + ".%s_proj.weight" % n] for n in "qkv")
+        # the three matrices leave the caller's dictionary here, so that they are freed once they are fused: binding a
+        # model never holds the separate matrices, the fused one and its tiled copy of all layers at once
+        q, k, v = (weights.pop(prefix + ".%s_proj.weight" % n) for n in "qkv")
         if not (q.dtype == k.dtype == v.dtype):
             q, k, v = q.float(), k.float(), v.float()
         # one product for q, k and v: rows [q heads | k heads | v heads]
         self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
+        del q, k, v
         self.w_o = weights[prefix + ".o_proj.weight"]
         self.w_qkv_tiled, self.w_o_tiled = ops.tile_weight(self.w_qkv), ops.tile_weight(self.w_o)
         if self.qk_norm_eps is not None:

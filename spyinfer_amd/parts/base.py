@@ -26,7 +26,8 @@ class Part:
         return []
 
     def bind(self, prefix: str, weights: Dict[str, torch.Tensor]) -> None:
-        """Take the tensors named by ``weight_specs(prefix)`` (already on the device)."""
+        """Take the tensors named by ``weight_specs(prefix)`` (already on the device).  A part that copies tensors into
+        a form of its own (fused, reordered) may take them out of ``weights`` (``pop``), so that the originals are freed."""
 
 
 class Norm(Part):

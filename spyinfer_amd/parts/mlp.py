@@ -26,10 +26,12 @@ class GatedMLP(FeedForward):
                 WeightSpec(prefix + ".down_proj.weight", (H, I))]
 
     def bind(self, prefix, weights):
-        g, u = weights[prefix + ".gate_proj.weight"], weights[prefix + ".up_proj.weight"]
+        # (popped: the separate matrices are freed once they are fused, see PagedAttention.bind)
+        g, u = weights.pop(prefix + ".gate_proj.weight"), weights.pop(prefix + ".up_proj.weight")
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
         self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
+        del g, u
         self.w_down = weights[prefix + ".down_proj.weight"]
         # tiles 0 .. I/16 - 1 of the tiled copy are gate rows, the rest up rows: what the fused SwiGLU kernel expects
         self.w_gate_up_tiled = ops.tile_weight(self.w_gate_up) if self.intermediate_size % 16 == 0 else None

@@ -13,13 +13,27 @@ def pytest_configure(config):
 
 
 @pytest.fixture
-def emu_ops():
-    """Routes the engine's operations to the CPU stand-in for the duration of a test."""
+def emu_ops(monkeypatch):
+    """Replaces the engine's operations (``spyinfer_amd.kernels.ops``) by the CPU stand-in for the duration of a test, so
+    that the engine's logic (batches, cache pages, block tables, scheduling) runs on a machine without a GPU.  The
+    product has no such switch: the stand-in is patched in from here."""
     from spyinfer_amd.kernels import ops
     from tests.emu_ops import EmuOps
-    ops.install_test_double(EmuOps())
-    yield
-    ops.install_test_double(None)
+    emu = EmuOps()
+    for name in ("embedding", "add_rms_norm", "rms_norm", "qk_norm_rope_store", "swiglu", "sample"):
+        monkeypatch.setattr(ops, name, getattr(emu, name))
+
+    def linear(x, w, out_dtype=None, tiled=None, out=None):
+        y = emu.linear(x, w, out_dtype)
+        return y if out is None else out.copy_(y)
+    monkeypatch.setattr(ops, "linear", linear)
+    monkeypatch.setattr(ops, "linear_swiglu", lambda x, w, tiled=None: emu.swiglu(emu.linear(x, w)))
+    monkeypatch.setattr(ops, "paged_attention", lambda q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window, raw=None,
+                        for_product=False: emu.paged_attention(q, k_cache, v_cache, page_size, meta, n_q, n_kv, d, scale, window))
+    monkeypatch.setattr(ops, "tile_weight", lambda w: None)
+    monkeypatch.setattr(ops, "fused_decode_ok", lambda *a, **k: False)
+    monkeypatch.setattr(ops, "fused_attention_ok", lambda *a, **k: False)
+    monkeypatch.setattr(ops, "hip", lambda: None)
 
 
 @pytest.fixture(autouse=True)

@@ -7,7 +7,6 @@ def require_gpu():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     from spyinfer_amd.kernels import ops
-    ops.install_test_double(None)
     ops.hip()
     return torch.device("cuda:0")
 

@@ -505,6 +505,33 @@ def _toy_parts():
     return ToyConfig, build
 
 
+def _plain_running_mean_lm(folder, tokens):
+    """The toy model of ``_toy_parts`` on a whole sequence, no cache, from the plain functions: layers 0 and 2 mix by a
+    running mean, layer 1 by attention over a window of 24, and the run order is layers 0, 1, 2, 1."""
+    from safetensors.torch import load_file
+    from tests.plain import qwen3_plain as P
+    w = {k: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    T = len(tokens)
+    cos, sin = P.rope_tables(T, 16, 10000.0)
+    pos = torch.arange(T)
+    h = P.embedding(torch.tensor(tokens), w["model.embed_tokens.weight"])
+    for layer in (0, 1, 2, 1):
+        p = "model.layers.%d." % layer
+        n1 = P.rms_norm(h, w[p + "input_layernorm.weight"], 1e-5)
+        if layer == 1:
+            q = P.rope_apply(P.linear(n1, w[p + "self_attn.q_proj.weight"]).view(T, 4, 16), pos, cos, sin)
+            k = P.rope_apply(P.linear(n1, w[p + "self_attn.k_proj.weight"]).view(T, 2, 16), pos, cos, sin)
+            v = P.linear(n1, w[p + "self_attn.v_proj.weight"]).view(T, 2, 16)
+            a = P.linear(P.attention(q, k, v, 24).reshape(T, -1), w[p + "self_attn.o_proj.weight"])
+        else:
+            a = torch.cumsum(n1, 0) / (pos + 1).float()[:, None] * w[p + "self_attn.gain"]
+        h = h + a
+        n2 = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], 1e-5)
+        h = h + P.linear(P.swiglu(P.linear(n2, w[p + "mlp.gate_proj.weight"]), P.linear(n2, w[p + "mlp.up_proj.weight"])),
+                         w[p + "mlp.down_proj.weight"])
+    return P.linear(P.rms_norm(h, w["model.norm.weight"], 1e-5), w["model.embed_tokens.weight"])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_toy_architecture_with_state(dtype, tmp_path):
     from spyinfer_amd.config import register_architecture, unregister_architecture
@@ -523,9 +550,9 @@ def test_toy_architecture_with_state(dtype, tmp_path):
             rc.run_replay_inprocess(folder, dtype, out, steps, rc.max_live_tokens(steps))
             outs[mode] = rc.collect(out, steps, 97)
         tol = TOL[dtype]
-        for mode in ("portions", "mixed"):
-            for key, row in outs[mode].items():
-                assert np.allclose(row, outs["whole"][key], atol=tol["atol"], rtol=tol["rtol"]), (mode, key)
+        ref = {rid: _plain_running_mean_lm(folder, t) for rid, t in reqs.items()}
+        for mode in ("whole", "portions", "mixed"):
+            rc.compare(outs[mode], ref, what="toy with state/%s/%s" % (mode, dtype), **tol)
         # the state matters: a request's logits differ from those of its second half alone
         first = next(iter(reqs))
         assert not np.allclose(outs["whole"][(first, 40)], outs["whole"][(first, 5)], atol=1e-3)

@@ -44,7 +44,7 @@ def _runners(dev, requests, pages, widths, sharp=False):
                     if k.endswith("q_norm.weight") or k.endswith("k_norm.weight"):
                         w16[k] = (w16[k].float() * 2.0).to(torch.bfloat16)
         weights = w16 if dtype == "bfloat16" else {k: (v.float() if v.dtype == torch.bfloat16 else v) for k, v in w16.items()}
-        model.bind(weights, dev)
+        model.bind(dict(weights), dev)       # a copy: parts take the matrices they fuse out of the dictionary
         out.append(ModelRunner(model, dtype, dev, 16, pages, requests, enforce_eager=True, max_model_len=1024))
     return out, raw, w16
 
