@@ -18,7 +18,6 @@ typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
 #define PF_KEYS 64       // keys staged per round
-#define PF_ROWS 128      // rows per block
 #define PF_SLACK 8.0f    // a score may exceed the running maximum by 2^8 before the maximum is raised
 
 __device__ __forceinline__ bf16x8_t pf_zero8() { return bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
@@ -30,7 +29,9 @@ __device__ __forceinline__ bf16x8_t pf_zero8() { return bf16x8_t{0, 0, 0, 0, 0, 
 // MINW: waves per SIMD that the registers must allow.  The 8-wave shape with 4 (128 registers, two blocks per CU) is
 // the fastest shape for grids of more than one block per CU; with one block per CU it is 6 % faster with the
 // registers of 2.
-template <int DMAX, bool DFULL, int RT, int MINW>
+// PF_ROWS: rows per block, 128 or 256.  With 256 rows (8 waves of two row tiles) a round's keys and values are staged
+// once for twice the rows: half the staging instructions and half the LDS reads per score of the 128-row shapes.
+template <int DMAX, bool DFULL, int RT, int MINW, int PF_ROWS>
 __global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
@@ -339,11 +340,15 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kern
     }   // which
 }
 
-extern "C" int64_t spy_attention_prefill_workspace(int num_tiles, int n_kv, int d, int splits) {
+extern "C" int64_t spy_attention_prefill_workspace(int num_tiles, int tile_rows, int n_kv, int d, int splits) {
     if (splits <= 1) return 0;
-    return (int64_t)num_tiles * (PF_ROWS / 16) * n_kv * splits * 16 * ((d <= 64 ? 64 : 128) + 2);
+    return (int64_t)num_tiles * (tile_rows / 16) * n_kv * splits * 16 * ((d <= 64 ? 64 : 128) + 2);
 }
 
+// Tiles of 256 rows against tiles of 128, same measurement: 92 against 73 us at 2048 tokens (128 blocks: half the CUs
+// idle), 125 against 133 at 3072, 170 against 195 at 4096, 607 against 675 at 8192, 2331 against 2565 at 16384 (0.94
+// PFLOP/s); the caller picks the tile size by the number of blocks.  One tile per block instead of two, so that a grid
+// of one block per CU becomes two per CU, was slower at every length (88 against 73 us at 2048 tokens).
 // Measured on MI355X (256 CUs), 32 query heads of 128, microseconds per call for 2048 / 2304 / 3072 / 4096 / 8192
 // tokens of one prompt (256 / 288 / 384 / 512 / 1024 blocks): 4 waves of two row tiles 85 / 115 / 148 / 193 / 717;
 // 8 waves of one row tile with registers for one block per CU 65 / 130 / 165 / 217 / 807, with 128 registers (two
@@ -360,8 +365,8 @@ static long long cu_count() {
 
 extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, const void* vc, int P, int num_pages, const int* cu_q,
                                      const int* pos0, const int* kv_len, const int* block_table, int max_blocks,
-                                     const int* tile_entry, const int* tile_row0, int num_tiles, int S, int T, int n_q, int n_kv,
-                                     int d, float scale, int window, int splits, float* ws, hipStream_t st) {
+                                     const int* tile_entry, const int* tile_row0, int num_tiles, int tile_rows, int S, int T, int n_q,
+                                     int n_kv, int d, float scale, int window, int splits, float* ws, hipStream_t st) {
     SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
                 "spy_attention_prefill: empty operand");
     SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "spy_attention_prefill: head_dim %d is not a multiple of 16 in 16..128", d);
@@ -372,20 +377,23 @@ extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, c
     SPY_REQUIRE(n_kv <= 65535, "spy_attention_prefill: too many kv heads");
     SPY_REQUIRE(splits >= 1 && splits <= 16, "spy_attention_prefill: %d key parts (1..16 allowed)", splits);
     SPY_REQUIRE(splits == 1 || ws, "spy_attention_prefill: key parts without a workspace");
+    SPY_REQUIRE(tile_rows == 128 || (tile_rows == 256 && (d == 64 || d == 128)),
+                "spy_attention_prefill: tiles of %d rows (128, or 256 for head sizes 64 and 128)", tile_rows);
     const dim3 grid(splits > 1 ? num_tiles : (num_tiles + 1) / 2, n_kv, splits);
-    const dim3 mgrid(num_tiles * (PF_ROWS / 16), n_kv);
+    const dim3 mgrid(num_tiles * (tile_rows / 16), n_kv);
     const bool one_per_cu = (long long)grid.x * grid.y * grid.z <= cu_count();
 #define PF_ARGS (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table,   \
                 max_blocks, tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p, num_tiles, splits, ws
     // (head sizes other than 64 and 128 keep the 4-wave shape: with conditions in the head-dim loops the other needs too many registers)
 #define PF_CASE(DM)                                                                                                              \
-    if (d == DM) {                                                                                                               \
-        if (one_per_cu) attention_prefill_kernel<DM, true, 1, 2><<<grid, PF_ROWS * 4, 0, st>>>(PF_ARGS);                         \
-        else attention_prefill_kernel<DM, true, 1, 4><<<grid, PF_ROWS * 4, 0, st>>>(PF_ARGS);                                    \
-    } else attention_prefill_kernel<DM, false, 2, 2><<<grid, PF_ROWS * 2, 0, st>>>(PF_ARGS);                                     \
+    if (tile_rows == 256) attention_prefill_kernel<DM, true, 2, 2, 256><<<grid, 512, 0, st>>>(PF_ARGS);                          \
+    else if (d == DM) {                                                                                                          \
+        if (one_per_cu) attention_prefill_kernel<DM, true, 1, 2, 128><<<grid, 512, 0, st>>>(PF_ARGS);                            \
+        else attention_prefill_kernel<DM, true, 1, 4, 128><<<grid, 512, 0, st>>>(PF_ARGS);                                       \
+    } else attention_prefill_kernel<DM, false, 2, 2, 128><<<grid, 256, 0, st>>>(PF_ARGS);                                        \
     if (splits > 1)                                                                                                              \
         attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits,    \
-                                                          PF_ROWS / 16);
+                                                          tile_rows / 16);
     if (d <= 64) { PF_CASE(64) } else { PF_CASE(128) }
 #undef PF_CASE
 #undef PF_ARGS

@@ -468,14 +468,15 @@ class AttentionMeta:
     tiles: {"small": (tile_entry [N], tile_row0 [N], N), "big": (...)}: 16-row tiles of (token,
     head-in-group) rows for entries with few rows and 128-row tiles for entries with many, built
     for one group size ``tiles_group``; None if not built.
+    ``big_rows``: rows of a "big" tile (128 or 256, see ``prefill_tile_rows``).
     Host-side: S, T, max_blocks, max_kv_len, max_q_len."""
 
     def __init__(self, cu_q, pos0, kv_len, block_table, token_entry, positions, S, T, max_blocks, max_kv_len, max_q_len,
-                 tiles=None, tiles_group=0, fixed_shape=False):
+                 tiles=None, tiles_group=0, fixed_shape=False, big_rows=128):
         self.cu_q, self.pos0, self.kv_len, self.block_table = cu_q, pos0, kv_len, block_table
         self.token_entry, self.positions = token_entry, positions
         self.S, self.T, self.max_blocks, self.max_kv_len, self.max_q_len = S, T, max_blocks, max_kv_len, max_q_len
-        self.tiles, self.tiles_group = tiles, tiles_group
+        self.tiles, self.tiles_group, self.big_rows = tiles, tiles_group, big_rows
         #: True: the step is captured in a graph (block tables have a fixed width; what a launch's shape takes from the
         #: requests' lengths, the number of key parts, is part of the graph's key)
         self.fixed_shape = fixed_shape
@@ -501,6 +502,21 @@ def prefill_attention_ok(d: int, page_size: int) -> bool:
     """Whether entries with many rows may be cut into 128-row tiles: the LDS-sharing kernel takes head
     sizes up to 128 and pages of a power of two; other shapes run wholly through the general kernel."""
     return d <= PREFILL_ATTENTION_MAX_HEAD_DIM and page_size >= 8 and page_size & (page_size - 1) == 0
+
+
+#: blocks (pairs of 256-row tiles times kv heads) from which the prefill kernel's tiles have 256 rows instead of 128:
+#: three quarters of the 256 compute units (measured: 7 % faster at 192 blocks, 15 % at 256, 26 % slower at 128)
+PREFILL_WIDE_TILES_MIN_BLOCKS = 192
+
+
+def prefill_tile_rows(d: int, rows_of_entries, n_kv: int) -> int:
+    """Rows of the tiles that entries with many rows are cut into: 256 for head sizes 64 and 128 when that still gives
+    enough blocks to fill the chip (a block takes two tiles of one kv head), else 128.  ``rows_of_entries``: the rows
+    (tokens times heads of a group) of every entry that goes to the prefill kernel."""
+    if d not in (64, 128):
+        return 128
+    tiles = sum(-(-int(r) // 256) for r in rows_of_entries)
+    return 256 if (tiles + 1) // 2 * n_kv >= PREFILL_WIDE_TILES_MIN_BLOCKS else 128
 
 
 def mfma_attention_ok(dtype, d: int, page_size: int) -> bool:
@@ -599,11 +615,12 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
             bsplits = 1
             if n_big * n_kv < PREFILL_SPLIT_BELOW:
                 bsplits = max(1, min(PREFILL_SPLIT_BELOW * 2 // (n_big * n_kv), meta.max_kv_len // 256, 16))
-            bws_floats = hip().lib.spy_attention_prefill_workspace(ctypes.c_int(n_big), ctypes.c_int(n_kv), ctypes.c_int(d),
-                                                                   ctypes.c_int(bsplits))
+            _check(meta.big_rows in (128, 256), "paged_attention: tiles of 128 or 256 rows expected")
+            bws_floats = hip().lib.spy_attention_prefill_workspace(ctypes.c_int(n_big), ctypes.c_int(meta.big_rows), ctypes.c_int(n_kv),
+                                                                   ctypes.c_int(d), ctypes.c_int(bsplits))
             bws = torch.empty((max(1, bws_floats),), dtype=torch.float32, device=q.device)
             hip().call("spy_attention_prefill", _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), *common, _ptr(big_entry),
-                       _ptr(big_row0), ctypes.c_int(n_big), *sizes, ctypes.c_int(bsplits), _ptr(bws), _Hip.stream())
+                       _ptr(big_row0), ctypes.c_int(n_big), ctypes.c_int(meta.big_rows), *sizes, ctypes.c_int(bsplits), _ptr(bws), _Hip.stream())
         if n_small:
             # Few 16-row tiles cannot fill the chip by themselves (decoding requests, short portions): their keys are
             # split into parts, each part a block of 4 waves that wants 128 keys at least, and a second kernel merges.

@@ -24,22 +24,22 @@ from .base import Mixer, PositionEncoding
 
 
 ROWS_PER_TILE = 16        # rows of (token, head-in-group) pairs in a small attention tile
-ROWS_PER_BIG_TILE = 128   # rows in a tile of the prefill attention kernel
 BIG_MIN_ROWS = 64         # entries with at least this many rows go to the prefill kernel
 
 
-def plan_attention_tiles(batch, group_size: int, big_tiles: bool = True) -> None:
+def plan_attention_tiles(batch, group_size: int, big_rows: int = 0) -> None:
     """Adds to the step's arrays the tiles over each entry's rows (token-major, head-in-group minor) for a query-head
-    group of ``group_size``: entries with at least BIG_MIN_ROWS rows are cut into 128-row tiles (the LDS-sharing
-    prefill kernel), the others into 16-row tiles (one block of waves each).  Once per step and group size."""
-    note = ("attention_tiles", group_size)
+    group of ``group_size``: entries with at least BIG_MIN_ROWS rows are cut into tiles of ``big_rows`` rows (the
+    LDS-sharing prefill kernel; 0: never), the others into 16-row tiles (one block of waves each).  Once per step,
+    group size and tile size."""
+    note = ("attention_tiles", group_size, big_rows)
     if note in batch.shared:
         return
     S, lens = batch.S, batch.lens
     rows = lens.astype(np.int64) * group_size
-    big = (rows >= BIG_MIN_ROWS) & bool(big_tiles)
+    big = (rows >= BIG_MIN_ROWS) & bool(big_rows)
     counts = {}
-    for kind, size, mask in (("small", ROWS_PER_TILE, ~big), ("big", ROWS_PER_BIG_TILE, big)):
+    for kind, size, mask in (("small", ROWS_PER_TILE, ~big), ("big", max(big_rows, 1), big)):
         ntiles = np.where(mask, (rows + size - 1) // size, 0)
         tile_entry = np.repeat(np.arange(S, dtype=np.int32), ntiles)
         first = np.zeros(S + 1, dtype=np.int64)
@@ -52,27 +52,28 @@ def plan_attention_tiles(batch, group_size: int, big_tiles: bool = True) -> None
             order = np.argsort(-(pos0 + last_tok), kind="stable")
             tile_entry, tile_row0 = tile_entry[order], tile_row0[order]
         counts[kind] = int(first[-1])
-        batch.add_array("tile_entry_%s_%d" % (kind, group_size), tile_entry)
-        batch.add_array("tile_row0_%s_%d" % (kind, group_size), tile_row0)
+        batch.add_array("tile_entry_%s_%d_%d" % (kind, group_size, big_rows), tile_entry)
+        batch.add_array("tile_row0_%s_%d_%d" % (kind, group_size, big_rows), tile_row0)
     batch.shared[note] = counts
     # the 16-row tiles' keys are split into a number of parts that follows the longest request: a launch shape
     batch.add_graph_key("attention_key_parts", ops.key_parts_for(batch.max_kv_len))
 
 
-def attention_meta(batch, group: int, group_size: int) -> ops.AttentionMeta:
+def attention_meta(batch, group: int, group_size: int, big_rows: int = 0) -> ops.AttentionMeta:
     """The step's description for the attention kernels, from the batch's arrays on the device (one object per step,
-    cache group and group size)."""
-    note = ("attention_meta", group, group_size)
+    cache group, group size and tile size)."""
+    note = ("attention_meta", group, group_size, big_rows)
     meta = batch.shared.get(note)
     if meta is None:
         tiles = None
-        counts = batch.shared.get(("attention_tiles", group_size))
+        counts = batch.shared.get(("attention_tiles", group_size, big_rows))
         if counts is not None:
-            tiles = {kind: (batch.array("tile_entry_%s_%d" % (kind, group_size)), batch.array("tile_row0_%s_%d" % (kind, group_size)), n)
-                     for kind, n in counts.items()}
+            tiles = {kind: (batch.array("tile_entry_%s_%d_%d" % (kind, group_size, big_rows)),
+                            batch.array("tile_row0_%s_%d_%d" % (kind, group_size, big_rows)), n) for kind, n in counts.items()}
         meta = ops.AttentionMeta(batch.array("cu_q"), batch.array("pos0"), batch.array("kv_len"), batch.block_table(group),
                                  batch.array("token_entry"), batch.array("positions"), batch.S, batch.T, batch.max_blocks[group],
-                                 batch.max_kv_len, batch.max_q_len, tiles, group_size, fixed_shape=batch.fixed_shape)
+                                 batch.max_kv_len, batch.max_q_len, tiles, group_size, fixed_shape=batch.fixed_shape,
+                                 big_rows=big_rows or 128)
         batch.shared[note] = meta
     return meta
 
@@ -123,7 +124,18 @@ class PagedAttention(Mixer):
         return PagedKV(self.num_kv_heads, self.head_dim, self.window)
 
     def plan(self, batch) -> None:
-        plan_attention_tiles(batch, self.num_heads // self.num_kv_heads, ops.prefill_attention_ok(self.head_dim, batch.page_size))
+        plan_attention_tiles(batch, self.num_heads // self.num_kv_heads, self._big_rows(batch, batch.page_size))
+
+    def _big_rows(self, batch, page_size: int) -> int:
+        """Rows of the tiles for this step's entries with many rows; 0 if the prefill kernel does not take this head
+        size or page."""
+        if not ops.prefill_attention_ok(self.head_dim, page_size):
+            return 0
+        note = ("attention_big_rows", self.num_heads, self.num_kv_heads, self.head_dim)
+        if note not in batch.shared:
+            rows = batch.lens.astype(np.int64) * (self.num_heads // self.num_kv_heads)
+            batch.shared[note] = ops.prefill_tile_rows(self.head_dim, rows[rows >= BIG_MIN_ROWS], self.num_kv_heads)
+        return batch.shared[note]
 
     # ---- step ------------------------------------------------------------
     def can_fold(self, batch):
@@ -138,7 +150,7 @@ class PagedAttention(Mixer):
         rot = self.position.rotary() if self.position is not None else None
         cos, sin, rdim = rot if rot is not None else (None, None, 0)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
-        meta = attention_meta(batch, cache.group, nq // nkv)
+        meta = attention_meta(batch, cache.group, nq // nkv, self._big_rows(batch, cache.page_size))
         if ops.fused_attention_ok(qkv.dtype, meta, nq, nkv, d, cache.page_size, rdim, self.q_norm, self.k_norm):
             # single tokens only: the attention kernel norms, rotates and stores by itself
             raw = ops.RawQKV(qkv, self.q_norm, self.k_norm, eps, cos if rdim else None, sin if rdim else None, store)

@@ -352,7 +352,7 @@ def plain_paged_attention(q, kc, vc, P, bt, token_entry, positions, n_q, n_kv, d
     return out.view(T, n_q * d)
 
 
-def make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed, window=None, spike=False):
+def make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed, window=None, spike=False, big_rows=128):
     """entries: list of (tokens already cached, tokens in this step).  Pages are dealt in a random
     order; unused pages and slots hold NaN."""
     from spyinfer_amd.kernels.ops import AttentionMeta
@@ -386,7 +386,7 @@ def make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed, window=None,
     G = n_q // n_kv
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
     tiles = {}
-    for kind, size in (("small", 16), ("big", 128)):
+    for kind, size in (("small", 16), ("big", big_rows)):
         tile_entry, tile_row0 = [], []
         for s, (a, n) in enumerate(entries):
             is_big = n * G >= 64 and d <= 128 and P & (P - 1) == 0
@@ -395,7 +395,7 @@ def make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed, window=None,
                     tile_entry.append(s); tile_row0.append(r0)
         tiles[kind] = (i32(tile_entry), i32(tile_row0), len(tile_entry))
     meta = AttentionMeta(i32(cu), i32(pos0), i32(kvl), i32(bt), i32(te), i32(ps), len(entries), T, maxb, max(kvl),
-                         max(n for _, n in entries), tiles, G)
+                         max(n for _, n in entries), tiles, G, big_rows=big_rows)
     return q, kc, vc, bt, te, ps, meta
 
 
@@ -422,18 +422,26 @@ ATT_CASES = [
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("case", range(len(ATT_CASES)))
-@pytest.mark.parametrize("mfma", [False, True])
+@pytest.mark.parametrize("mfma", [False, True, 256])
 def test_paged_attention(dtype, case, mfma):
+    """mfma: False = the float32 kernel, True = the MFMA kernels with 128-row tiles for entries of many rows, 256 = the
+    same with 256-row tiles (head sizes 64 and 128)."""
     from spyinfer_amd.kernels import ops
     dev = require_gpu()
     n_q, n_kv, d, P, entries, window = ATT_CASES[case]
     if mfma and not (dtype == torch.bfloat16 and d % 16 == 0 and P % 8 == 0):
         pytest.skip("the MFMA kernel takes bfloat16, head sizes in steps of 16 and pages of a multiple of 8")
-    q, kc, vc, bt, te, ps, meta = make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed=case, window=window, spike=True)
+    big_rows = 128
+    if mfma == 256:
+        if d not in (64, 128) or P & (P - 1) or not any(n * (n_q // n_kv) >= 64 for _, n in entries):
+            pytest.skip("tiles of 256 rows are for head sizes 64 and 128 and entries of many rows")
+        big_rows = 256
+    q, kc, vc, bt, te, ps, meta = make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed=case, window=window, spike=True,
+                                                      big_rows=big_rows)
     scale = 1.0 / math.sqrt(d)
     ref = plain_paged_attention(q, kc, vc, P, bt, te, ps, n_q, n_kv, d, scale, window)
     old = ops.MFMA_ATTENTION
-    ops.MFMA_ATTENTION = mfma
+    ops.MFMA_ATTENTION = bool(mfma)
     try:
         out = ops.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), P, meta, n_q, n_kv, d, scale, window)
     finally:
@@ -441,7 +449,7 @@ def test_paged_attention(dtype, case, mfma):
     close(out, ref, dtype, scale=2.0, what="attention case %d" % case)
 
 
-def _long_case(dtype, dev, n_q, n_kv, d, P, entries, seed):
+def _long_case(dtype, dev, n_q, n_kv, d, P, entries, seed, big_rows=128):
     """As make_attention_case, for thousands of keys: filled and gathered with tensor operations.  Returns also the
     keys and values of each entry in order, for the reference."""
     from spyinfer_amd.kernels.ops import AttentionMeta
@@ -473,7 +481,7 @@ def _long_case(dtype, dev, n_q, n_kv, d, P, entries, seed):
     G = n_q // n_kv
     i32 = lambda x: torch.as_tensor(x, dtype=torch.int32).to(dev)
     tiles = {}
-    for kind, size in (("small", 16), ("big", 128)):
+    for kind, size in (("small", 16), ("big", big_rows)):
         te, tr = [], []
         for s, (a, n) in enumerate(entries):
             if (n * G >= 64) == (kind == "big"):
@@ -486,21 +494,23 @@ def _long_case(dtype, dev, n_q, n_kv, d, P, entries, seed):
     token_entry = [s for s, (a, n) in enumerate(entries) for _ in range(n)]
     positions = [a + i for a, n in entries for i in range(n)]
     meta = AttentionMeta(i32(cu), i32([a for a, n in entries]), i32([a + n for a, n in entries]), i32(bt), i32(token_entry),
-                         i32(positions), len(entries), cu[-1], maxb, max(a + n for a, n in entries), max(n for _, n in entries), tiles, G)
+                         i32(positions), len(entries), cu[-1], maxb, max(a + n for a, n in entries), max(n for _, n in entries), tiles, G,
+                         big_rows=big_rows)
     return q, kc, vc, kept, cu, meta
 
 
 @pytest.mark.parametrize("case", [(32, 8, 128, 16, [(9000, 1), (8191, 1), (4000, 1)]),        # 16 key parts and the merge
                                   (8, 2, 128, 16, [(8800, 200), (0, 300)]),                   # few 128-row tiles far into a request: key parts
                                   (16, 2, 64, 32, [(9100, 70), (5000, 1)])])                   # both kernels in one step
-def test_paged_attention_over_9000_keys(case):
+@pytest.mark.parametrize("big_rows", [128, 256])
+def test_paged_attention_over_9000_keys(case, big_rows):
     """The lengths that the benchmarks run (15 000-key decode steps, portions late in 16 000-token prompts): block tables
     of hundreds of pages, the most key parts, tiles sorted by work.  Reference: float64 softmax over the entry's keys."""
     from spyinfer_amd.kernels import ops
     dev = require_gpu()
     n_q, n_kv, d, P, entries = case
     dtype = torch.bfloat16
-    q, kc, vc, kept, cu, meta = _long_case(dtype, dev, n_q, n_kv, d, P, entries, seed=len(entries) + n_q)
+    q, kc, vc, kept, cu, meta = _long_case(dtype, dev, n_q, n_kv, d, P, entries, seed=len(entries) + n_q, big_rows=big_rows)
     assert ops.key_parts_for(meta.max_kv_len) == 16
     scale = 1.0 / math.sqrt(d)
     out = ops.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), P, meta, n_q, n_kv, d, scale, None).cpu().double()

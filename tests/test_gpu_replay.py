@@ -64,6 +64,25 @@ def test_replay_matches_plain(dtype, name, mode, models, tmp_path, monkeypatch):
     assert bool(folded) == (name in "DE" and dtype == "bfloat16")
 
 
+@pytest.mark.parametrize("name", ["D", "E"])
+@pytest.mark.parametrize("mode", ["whole", "portions", "mixed"])
+def test_replay_with_tiles_of_256_rows(name, mode, models, tmp_path, monkeypatch):
+    """Prompts long enough to fill the chip are cut into attention tiles of 256 rows instead of 128 (head sizes 64 and
+    128: configurations D and E).  Here the threshold is lowered so that the tests' prompts take them."""
+    require_gpu()
+    from spyinfer_amd.kernels import ops
+    monkeypatch.setattr(ops, "PREFILL_WIDE_TILES_MIN_BLOCKS", 1)
+    seen = []
+    real = ops.paged_attention
+    monkeypatch.setattr(ops, "paged_attention", lambda *a, **k: (seen.append((a[4].big_rows, a[4].tiles["big"][2])), real(*a, **k))[1])
+    cfg, lengths, page = CASES[name]
+    folder, reqs, ref = models[name]
+    steps = getattr(rc, mode)(reqs)
+    rc.run_replay_inprocess(folder, "bfloat16", str(tmp_path), steps, rc.max_live_tokens(steps), ["--kvcache-block-size", str(page)])
+    rc.compare(rc.collect(str(tmp_path), steps, cfg["vocab_size"]), ref, what="256-row tiles/%s/%s" % (name, mode), **TOL["bfloat16"])
+    assert any(rows == 256 and n > 0 for rows, n in seen) or mode != "whole"
+
+
 def _count_pages_handed_out(monkeypatch):
     """{page: times it was handed out} over all pools made from now on."""
     from spyinfer_amd.cache.pages import PagePool
