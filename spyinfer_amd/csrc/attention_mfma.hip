@@ -122,7 +122,15 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     int n_q, int n_kv, int d, float scale, int window, int splits, float* __restrict__ ws, FusedQKV fz, int out_tiles) {
     constexpr int KK = DMAX / 32;   // 32-wide chunks of the head dim for Q.K
     constexpr int DT = DMAX / 16;   // 16-row tiles of the head dim for P.V
-    extern __shared__ float lds[];   // (AW - 1) * (DT * 4 + 2) * 64 floats: the other waves' O, m, l
+    extern __shared__ float lds[];   // the waves' O, m, l: AW (head sizes up to 128) or AW - 1 times (DT * 4 + 2) * 64 floats
+#ifdef AM_TIMING
+    long long tstamp[8];
+    int nstamp = 0;
+#define AM_STAMP(dep) { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); tstamp[nstamp++] = clock64() + ((dep) & 0); }
+    AM_STAMP(0)
+#else
+#define AM_STAMP(dep)
+#endif
     const int tile = blockIdx.x, hk = blockIdx.y, sp = blockIdx.z;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: loops over it stay scalar
     const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
@@ -164,6 +172,7 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     const int per = (nblk + splits - 1) / splits;
     const int b_begin = sp * per, b_end = min(nblk, b_begin + per);
 
+    AM_STAMP(nblk)      // 1: the entry's description and the query row are there
     f32x4_t acc[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -171,18 +180,22 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
 
     // FUSED: the entry's one new token lies at position p0 = kvl - 1; its query rows have that position too.  The block
     // whose keys reach it prepares the new key (every lane its pieces for its g, as for q) and takes the new value's
-    // elements of its rows dd.  All loads of this preparation are issued together, before anything waits for them.
+    // elements of its rows dd.
+    // The kernel's start is a chain of memory round trips (about a microsecond each when the step's weights have swept
+    // the caches), so loads are issued in the order of what they depend on, each group together and ahead of any wait:
+    // what depends on the block alone (raw k and v, the norm weights; the raw query row is on its way already), then
+    // what needs the entry's position (rotation table, pages), then the first keys (they need the pages); the norm and
+    // the rotation are worked out while the keys are on their way.
     const int newpos = p0;
     bool has_new = false;
     bf16x8_t knew[KK];
     bf16_t vnew[DT];
     int new_page = -1;
-    if (FUSED) {
-        constexpr int HK = KK / 2;
-        has_new = fz.store && n == 1 && newpos >= lo + 32 * b_begin && newpos < lo + 32 * b_end;
-        const bool normed = fz.qw != nullptr, rotated = fz.cos_t != nullptr;
-        float wq[KK][8], wk[KK][8], cs[HK][8], sn[HK][8];
-        if (has_new) {
+    constexpr int HKF = FUSED ? KK / 2 : 1;
+    float wq[FUSED ? KK : 1][8], wk[FUSED ? KK : 1][8], cs[HKF][8], sn[HKF][8];
+    const bool normed = FUSED && fz.qw != nullptr, rotated = FUSED && fz.cos_t != nullptr;
+    if constexpr (FUSED) {
+        if (fz.store) {
             const bf16_t* base = fz.qkv + (size_t)q0 * (n_q + 2 * n_kv) * d;
             const bf16_t* kp_raw = base + (size_t)(n_q + hk) * d;
             const bf16_t* vp_raw = base + (size_t)(n_q + n_kv + hk) * d;
@@ -190,29 +203,12 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
             for (int kk = 0; kk < KK; ++kk) knew[kk] = *reinterpret_cast<const bf16x8_t*>(kp_raw + kk * 32 + 8 * g);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) vnew[dt] = vp_raw[dt * 16 + r16];
-            new_page = bt[newpos / P];
             if (normed) load_weight_pieces<KK>(wk, fz.kw, fz.w_dtype, g);
         }
         if (normed) load_weight_pieces<KK>(wq, fz.qw, fz.w_dtype, g);
-        if (rotated) {
-            const size_t trow = (size_t)min(newpos, fz.max_pos - 1) * (d / 2);
-#pragma unroll
-            for (int kk = 0; kk < HK; ++kk) {
-                const f32x4_t c0 = *reinterpret_cast<const f32x4_t*>(fz.cos_t + trow + kk * 32 + 8 * g);
-                const f32x4_t c1 = *reinterpret_cast<const f32x4_t*>(fz.cos_t + trow + kk * 32 + 8 * g + 4);
-                const f32x4_t s0 = *reinterpret_cast<const f32x4_t*>(fz.sin_t + trow + kk * 32 + 8 * g);
-                const f32x4_t s1 = *reinterpret_cast<const f32x4_t*>(fz.sin_t + trow + kk * 32 + 8 * g + 4);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) { cs[kk][e] = c0[e]; cs[kk][e + 4] = c1[e]; sn[kk][e] = s0[e]; sn[kk][e + 4] = s1[e]; }
-            }
-        }
-        norm_rotate<KK>(bq, normed, wq, fz.eps, rotated, cs, sn, d);
-        if (has_new) {
-            norm_rotate<KK>(knew, normed, wk, fz.eps, rotated, cs, sn, d);
-            if (new_page < 0 || new_page >= num_pages) has_new = false;   // no page: nothing to store or to use
-        }
+        __builtin_amdgcn_sched_barrier(0);
+        has_new = fz.store && n == 1 && newpos >= lo + 32 * b_begin && newpos < lo + 32 * b_end;
     }
-
     // A wave's loop is a chain of memory round trips, so they are overlapped: pages are looked up two blocks ahead (both
     // lookups together); the keys of the next block are asked for as soon as this block's S^T products have read the
     // key registers, and arrive while the softmax and the second product run; the values are asked for at the top of
@@ -253,7 +249,33 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     }
     AM_LOOKUP(b_begin + wave, kpage, vpage)
     AM_LOOKUP(b_begin + wave + AW, kpage_n, vpage_n)
+    if constexpr (FUSED) {
+        if (has_new) new_page = bt[newpos / P];
+        if (rotated) {
+            const size_t trow = (size_t)min(newpos, fz.max_pos - 1) * (d / 2);
+#pragma unroll
+            for (int kk = 0; kk < HKF; ++kk) {
+                const f32x4_t c0 = *reinterpret_cast<const f32x4_t*>(fz.cos_t + trow + kk * 32 + 8 * g);
+                const f32x4_t c1 = *reinterpret_cast<const f32x4_t*>(fz.cos_t + trow + kk * 32 + 8 * g + 4);
+                const f32x4_t s0 = *reinterpret_cast<const f32x4_t*>(fz.sin_t + trow + kk * 32 + 8 * g);
+                const f32x4_t s1 = *reinterpret_cast<const f32x4_t*>(fz.sin_t + trow + kk * 32 + 8 * g + 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { cs[kk][e] = c0[e]; cs[kk][e + 4] = c1[e]; sn[kk][e] = s0[e]; sn[kk][e + 4] = s1[e]; }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    AM_STAMP(kpage)     // 3: pages looked up
     if (b_begin + wave < b_end) AM_LOAD_K(b_begin + wave, kpage)
+    if constexpr (FUSED) {
+        __builtin_amdgcn_sched_barrier(0);
+        norm_rotate<KK>(bq, normed, wq, fz.eps, rotated, cs, sn, d);
+        if (has_new) {
+            norm_rotate<KK>(knew, normed, wk, fz.eps, rotated, cs, sn, d);
+            if (new_page < 0 || new_page >= num_pages) has_new = false;   // no page: nothing to store or to use
+        }
+    }
+    AM_STAMP(kpage)     // 4: first keys there
     // One block of 32 keys.  LAST: the wave's last block, which alone can hold keys beyond the request's and the step's
     // new key, and after which no keys are asked for; the blocks before it have no condition around their loads.
     auto block = [&](const int b, auto last_block) {
@@ -364,13 +386,50 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     }
 #undef AM_LOOKUP
 #undef AM_LOAD_K
+    AM_STAMP(0)         // 5: key blocks done
     // the four lanes of a row hold partial sums of l
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
 
-    // merge the waves of the block: wave 0 takes the others' (O, m, l) from LDS, lane for lane
-    {
-        constexpr int PER = DT * 4 + 2;
+    // Merge the waves of the block.  Every wave puts its (O, m, l) into LDS, lane for lane (O as vectors of four), and
+    // then merges and writes out its share of the head dim's tiles: DT / AW tiles of every wave's O.  (For head sizes
+    // beyond 128 the four waves' sums do not fit the LDS that a block may ask for: there wave 0 merges them all.)
+    constexpr int PER = DT * 4 + 2;
+    constexpr bool SPREAD = DMAX <= 128;
+    constexpr int MINE = SPREAD ? DT / AW : DT;       // tiles of the head dim that this wave merges
+    static_assert(!SPREAD || DT % AW == 0, "the head dim's tiles are dealt evenly to the waves");
+    const int dt0 = SPREAD ? wave * MINE : 0;
+    f32x4_t mo[MINE];
+    if (SPREAD) {
+        float* mine = lds + (size_t)wave * PER * 64;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4_t*>(mine + (dt * 64 + lane) * 4) = acc[dt];
+        mine[(DT * 4) * 64 + lane] = m;
+        mine[(DT * 4 + 1) * 64 + lane] = l;
+        __syncthreads();
+        float mw[AW], lw[AW];
+        float mn = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < AW; ++w) {
+            mw[w] = lds[((size_t)w * PER + DT * 4) * 64 + lane];
+            lw[w] = lds[((size_t)w * PER + DT * 4 + 1) * 64 + lane];
+            mn = fmaxf(mn, mw[w]);
+        }
+        l = 0.f;
+#pragma unroll
+        for (int i = 0; i < MINE; ++i) mo[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < AW; ++w) {                 // in the order of the waves, whichever wave adds
+            const float a = (mw[w] == -INFINITY) ? 0.f : __expf(mw[w] - mn);
+            l += lw[w] * a;
+#pragma unroll
+            for (int i = 0; i < MINE; ++i) {
+                const f32x4_t o = *reinterpret_cast<const f32x4_t*>(lds + (((size_t)w * PER * 64) + ((dt0 + i) * 64 + lane) * 4));
+                mo[i] += o * a;
+            }
+        }
+        m = mn;
+    } else {
         if (wave > 0) {
             float* mine = lds + (size_t)(wave - 1) * PER * 64;
 #pragma unroll
@@ -385,12 +444,12 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
 #pragma unroll
         for (int w = 1; w < AW; ++w) {
             const float* other = lds + (size_t)(w - 1) * PER * 64;
-            const float mo = other[(DT * 4) * 64 + lane];
+            const float mo_ = other[(DT * 4) * 64 + lane];
             const float lo_ = other[(DT * 4 + 1) * 64 + lane];
-            const float mn = fmaxf(m, mo);
+            const float mn = fmaxf(m, mo_);
             if (mn == -INFINITY) continue;
             const float a = (m == -INFINITY) ? 0.f : __expf(m - mn);
-            const float bsc = (mo == -INFINITY) ? 0.f : __expf(mo - mn);
+            const float bsc = (mo_ == -INFINITY) ? 0.f : __expf(mo_ - mn);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -398,19 +457,27 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
             l = l * a + lo_ * bsc;
             m = mn;
         }
+#pragma unroll
+        for (int i = 0; i < MINE; ++i) mo[i] = acc[i];
     }
 
+    AM_STAMP(0)         // 6: waves merged
+#ifdef AM_TIMING
+    if (tile == 0 && hk == 0 && sp == 0 && threadIdx.x == 0 && ws) {
+        for (int i = 0; i < nstamp; ++i) reinterpret_cast<long long*>(ws)[i] = tstamp[i];
+    }
+#endif
     if (splits == 1) {
         if (!row_ok) return;
         const float inv = l > 0.f ? 1.0f / l : 0.f;
         bf16_t* op = out + ((size_t)(q0 + tq) * n_q + head) * d;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const int dd = dt * 16 + 4 * g;
+        for (int i = 0; i < MINE; ++i) {
+            const int dd = (dt0 + i) * 16 + 4 * g;
             if (dd < d) {
                 uint2 w;
-                w.x = pack_bf16x2(acc[dt][0] * inv, acc[dt][1] * inv);
-                w.y = pack_bf16x2(acc[dt][2] * inv, acc[dt][3] * inv);
+                w.x = pack_bf16x2(mo[i][0] * inv, mo[i][1] * inv);
+                w.y = pack_bf16x2(mo[i][2] * inv, mo[i][3] * inv);
                 // (four columns from a multiple of 4 never cross a group of 8: one store either way)
                 if (out_tiles) *reinterpret_cast<uint2*>(out + attention_out_operand_order(q0 + tq, head * d + dd, out_tiles)) = w;
                 else *reinterpret_cast<uint2*>(op + dd) = w;
@@ -421,11 +488,11 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     // partial result: ws[((tile * n_kv + hk) * splits + sp)] = { O[16][DMAX], m[16], l[16] }
     float* w = ws + (((size_t)tile * n_kv + hk) * splits + sp) * (16 * (DMAX + 2));
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-        const int dd = dt * 16 + 4 * g;
-        *reinterpret_cast<f32x4_t*>(w + r16 * DMAX + dd) = acc[dt];
+    for (int i = 0; i < MINE; ++i) {
+        const int dd = (dt0 + i) * 16 + 4 * g;
+        *reinterpret_cast<f32x4_t*>(w + r16 * DMAX + dd) = mo[i];
     }
-    if (g == 0) {
+    if (g == 0 && wave == 0) {
         w[16 * DMAX + r16] = m;
         w[16 * DMAX + 16 + r16] = l;
     }
@@ -473,7 +540,7 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
     const dim3 grid(num_tiles, n_kv, splits);
     const dim3 mgrid(num_tiles, n_kv);
 #define ATT_LAUNCH(DM, FZ, FL)                                                                                                \
-    attention_mfma_kernel<DM, FZ, FL><<<grid, AW * 64, (AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>(                \
+    attention_mfma_kernel<DM, FZ, FL><<<grid, AW * 64, (DM <= 128 ? AW : AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>(  \
         (bf16_t*)out, (const bf16_t*)q, (bf16_t*)kc, (bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,  \
         tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz, out_tiles)
 #define ATT_CASE(DM)                                                                                                          \

@@ -8,6 +8,7 @@ beside single decoded tokens, cut anywhere.
 """
 from __future__ import annotations
 
+import gc
 from typing import List, Optional, Sequence
 
 import torch
@@ -218,8 +219,19 @@ class ModelRunner:
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
         out = self._graph_logits[:batch.R] if batch.R <= self.max_num_seqs else None
-        with torch.cuda.graph(graph, pool=self._graph_pool):
-            logits = self.model.forward(batch, self.storage, out)
+        # Python's cycle collector must not run inside the capture: what it frees there (dead engines, their graphs and
+        # memory pools, pinned buffers) frees device memory and queries events, which HIP forbids while a stream
+        # captures, and the error, raised inside a destructor, ends the process.  So dead cycles are collected now,
+        # and the collector rests until the capture is over.
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                logits = self.model.forward(batch, self.storage, out)
+        finally:
+            if collecting:
+                gc.enable()
         self._graphs[key] = (graph, dev_buf, logits)
         graph.replay()                          # capture launches nothing: this replay is the step
         self.graph_replays += 1

@@ -196,6 +196,41 @@ def test_captured_steps_share_their_memory():
     assert runner.graph_memory_bound() >= 4 * R * V
 
 
+def test_no_garbage_collection_inside_a_capture(folder_a):
+    """While a step is captured as a graph Python's cycle collector rests, and dead cycles are collected just before: a
+    dead engine freed inside a capture (its graphs, pools and pinned buffers) makes calls that HIP forbids while a
+    stream captures, which ended the process.  Here a dead engine with captured graphs lies in a reference cycle when
+    the next engine captures; the model's forward records what it sees."""
+    import gc
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    require_gpu()
+    ps = prompts(256, [9, 30], 5)
+    sp = SamplingParams(max_new_tokens=6, ignore_eos=True)
+    kw = dict(dtype="bfloat16", max_model_len=128, num_kvcache_blocks=40)
+    dead = LLMEngine(folder_a, **kw)
+    dead.generate(ps, sp)
+    assert dead.runner._graphs
+    dead.cycle = dead                                     # only the cycle collector can free it now
+    del dead
+    eng = LLMEngine(folder_a, **kw)
+    seen = []
+    real = eng.model.forward
+
+    def forward(batch, storage, logits_out=None):
+        if torch.cuda.is_current_stream_capturing():
+            seen.append(gc.isenabled())
+        return real(batch, storage, logits_out)
+    eng.model.forward = forward
+    try:
+        assert gc.isenabled()
+        eng.generate(ps, sp)
+        assert seen and not any(seen), "the collector ran free inside %d of %d captures" % (sum(seen), len(seen))
+        assert gc.isenabled()
+    finally:
+        eng.model.forward = real
+
+
 def test_number_of_graphs_is_bounded(folder_a):
     """The runner captures a bounded number of step shapes (each captured step holds its activations); with room for
     two, a run whose batch shrinks from four requests to one runs its later shapes kernel by kernel and still gives
