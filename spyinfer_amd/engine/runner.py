@@ -221,9 +221,9 @@ class ModelRunner:
         out = self._graph_logits[:batch.R] if batch.R <= self.max_num_seqs else None
         # Python's cycle collector must not run inside the capture: what it frees there (dead engines, their graphs and
         # memory pools, pinned buffers) frees device memory and queries events, which HIP forbids while a stream
-        # captures, and the error, raised inside a destructor, ends the process.  So dead cycles are collected now,
-        # and the collector rests until the capture is over.
-        gc.collect()
+        # captures, and the error, raised inside a destructor, ends the process.  So the collector rests until the
+        # capture is over (dead cycles wait for its next turn; collecting them here, before every capture, cost a serving
+        # run with a hundred shapes more than the captures themselves).
         collecting = gc.isenabled()
         gc.disable()
         try:

@@ -165,11 +165,10 @@ def default_fold_rows(weight_elements: int) -> int:
     """Most rows of a step for which a part with ``weight_elements`` matrix elements should run its products with the
     norms and residual sums folded in (above: the library product with norm kernels of their own), where the part's
     builder names no limit.  Measured on MI355X: such products beat the library's by 16 % at 32 rows and are level with
-    it at 64 rows; with four row tiles (49 to 64 rows) the products themselves are 8-12 % slower than the library's (every
-    block reads all of X) and the step gains only by the norm and SwiGLU kernels it does not run, a fixed time per layer.
-    With 151 M elements in a feed-forward the step at 64 rows gains 1.5 %, with 393 M it loses 5 %: parts with more than
-    2^28 elements fold up to 48 rows only."""
-    return 48 if weight_elements > (1 << 28) else FUSED_DECODE_MAX_ROWS
+    it at 64 rows, where the step still gains by the norm and SwiGLU kernels it does not run: 1.5 % at the Qwen3-8B
+    shape, 1.7 % at the 32B shape (5.5 % at 56 rows) since the gated product walks runs of column tiles.  So: as many
+    rows as the decode products take, whatever the size."""
+    return FUSED_DECODE_MAX_ROWS
 
 
 def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:

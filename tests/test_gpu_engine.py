@@ -197,7 +197,7 @@ def test_captured_steps_share_their_memory():
 
 
 def test_no_garbage_collection_inside_a_capture(folder_a):
-    """While a step is captured as a graph Python's cycle collector rests, and dead cycles are collected just before: a
+    """While a step is captured as a graph Python's cycle collector rests: a
     dead engine freed inside a capture (its graphs, pools and pinned buffers) makes calls that HIP forbids while a
     stream captures, which ended the process.  Here a dead engine with captured graphs lies in a reference cycle when
     the next engine captures; the model's forward records what it sees."""
@@ -370,8 +370,7 @@ def test_folded_decode_steps(tmp_path_factory):
 def test_folded_decode_steps_of_many_requests(tmp_path_factory, requests):
     """Decode steps of 17 to 64 requests take the folded products with two to four row tiles (70 requests: the library's); their logits equal, up to
     bfloat16 rounding, those of the same steps with the norms as kernels of their own, from graphs as well, and the last
-    step's equal the plain implementation's.  Parts may be built to fold up to fewer rows (48 here, as parts with large
-    matrices are): the embedding then still prepares the first norm's input, which the unfolded block does not use."""
+    step's equal the plain implementation's.  Parts may be built to fold up to fewer rows (48 here): the embedding then still prepares the first norm's input, which the unfolded block does not use."""
     from spyinfer_amd.engine.batch import StepEntry
     from spyinfer_amd.engine.runner import ModelRunner, load_model
     from spyinfer_amd.kernels import ops
@@ -383,7 +382,7 @@ def test_folded_decode_steps_of_many_requests(tmp_path_factory, requests):
     ps = prompts(400, [3 + (7 * i) % 23 for i in range(requests)], 5)
     runs, calls = [], []
     real = ops.decode_linear_residual
-    assert ops.default_fold_rows(1 << 20) == 64 and ops.default_fold_rows((1 << 28) + 1) == 48
+    assert ops.default_fold_rows(1 << 20) == 64
     for folded, eager, fold_rows in ((True, True, None), (True, False, None), (False, True, None), (True, True, 48)):
         ops.FUSED_DECODE = folded
         for layer in model.layers:
