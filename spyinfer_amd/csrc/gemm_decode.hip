@@ -323,12 +323,13 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
 // half a chunk at a time (the accumulators of CT tiles take the registers of the other half); the waves' sums of one
 // column tile are added through LDS by the wave that owns the tile (tile ct -> wave ct), in the order of the waves, and
 // that wave runs the tile's epilogue.  Store and gated epilogues only.
-template <int EPI, bool SCALED, typename TC, int MT, int CT, bool XT, bool OT>
+template <int EPI, bool SCALED, typename TC, int MT, int CT, bool XT, bool OT, int STEPS = 2>
 __global__ __launch_bounds__(512, 1) void gemm_decode_wide_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, const float* __restrict__ ss_in,
     int n_parts, float eps, int M, int N, int K) {
     static_assert(EPI == EPI_STORE || EPI == EPI_GATED, "the wide kernel has no residual epilogue");
     static_assert(CT <= 8, "a wave owns at most one column tile of a group");
+    static_assert((EPI == EPI_GATED ? 2 : 1) * CT * MT <= 24, "the accumulators of a group must fit the registers");
     constexpr int GW = 8;
     constexpr int GATES = EPI == EPI_GATED ? 2 : 1;
     constexpr int NT = GATES * CT;
@@ -383,10 +384,10 @@ __global__ __launch_bounds__(512, 1) void gemm_decode_wide_kernel(
             const char* wb = wbase + (size_t)c * chunk_stride;
             const char* xb = xbase + (size_t)c * (XT ? 4 * MT * 1024 : GD_CHUNK * 2);
 #pragma unroll
-            for (int h = 0; h < 4; h += 2) {
-                bf16x8_t a[NT][2], b[MT][2];
+            for (int h = 0; h < 4; h += STEPS) {
+                bf16x8_t a[NT][STEPS], b[MT][STEPS];
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
+                for (int j = 0; j < STEPS; ++j) {
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt) {
                         // a tile that the group does not have reads the group's first tile again (its sums are dropped)
@@ -400,7 +401,7 @@ __global__ __launch_bounds__(512, 1) void gemm_decode_wide_kernel(
                                             : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
                 }
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < STEPS; ++j)
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -480,6 +481,7 @@ static int compute_units() {
 static int wide_ct(int per, int MT, int gates, int max_ct) {
     int best = 1, best_cost = 1 << 30;
     for (int ct = 1; ct <= max_ct; ++ct) {
+        if (ct == 5) continue;                      // (not built)
         const int cost = ((per + ct - 1) / ct) * MT + per * gates;
         if (cost < best_cost) { best = ct; best_cost = cost; }
     }
@@ -488,20 +490,26 @@ static int wide_ct(int per, int MT, int gates, int max_ct) {
 
 template <int EPI, bool SCALED, typename TC, int MT, bool XT, bool OT>
 static bool gd_launch_wide(const GdArgs& a) {
-    if constexpr (EPI == EPI_RESID) return false;
+    // (only the combination that a decode step has, a normed input in operand order, to keep the library's build short)
+    if constexpr (EPI == EPI_RESID || !SCALED || !XT) return false;
     else {
         constexpr int GATES = EPI == EPI_GATED ? 2 : 1;
-        constexpr int MAX_CT = EPI == EPI_GATED ? 3 : 4;
+        // a group's accumulators (GATES * CT * MT tiles of four registers) leave room for its operands up to 24 tiles
+        constexpr int MAX_CT = 24 / (GATES * MT) < 6 ? 24 / (GATES * MT) : 6;
         const int cus = compute_units(), tiles = a.N / 16;
         if (!GD_WIDE || tiles < 2 * cus) return false;       // fewer than two tiles per CU: one tile per block, two blocks per CU
         const int ct = wide_ct((tiles + cus - 1) / cus, MT, GATES, MAX_CT);
-#define GD_WIDE_ARGS a.x, a.w, (TC*)a.c, a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K
-        if (ct == 1) return false;
-        if (ct == 2) gemm_decode_wide_kernel<EPI, SCALED, TC, MT, 2, XT, OT><<<cus, 512, 0, a.st>>>(GD_WIDE_ARGS);
-        else if (ct == 3) gemm_decode_wide_kernel<EPI, SCALED, TC, MT, 3, XT, OT><<<cus, 512, 0, a.st>>>(GD_WIDE_ARGS);
-        else gemm_decode_wide_kernel<EPI, SCALED, TC, MT, MAX_CT, XT, OT><<<cus, 512, 0, a.st>>>(GD_WIDE_ARGS);
-#undef GD_WIDE_ARGS
-        return true;
+#define GD_WIDE_CASE(C)                                                                                               \
+        if constexpr (C <= MAX_CT) {                                                                                  \
+            if (ct == C) {                                                                                            \
+                gemm_decode_wide_kernel<EPI, SCALED, TC, MT, C, XT, OT><<<cus, 512, 0, a.st>>>(                        \
+                    a.x, a.w, (TC*)a.c, a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K);                                    \
+                return true;                                                                                          \
+            }                                                                                                         \
+        }
+        GD_WIDE_CASE(2) GD_WIDE_CASE(3) GD_WIDE_CASE(4) GD_WIDE_CASE(6)
+#undef GD_WIDE_CASE
+        return false;                                          // one tile at a time: the kernel with a tile per block stands
     }
 }
 
