@@ -18,6 +18,7 @@ typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
 #define PF_KEYS 64       // keys staged per round
+#define PF_DIES 8        // dies (XCDs) of the chip, each with its own L2; blocks go to them in turn
 #define PF_SLACK 8.0f    // a score may exceed the running maximum by 2^8 before the maximum is raised
 
 __device__ __forceinline__ bf16x8_t pf_zero8() { return bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
@@ -50,16 +51,30 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kern
     // A block works on two tiles, one after the other: tile b and tile n - 1 - b of a list that the host
     // has sorted by the number of keys a tile reads.  So every block has about the same work, which a
     // causal prompt's tiles alone (few keys early, many late) do not give.
-    const int hk = blockIdx.y;
+    // Blocks go to the chip's 8 dies in turn, by their number in the grid, and each die has an L2 of its own.  So the
+    // grid's numbers are dealt out again: a die gets a run of blocks that follow each other in (part, kv head, tile)
+    // order, which read the same head's keys and values, and these stay in that die's L2 (with 8 kv heads a die has one
+    // head; dealt out plainly, every die reads every head).  Measured, 32 query heads of 128 in 8 groups: 73.9 -> 71.1
+    // us at 2048 tokens, 176 -> 168 at 4096, 618 -> 602 at 8192, 2376 -> 2320 at 16384.
+    int bx, hk, part;
+    {
+        const int gx = gridDim.x, gy = gridDim.y, n = gx * gy * (int)gridDim.z;
+        const int lin = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
+        const int die = lin % PF_DIES, idx = lin / PF_DIES;
+        const int per = (n + PF_DIES - 1) / PF_DIES, rem = n % PF_DIES;      // the first rem dies have per blocks, the others one fewer
+        const int v = (rem == 0 || die < rem) ? die * per + idx : rem * per + (die - rem) * (per - 1) + idx;
+        bx = v % gx;
+        hk = (v / gx) % gy;
+        part = v / (gx * gy);
+    }
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
     // With key parts (splits > 1: few tiles, many keys, e.g. a late portion of a long prompt) a block has one
     // tile and the rounds of one part; the parts are merged by attention_merge_kernel.
-    const int part = blockIdx.z;
     for (int which = 0; which < 2; ++which) {
-    const int tile = which == 0 ? (int)blockIdx.x : num_tiles - 1 - (int)blockIdx.x;
-    if (which == 1 && (splits > 1 || tile <= (int)blockIdx.x)) break;
+    const int tile = which == 0 ? bx : num_tiles - 1 - bx;
+    if (which == 1 && (splits > 1 || tile <= bx)) break;
     __syncthreads();                                   // the first tile's last readers of LDS are done
     const int s = tile_entry[tile];
     const int row0 = tile_row0[tile];

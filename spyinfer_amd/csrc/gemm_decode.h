@@ -1,0 +1,31 @@
+// What the decode products' source files share: vector types, the epilogues' codes, the operand order, the arguments
+// of a call.
+#pragma once
+#include "common.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
+#define GD_CHUNK 128
+#define EPI_STORE 0
+#define EPI_GATED 1
+#define EPI_RESID 2
+
+// Where element (row m, column n) of a matrix of MT row tiles lies in operand order, in elements:
+// [N/32 steps][MT row tiles][64 lanes][8], lane 16 g + r of step s holding x[r][32 s + 8 g ..] of its row tile.
+__device__ __forceinline__ size_t operand_order(int m, int n, int MT = 1) {
+    return ((((size_t)(n >> 5) * MT + (m >> 4)) * 64 + ((n & 31) >> 3) * 16 + (m & 15)) * 8) + (n & 7);
+}
+
+struct GdArgs {
+    const bf16_t* x; const bf16_t* w; void* c; float* resid; bf16_t* xw_out; const bf16_t* w_next; float* ss_out; const float* ss_in;
+    int n_parts; float eps; int M, N, K; bool xt, ot; hipStream_t st;
+    void* ws; long long ws_bytes;          // the device's workspace of the products that split K over blocks (or none)
+};
+
+// Compute units of the current device (asked for once per device).
+int gd_compute_units();
+
+// The product with K split over blocks (gemm_decode_splitk.hip): true if it has launched the call.
+bool gd_splitk_try(const GdArgs& a, int epi, bool scaled, bool f32_out);
+long long gd_splitk_workspace_bytes();

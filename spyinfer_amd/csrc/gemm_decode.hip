@@ -22,26 +22,14 @@
 // to each other in memory (with tiles outermost the blocks' addresses differ by multiples of the tile size and crowd
 // on a part of the memory channels: 8-10 % slower).  One 16-row tile (two for EPI_GATED: gate tile t and up tile
 // N/16 + t) per block; its waves split K in interleaved chunks and add through LDS in a fixed order.
-#include "common.h"
+#include "gemm_decode.h"
 #include <math.h>
 
-typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 
-#define GD_CHUNK 128
 #ifndef GD_WAVES_GATED
 #define GD_WAVES_GATED 4
 #endif
-#define EPI_STORE 0
-#define EPI_GATED 1
-#define EPI_RESID 2
-
-// Where element (row m, column n) of a matrix of MT row tiles lies in operand order (see XT / OT above), in elements:
-// [N/32 steps][MT row tiles][64 lanes][8].
-__device__ __forceinline__ size_t operand_order(int m, int n, int MT = 1) {
-    return ((((size_t)(n >> 5) * MT + (m >> 4)) * 64 + ((n & 31) >> 3) * 16 + (m & 15)) * 8) + (n & 7);
-}
 
 template <int EPI, bool SCALED, typename TC, int GD_WAVES, bool XT, bool OT>
 __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
@@ -453,15 +441,9 @@ __global__ __launch_bounds__(512, 1) void gemm_decode_wide_kernel(
     }
 }
 
-struct GdArgs {
-    const bf16_t* x; const bf16_t* w; void* c; float* resid; bf16_t* xw_out; const bf16_t* w_next; float* ss_out; const float* ss_in;
-    int n_parts; float eps; int M, N, K; bool xt, ot; hipStream_t st;
-};
-
 // Blocks of 8 waves, one per 16 columns; the gated product (two tiles per block, usually three blocks per CU)
 // takes blocks of GD_WAVES_GATED waves so that all of them are resident at once.
-// Compute units of the current device (asked for once per device).
-static int compute_units() {
+int gd_compute_units() {
     static int cached[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
@@ -496,7 +478,7 @@ static bool gd_launch_wide(const GdArgs& a) {
         constexpr int GATES = EPI == EPI_GATED ? 2 : 1;
         // a group's accumulators (GATES * CT * MT tiles of four registers) leave room for its operands up to 24 tiles
         constexpr int MAX_CT = 24 / (GATES * MT) < 6 ? 24 / (GATES * MT) : 6;
-        const int cus = compute_units(), tiles = a.N / 16;
+        const int cus = gd_compute_units(), tiles = a.N / 16;
         if (!GD_WIDE || tiles < 2 * cus) return false;       // fewer than two tiles per CU: one tile per block, two blocks per CU
         const int ct = wide_ct((tiles + cus - 1) / cus, MT, GATES, MAX_CT);
 #define GD_WIDE_CASE(C)                                                                                               \
@@ -543,6 +525,10 @@ static void gd_launch(const GdArgs& a) {
     else { if (CAN_OT && a.ot) gd_launch2<EPI, SCALED, TC, false, CAN_OT>(a); else gd_launch2<EPI, SCALED, TC, false, false>(a); }
 }
 
+// Bytes of the device's workspace for the products that split K over blocks: zeroed once by the caller, then handed to
+// every call on that device (ws; none: those products are not taken).  Calls on one device that overlap race on it.
+extern "C" int64_t spy_gemm_decode_workspace() { return gd_splitk_workspace_bytes(); }
+
 // x: bfloat16 [M, K], M <= 64; MP = M rounded up to a multiple of 16.  scaled != 0: x = bf16(h * w_norm) and ss_in
 // [n_parts, MP] holds the parts of sum(h^2); the result is multiplied by rsqrt(sum / K + eps).
 // epi 0: C [M, N] (c_dtype);  epi 1: W = [gate | up], C [M, N] = silu(gate) * up;  epi 2: resid [M, N] += result,
@@ -550,7 +536,7 @@ static void gd_launch(const GdArgs& a) {
 // x_tiled / out_tiled: X / the bfloat16 output for the next product (xw_out of epi 2, C of epi 1) are in operand order.
 extern "C" int spy_gemm_decode(const void* X, int scaled, const float* ss_in, int n_parts, float eps, const void* Wt, int epi,
                                void* C, int c_dtype, float* resid, void* xw_out, const void* w_next, float* ss_out, int M, int N,
-                               int K, int x_tiled, int out_tiled, hipStream_t st) {
+                               int K, int x_tiled, int out_tiled, void* ws, int64_t ws_bytes, hipStream_t st) {
     SPY_REQUIRE(M > 0 && M <= 64, "spy_gemm_decode: M = %d rows (1..64 allowed)", M);
     SPY_REQUIRE(N > 0 && N % 16 == 0 && K > 0 && K % 128 == 0, "spy_gemm_decode: N = %d must be a multiple of 16 and K = %d of 128", N, K);
     SPY_REQUIRE(epi >= 0 && epi <= 2, "spy_gemm_decode: unknown epilogue %d", epi);
@@ -564,8 +550,12 @@ extern "C" int spy_gemm_decode(const void* X, int scaled, const float* ss_in, in
     SPY_REQUIRE(!out_tiled || (N % 32 == 0 && (epi == EPI_RESID || (epi == EPI_GATED && c_dtype == SPY_BF16))),
                 "spy_gemm_decode: operand order is for the bfloat16 output of the gated and the residual epilogue, N a multiple of 32");
     GdArgs a = {(const bf16_t*)X, (const bf16_t*)Wt, C, resid, (bf16_t*)xw_out, (const bf16_t*)w_next, ss_out, ss_in, n_parts, eps, M, N, K,
-                x_tiled != 0, out_tiled != 0, st};
+                x_tiled != 0, out_tiled != 0, st, ws, (long long)ws_bytes};
     const bool f32 = c_dtype == SPY_F32;
+    if (gd_splitk_try(a, epi, scaled != 0, f32)) {
+        SPY_CHECK_LAUNCH("spy_gemm_decode");
+        return 0;
+    }
     if (epi == EPI_RESID) { if (scaled) gd_launch<EPI_RESID, true, bf16_t>(a); else gd_launch<EPI_RESID, false, bf16_t>(a); }
     else if (epi == EPI_GATED) {
         if (scaled) { if (f32) gd_launch<EPI_GATED, true, float>(a); else gd_launch<EPI_GATED, true, bf16_t>(a); }

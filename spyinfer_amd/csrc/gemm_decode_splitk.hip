@@ -1,0 +1,283 @@
+// Decode products of 17 to 64 rows for matrices with about one column tile of 16 per compute unit (o, down, qkv).
+//
+// With a column tile per block every block pulls all of X through L2, MT row tiles against one tile of W: MT times the
+// bytes of W, and the L2's throughput bounds the product, not the matrix' way from memory.  Sharing the X fragments
+// between several column tiles of a block (as for the gated product) leaves too few blocks here.  So K is split over
+// blocks as well: block (column group cg, part ks) has CT neighbouring column tiles and the chunks [nfull ks / KS,
+// nfull (ks + 1) / KS) of K; it reads 1 / KS of X against CT tiles of W, and X's traffic falls from MT to MT / CT
+// times W's.  The block's 8 waves split its chunks and add through LDS in the order of the waves (tile ct is owned by
+// wave ct); the owners write the block's sums to the workspace.  The block that finishes a column group last (a
+// counter per group) adds the group's KS parts in the order of ks and runs the epilogue, so the result does not depend
+// on which block that is.  It leaves the counter at zero for the next call.
+//
+// The dies' L2s are not coherent with each other inside a kernel, and the fences that make them so (write back and
+// invalidate the whole L2) cost about 30 us per call here.  So the parts are written through the caches (stores of
+// system scope), waited for before the block's barrier and its count, and read past the caches (loads of system
+// scope); the counter is an atomic of device scope.  Everything else is read and written as usual.
+//
+// The workspace (counters, then the parts) belongs to the device and is shared by all calls: it starts zeroed, and
+// calls that overlap on two streams of one device race.
+#include "gemm_decode.h"
+#include <math.h>
+
+#define SK_COUNTER_BYTES 16384            // 4096 column groups at most
+#define SK_MAX_TILES_PER_BLOCK 16         // CT * MT at most
+
+template <int EPI, bool SCALED, typename TC, int MT, int CT, bool XT, bool OT, int STEPS = 2>
+__global__ __launch_bounds__(512, 1) void gemm_decode_splitk_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, float* __restrict__ resid_out,
+    bf16_t* __restrict__ xw_out, const bf16_t* __restrict__ w_next, float* __restrict__ ss_out, const float* __restrict__ ss_in,
+    int n_parts, float eps, int M, int N, int K, int KS, unsigned* counters, float* parts) {
+    static_assert(EPI == EPI_STORE || EPI == EPI_RESID, "store and residual epilogues");
+    static_assert(CT <= 8 && CT * MT <= SK_MAX_TILES_PER_BLOCK, "a wave owns at most one column tile; the sums must fit the registers");
+    constexpr int GW = 8;
+    constexpr int MP = 16 * MT;
+    __shared__ float red[(GW - 1) * MT * 64 * 4];
+    __shared__ float ss_red[SCALED ? GW * 4 * MP : 1];
+    __shared__ float row_scale[SCALED ? MP : 1];
+    __shared__ unsigned is_last;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    // neighbouring blocks, which go to different dies, have different parts of K: a die's L2 then holds 1 / KS of X
+    const int cg = blockIdx.x / KS, ks = blockIdx.x % KS;
+
+    if (SCALED) {
+        float part[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) part[mt] = 0.f;
+        for (int p = wave * 4 + g; p < n_parts; p += GW * 4)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) part[mt] += ss_in[p * MP + 16 * mt + r];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) ss_red[(wave * 4 + g) * MP + 16 * mt + r] = part[mt];
+        __syncthreads();
+        if (threadIdx.x < MP) {
+            float s = 0.f;
+            for (int i = 0; i < GW * 4; ++i) s += ss_red[i * MP + threadIdx.x];
+            row_scale[threadIdx.x] = 1.0f / sqrtf(s / (float)K + eps);
+        }
+        // (read after the barriers below)
+    }
+
+    const int tiles = N / 16;
+    const int t0 = cg * CT;
+    const int here = min(CT, tiles - t0);              // the last group may have fewer tiles
+    const size_t chunk_stride = (size_t)tiles * 4096;
+    unsigned xoff[MT];
+    bool x_ok[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        x_ok[mt] = 16 * mt + r < M;
+        xoff[mt] = XT ? (unsigned)mt * 1024u + 16u * lane : (unsigned)min(16 * mt + r, M - 1) * (unsigned)K * 2u + 16u * g;
+    }
+    const char* xbase = reinterpret_cast<const char*>(X);
+    const int nfull = K / GD_CHUNK;
+    const int c_begin = (int)((long long)nfull * ks / KS), c_end = (int)((long long)nfull * (ks + 1) / KS);
+
+    // What the epilogue of this wave's tile needs beside the sums is asked for now, by every block: the last one's
+    // chain of round trips (parts out, count, parts in) is long enough without the stream's and the norm weight's.
+    const bool owner = wave < here;
+    const int tile = t0 + wave, n = tile * 16 + 4 * g;
+    f32x4_t h_old[MT];
+    uint2 wn = {0u, 0u};
+    if (EPI == EPI_RESID && owner) {
+        wn = *reinterpret_cast<const uint2*>(w_next + n);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            h_old[mt] = 16 * mt + r < M ? *reinterpret_cast<const f32x4_t*>(resid_out + (size_t)(16 * mt + r) * N + n) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+
+    f32x4_t acc[CT][MT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[ct][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)t0 * 4096 + 16u * lane;
+    for (int c = c_begin + wave; c < c_end; c += GW) {
+        const char* wb = wbase + (size_t)c * chunk_stride;
+        const char* xb = xbase + (size_t)c * (XT ? 4 * MT * 1024 : GD_CHUNK * 2);
+#pragma unroll
+        for (int h = 0; h < 4; h += STEPS) {
+            bf16x8_t a[CT][STEPS], b[MT][STEPS];
+#pragma unroll
+            for (int j = 0; j < STEPS; ++j) {
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    // a tile that the group does not have reads the group's first tile again (its sums are dropped)
+                    const int t = ct < here ? ct : 0;
+                    a[ct][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wb + (size_t)t * 4096 + 1024 * (h + j)));
+                }
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    b[mt][j] = x_ok[mt] ? *reinterpret_cast<const bf16x8_t*>(xb + xoff[mt] + (XT ? MT * 1024 : 64) * (h + j))
+                                        : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int j = 0; j < STEPS; ++j)
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[ct][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ct][j], b[mt][j], acc[ct][mt], 0, 0, 0);
+        }
+    }
+    // ---- add the waves' sums tile by tile; tile ct belongs to wave ct -------------------------------------------------
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        if (wave != ct) {
+            const int slot = wave < ct ? wave : wave - 1;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) red[((slot * MT + mt) * 4 + i) * 64 + lane] = acc[ct][mt][i];
+        }
+        __syncthreads();
+        if (wave == ct) {
+#pragma unroll
+            for (int w = 0; w < GW - 1; ++w)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[ct][mt][i] += red[((w * MT + mt) * 4 + i) * 64 + lane];
+        }
+        __syncthreads();
+    }
+    // ---- the block's sums to the workspace; who finishes the group last goes on ---------------------------------------
+    // parts: [block][column tile][row tile][4][64 lanes]
+    if (owner) {
+        float* const mine = parts + ((size_t)blockIdx.x * CT + wave) * MT * 256 + lane;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+            if (wave == ct) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        __hip_atomic_store(mine + (mt * 4 + i) * 64, acc[ct][mt][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+        __builtin_amdgcn_s_waitcnt(0);                     // the stores have arrived before the block counts itself done
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned before = __hip_atomic_fetch_add(&counters[cg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = before == (unsigned)KS - 1u;
+        // every block of the group has counted: zero for the next call
+        if (before == (unsigned)KS - 1u) __hip_atomic_store(&counters[cg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!is_last || !owner) return;
+    f32x4_t sum[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) sum[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    {
+        const float* p = parts + ((size_t)cg * KS * CT + wave) * MT * 256 + lane;
+        for (int k = 0; k < KS; ++k, p += (size_t)CT * MT * 256) {
+            float v[MT][4];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[mt][i] = __hip_atomic_load(p + (mt * 4 + i) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sum[mt][i] += v[mt][i];
+        }
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = 16 * mt + r;
+        if (SCALED) {
+            const float scale = row_scale[m];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sum[mt][i] *= scale;
+        }
+        if (EPI == EPI_RESID) {
+            float s = 0.f;
+            if (m < M) {
+                f32x4_t h = h_old[mt];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { h[i] += sum[mt][i]; s += h[i] * h[i]; }
+                *reinterpret_cast<f32x4_t*>(resid_out + (size_t)m * N + n) = h;
+                uint2 o;
+                o.x = pack_bf16x2(h[0] * __uint_as_float(wn.x << 16), h[1] * __uint_as_float(wn.x & 0xffff0000u));
+                o.y = pack_bf16x2(h[2] * __uint_as_float(wn.y << 16), h[3] * __uint_as_float(wn.y & 0xffff0000u));
+                *reinterpret_cast<uint2*>(xw_out + (OT ? operand_order(m, n, MT) : (size_t)m * N + n)) = o;
+            }
+            s += __shfl_xor(s, 16, 64);
+            s += __shfl_xor(s, 32, 64);
+            if (g == 0) ss_out[tile * MP + m] = s;      // rows beyond M: 0
+            continue;
+        }
+        if (m >= M) continue;
+        TC* out = C + (size_t)m * N + n;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) out[i] = from_f32<TC>(sum[mt][i]);
+    }
+}
+
+long long gd_splitk_workspace_bytes() {
+    return SK_COUNTER_BYTES + (long long)gd_compute_units() * SK_MAX_TILES_PER_BLOCK * 1024;
+}
+
+#ifndef GD_SPLITK
+#define GD_SPLITK 1       // 0: never taken (for measurements)
+#endif
+
+// Column tiles per block and parts of K: the pair that gives the most compute units a block, each of a part's 8 waves
+// at least two chunks of K (with one, the way of the parts through memory costs more than X's traffic: the o product
+// of 4096 x 4096 at 64 rows took 17.3 us against 15.1 with a column tile per block; down, 4096 x 12288, 27.6 against
+// 35.1, and qkv, 6144 x 4096 in two parts, 18.6 against 19.3); among equals the most column tiles.
+static void sk_shape(int tiles, int nfull, int cus, int* ct_out, int* ks_out) {
+    int best_ct = 0, best_ks = 0, best_blocks = 0;
+    for (int ct = 4; ct >= 3; --ct) {
+        const int groups = (tiles + ct - 1) / ct;
+        int ks = cus / groups;
+        if (ks > nfull / 16) ks = nfull / 16;
+        if (ks > 16) ks = 16;
+        if (ks < 2) continue;
+        if (groups * ks > best_blocks) { best_blocks = groups * ks; best_ct = ct; best_ks = ks; }
+    }
+    *ct_out = best_ct;
+    *ks_out = best_ks;
+}
+
+template <int EPI, bool SCALED, typename TC, int MT, bool XT, bool OT>
+static bool sk_launch(const GdArgs& a) {
+    const int cus = gd_compute_units(), tiles = a.N / 16, nfull = a.K / GD_CHUNK;
+    int ct = 0, ks = 0;
+    sk_shape(tiles, nfull, cus, &ct, &ks);
+    if (ct == 0) return false;
+    const int groups = (tiles + ct - 1) / ct;
+    if (groups * 4 > SK_COUNTER_BYTES || (long long)groups * ks > cus) return false;
+    if (a.ws_bytes < gd_splitk_workspace_bytes()) return false;
+    unsigned* counters = reinterpret_cast<unsigned*>(a.ws);
+    float* parts = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws) + SK_COUNTER_BYTES);
+#define SK_CASE(C)                                                                                                      \
+    if (ct == C) {                                                                                                      \
+        gemm_decode_splitk_kernel<EPI, SCALED, TC, MT, C, XT, OT><<<groups * ks, 512, 0, a.st>>>(                        \
+            a.x, a.w, (TC*)a.c, a.resid, a.xw_out, a.w_next, a.ss_out, a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K, ks, counters, parts); \
+        return true;                                                                                                    \
+    }
+    SK_CASE(3) SK_CASE(4)
+#undef SK_CASE
+    return false;
+}
+
+template <int EPI, bool SCALED, typename TC, bool XT, bool OT>
+static bool sk_rows(const GdArgs& a) {
+    if (a.M > 48) return sk_launch<EPI, SCALED, TC, 4, XT, OT>(a);
+    if (a.M > 32) return sk_launch<EPI, SCALED, TC, 3, XT, OT>(a);
+    return sk_launch<EPI, SCALED, TC, 2, XT, OT>(a);
+}
+
+// Built for the combinations that a decode step has: the residual product of a plain input (row-major or in operand
+// order) with its output in operand order, and the stored bfloat16 product of a normed input in operand order.
+bool gd_splitk_try(const GdArgs& a, int epi, bool scaled, bool f32_out) {
+    if (!GD_SPLITK || a.ws == nullptr || a.M <= 16 || a.M > 64 || a.N % 16 != 0 || a.K % GD_CHUNK != 0) return false;
+    if (a.N / 16 >= 2 * gd_compute_units()) return false;           // many columns: the kernels that walk column tiles
+    if (epi == EPI_RESID && !scaled && a.ot) {
+        return a.xt ? sk_rows<EPI_RESID, false, bf16_t, true, true>(a) : sk_rows<EPI_RESID, false, bf16_t, false, true>(a);
+    }
+    if (epi == EPI_STORE && scaled && a.xt && !f32_out && !a.ot) return sk_rows<EPI_STORE, true, bf16_t, true, false>(a);
+    return false;
+}

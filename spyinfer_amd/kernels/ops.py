@@ -67,7 +67,7 @@ class _Hip:
                      "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_prefill",
                      "spy_attention_prefill_workspace", "spy_swiglu",
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
-                     "spy_gemm_decode", "spy_embedding_sumsq", "spy_sample_static"):
+                     "spy_gemm_decode", "spy_gemm_decode_workspace", "spy_embedding_sumsq", "spy_sample_static"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: it is older than its sources; build it again "
                                   "(spyinfer_amd.kernels.build.build())" % (self.lib._name, name))
@@ -311,6 +311,23 @@ def fused_decode_ok(rows: int, act_dtype, *tiled_weights, max_rows: Optional[int
                for t in tiled_weights)
 
 
+_decode_workspaces = {}
+
+
+def decode_workspace(device) -> Optional[torch.Tensor]:
+    """The device's workspace of the decode products that split K over blocks (counters that every call leaves at zero,
+    and the blocks' partial sums): made once per device, outside any stream capture, and shared by all calls on the
+    device, which therefore must not overlap (the engine runs them on one stream).  None while a capture is under way
+    and the device has none yet: those products are then not taken."""
+    device = torch.device(device)
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    ws = _decode_workspaces.get(index)
+    if ws is None and not torch.cuda.is_current_stream_capturing():
+        ws = torch.zeros((hip().lib.spy_gemm_decode_workspace(),), dtype=torch.uint8, device=torch.device("cuda", index))
+        _decode_workspaces[index] = ws
+    return ws
+
+
 def _gemm_decode(x, tiled: torch.Tensor, epi: int, n_out: int, out, resid, xw_out, w_next, ss_out) -> None:
     _check(tiled.dtype == torch.bfloat16 and tiled.dim() == 2, "decode product: the tiled matrix must be bfloat16 [N, K]")
     K = tiled.shape[1]
@@ -340,10 +357,12 @@ def _gemm_decode(x, tiled: torch.Tensor, epi: int, n_out: int, out, resid, xw_ou
     xw_t = xw_out.data if isinstance(xw_out, OperandRows) else xw_out
     _dev(xs, ss, tiled, out_t, resid, xw_t, w_next, ss_out)
     _check(0 < M <= FUSED_DECODE_MAX_ROWS, "decode product: %d rows (1..%d allowed)" % (M, FUSED_DECODE_MAX_ROWS))
+    ws = decode_workspace(xs.device) if M > 16 else None
     hip().call("spy_gemm_decode", _ptr(xs), ctypes.c_int(0 if ss is None else 1), _ptr(ss), ctypes.c_int(0 if ss is None else ss.shape[0]),
                ctypes.c_float(eps), _ptr(tiled), ctypes.c_int(epi), _ptr(out_t), ctypes.c_int(0 if out_t is None else _code(out_t, "out")),
                _ptr(resid), _ptr(xw_t), _ptr(w_next), _ptr(ss_out), ctypes.c_int(M), ctypes.c_int(n_out), ctypes.c_int(K),
-               ctypes.c_int(1 if x_tiled else 0), ctypes.c_int(1 if out_tiled else 0), _Hip.stream())
+               ctypes.c_int(1 if x_tiled else 0), ctypes.c_int(1 if out_tiled else 0), _ptr(ws),
+               ctypes.c_int64(0 if ws is None else ws.numel()), _Hip.stream())
 
 
 def _rows_of(x) -> int:

@@ -119,7 +119,10 @@ def test_linear_with_tiled_weights(M, N, K):
                                             # many column tiles (two and more per compute unit): blocks that walk a run of
                                             # tiles, several at a time, the last group of a run with fewer
                                             (64, 128, 8320, 8208, 1e-6), (37, 256, 8448, 9008, 1e-5), (20, 128, 8192, 16400, 1e-6),
-                                            (48, 128, 128, 151936, 1e-6), (16, 128, 8320, 8208, 1e-6)])
+                                            (48, 128, 128, 151936, 1e-6), (16, 128, 8320, 8208, 1e-6),
+                                            # about a column tile per compute unit and a long K: K split over blocks, the
+                                            # group's last block adding the parts (a last group with fewer tiles; 2, 3, 4 parts)
+                                            (64, 4096, 4096, 6144, 1e-6), (40, 4224, 2176, 6176, 1e-5), (20, 5120, 3200, 6160, 1e-6)])
 def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
     """The chain of a decode step's products with the norms folded in: the residual epilogue adds to the stream,
     prepares bf16(h * w) and the parts of sum(h^2); the next products scale their sums by rsqrt(mean(h^2) + eps).
@@ -162,27 +165,40 @@ def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
     h2 = resid.double() + norm64(resid, wn1) @ w_sq.double().t()
     close(resid2, h2, torch.bfloat16, scale=2.0, what="stream after a scaled product")
     assert torch.equal(si2.xw.to_rows(), (resid2 * wn2.float()).bfloat16())
-    # the same chain with row-major hand-over gives the same numbers
-    ops.OPERAND_ORDER = False
+    # the same chain with row-major hand-over gives the same numbers (both through the kernels with a column tile per
+    # block: the products that split K over blocks add in another order, and are built for operand order only)
+    real_ws = ops.decode_workspace
+    ops.decode_workspace = lambda device: None
     try:
-        resid_r = resid0.clone()
-        si_r = ops.decode_linear_residual(a, ops.tile_weight(w_in), resid_r, wn1, eps)
-        assert not isinstance(si_r.xw, ops.OperandRows) and torch.equal(si_r.xw, si.xw.to_rows()) and torch.equal(resid_r, resid)
-        assert torch.equal(ops.decode_linear(si_r, ops.tile_weight(w_qkv)), ops.decode_linear(si, ops.tile_weight(w_qkv)))
-        g_rows = ops.decode_linear_swiglu(si_r, ops.tile_weight(w_gu), for_product=True)
+        resid_t = resid0.clone()
+        si_t = ops.decode_linear_residual(a, ops.tile_weight(w_in), resid_t, wn1, eps)
+        close(resid_t, h, torch.float32, scale=4.0, what="stream after the residual epilogue, K not split")
+        qkv_t = ops.decode_linear(si_t, ops.tile_weight(w_qkv))
+        g_tiled = ops.decode_linear_swiglu(si_t, ops.tile_weight(w_gu), for_product=True)
+        w_dn = rnd((H, I), torch.bfloat16, dev, 40, 0.05)
+        ra, rb = resid_t.clone(), resid_t.clone()
+        sa = ops.decode_linear_residual(g_tiled, ops.tile_weight(w_dn), ra, wn2, eps)
+        ops.OPERAND_ORDER = False
+        try:
+            resid_r = resid0.clone()
+            si_r = ops.decode_linear_residual(a, ops.tile_weight(w_in), resid_r, wn1, eps)
+            assert not isinstance(si_r.xw, ops.OperandRows) and torch.equal(si_r.xw, si_t.xw.to_rows()) and torch.equal(resid_r, resid_t)
+            assert torch.equal(ops.decode_linear(si_r, ops.tile_weight(w_qkv)), qkv_t)
+            g_rows = ops.decode_linear_swiglu(si_r, ops.tile_weight(w_gu), for_product=True)
+            sb = ops.decode_linear_residual(g_rows, ops.tile_weight(w_dn), rb, wn2, eps)
+        finally:
+            ops.OPERAND_ORDER = True
     finally:
-        ops.OPERAND_ORDER = True
-    g_tiled = ops.decode_linear_swiglu(si, ops.tile_weight(w_gu), for_product=True)
+        ops.decode_workspace = real_ws
     assert isinstance(g_tiled, ops.OperandRows) and torch.equal(g_tiled.to_rows(), g_rows)
-    w_dn = rnd((H, I), torch.bfloat16, dev, 40, 0.05)
-    ra, rb = resid.clone(), resid.clone()
-    sa = ops.decode_linear_residual(g_tiled, ops.tile_weight(w_dn), ra, wn2, eps)
-    ops.OPERAND_ORDER = False
-    try:
-        sb = ops.decode_linear_residual(g_rows, ops.tile_weight(w_dn), rb, wn2, eps)
-    finally:
-        ops.OPERAND_ORDER = True
     assert torch.equal(ra, rb) and torch.equal(sa.xw.to_rows(), sb.xw) and torch.equal(sa.ss_parts, sb.ss_parts)
+    # the down product (its input in operand order) against float64, K split where the shape allows
+    rd = resid.clone()
+    g_in = ops.decode_linear_swiglu(si, ops.tile_weight(w_gu), for_product=True)
+    sd = ops.decode_linear_residual(g_in, ops.tile_weight(w_dn), rd, wn2, eps)
+    close(rd, resid.double() + g_in.to_rows().double() @ w_dn.double().t(), torch.float32, scale=4.0, what="stream after the down product")
+    assert torch.equal(sd.xw.to_rows(), (rd * wn2.float()).bfloat16())
+    assert torch.allclose(sd.ss_parts.sum(0)[:M], (rd * rd).sum(1), rtol=1e-5)
     # 4. the scale matters: another eps or a missing part changes the result by far more than the tolerance
     far = ops.decode_linear(ops.ScaledInput(si.xw, si.ss_parts * 4.0, eps), ops.tile_weight(w_qkv), torch.float32)
     ref = (norm64(resid, wn1) @ w_qkv.double().t()).float()
