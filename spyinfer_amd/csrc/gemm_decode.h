@@ -17,6 +17,30 @@ __device__ __forceinline__ size_t operand_order(int m, int n, int MT = 1) {
     return ((((size_t)(n >> 5) * MT + (m >> 4)) * 64 + ((n & 31) >> 3) * 16 + (m & 15)) * 8) + (n & 7);
 }
 
+// This thread's share of the parts of the rows' sums of squares, for MT row tiles: parts slot, slot + GROUPS, ... of row
+// 16 mt + r.  The first 256 parts are asked for at once (one memory round trip; a loop that adds as it loads has one
+// per turn) and added in the order of the parts.
+template <int MT, int GROUPS>
+__device__ __forceinline__ void gd_ss_share(const float* __restrict__ ss_in, int n_parts, int slot, int r, float (&out)[MT]) {
+    constexpr int NPV = 256 / GROUPS, MP = 16 * MT;
+    float pv[NPV][MT];
+#pragma unroll
+    for (int i = 0; i < NPV; ++i) {
+        const int p = slot + GROUPS * i;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) pv[i][mt] = p < n_parts ? ss_in[p * MP + 16 * mt + r] : 0.f;
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) out[mt] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NPV; ++i)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) out[mt] += pv[i][mt];
+    for (int p = 256 + slot; p < n_parts; p += GROUPS)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) out[mt] += ss_in[p * MP + 16 * mt + r];
+}
+
 struct GdArgs {
     const bf16_t* x; const bf16_t* w; void* c; float* resid; bf16_t* xw_out; const bf16_t* w_next; float* ss_out; const float* ss_in;
     int n_parts; float eps; int M, N, K; bool xt, ot; hipStream_t st;

@@ -180,20 +180,22 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
     int n_parts, float eps, int M, int N, int K) {
     constexpr int NT = (EPI == EPI_GATED ? 2 : 1) * CT;      // W tiles per block: [gate tiles | up tiles] for the gated product
     constexpr int MP = 16 * MT;
-    __shared__ float red[(GD_WAVES - 1) * NT * MT * 64 * 4];
+    __shared__ f32x4_t red[(GD_WAVES - 1) * NT * MT * 64];
     __shared__ float ss_red[GD_WAVES * 4 * MP];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int r = lane & 15, g = lane >> 4;
 
-    if (SCALED) {
-        float part[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) part[mt] = 0.f;
-        for (int p = wave * 4 + g; p < n_parts; p += GD_WAVES * 4)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) part[mt] += ss_in[p * MP + 16 * mt + r];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) ss_red[(wave * 4 + g) * MP + 16 * mt + r] = part[mt];
+    // What is needed only after the product is asked for now: this thread's share of the rows' sums of squares (all of
+    // it under way at once), and for the residual epilogue the piece of the stream and of the next norm's weight of
+    // the wave that will run it (row tile mt belongs to wave mt).
+    float ss_part[MT];
+    if (SCALED) gd_ss_share<MT, GD_WAVES * 4>(ss_in, n_parts, wave * 4 + g, r, ss_part);
+    f32x4_t h_old = {0.f, 0.f, 0.f, 0.f};
+    uint2 wn = {0u, 0u};
+    if (EPI == EPI_RESID && wave < MT && 16 * wave + r < M) {
+        static_assert(EPI != EPI_RESID || CT == 1, "the residual epilogue has one column tile per block");
+        h_old = *reinterpret_cast<const f32x4_t*>(resid_out + (size_t)(16 * wave + r) * N + blockIdx.x * 16 + 4 * g);
+        wn = *reinterpret_cast<const uint2*>(w_next + blockIdx.x * 16 + 4 * g);
     }
 
     f32x4_t acc[NT][MT];
@@ -231,33 +233,37 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
         _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                            \
             _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                        \
                 acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[nt][j], B[mt][j], acc[nt][mt], 0, 0, 0);
-    for (int c = wave; c < nfull; c += GD_WAVES) {     // (two chunks per round were measured at two row tiles: no gain)
+    // (two chunks per round, and the next chunk's operands asked for before this chunk's products, were measured at two
+    // to four row tiles: no gain either)
+    for (int c = wave; c < nfull; c += GD_WAVES) {
         bf16x8_t a[NT][4], b[MT][4];
         GDR_LOAD(a, b, c)
         GDR_MFMA(a, b)
     }
 #undef GDR_LOAD
 #undef GDR_MFMA
-    if (wave > 0) {
+    // ---- add the waves' sums in a fixed order: row tile mt is summed, and its epilogue run, by wave mt ------------------
+    static_assert(MT <= GD_WAVES, "a wave per row tile");
+    if (SCALED) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) red[((((wave - 1) * NT + nt) * MT + mt) * 4 + i) * 64 + lane] = acc[nt][mt][i];
+        for (int mt = 0; mt < MT; ++mt) ss_red[(wave * 4 + g) * MP + 16 * mt + r] = ss_part[mt];
     }
-    __syncthreads();
-    if (wave > 0) return;
-#pragma unroll
-    for (int w = 1; w < GD_WAVES; ++w)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[nt][mt][i] += red[((((w - 1) * NT + nt) * MT + mt) * 4 + i) * 64 + lane];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
+        if (wave == mt) continue;
+        const int slot = wave < mt ? wave : wave - 1;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) red[((slot * NT + nt) * MT + mt) * 64 + lane] = acc[nt][mt];
+    }
+    __syncthreads();
+    if (wave >= MT) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        if (wave != mt) continue;
+#pragma unroll
+        for (int w = 0; w < GD_WAVES - 1; ++w)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[nt][mt] += red[((w * NT + nt) * MT + mt) * 64 + lane];
         const int m = 16 * mt + r;
         float scale = 1.f;
         if (SCALED) {
@@ -275,12 +281,10 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
             if (EPI == EPI_RESID) {
                 float s = 0.f;
                 if (m < M) {
-                    float* hp = resid_out + (size_t)m * N + n;
-                    f32x4_t h = *reinterpret_cast<const f32x4_t*>(hp);
-                    const uint2 wn = *reinterpret_cast<const uint2*>(w_next + n);
+                    f32x4_t h = h_old;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) { h[i] += acc[ct][mt][i]; s += h[i] * h[i]; }
-                    *reinterpret_cast<f32x4_t*>(hp) = h;
+                    *reinterpret_cast<f32x4_t*>(resid_out + (size_t)m * N + n) = h;
                     uint2 o;
                     o.x = pack_bf16x2(h[0] * __uint_as_float(wn.x << 16), h[1] * __uint_as_float(wn.x & 0xffff0000u));
                     o.y = pack_bf16x2(h[2] * __uint_as_float(wn.y << 16), h[3] * __uint_as_float(wn.y & 0xffff0000u));
@@ -309,42 +313,32 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
 // CT at a time, against the same X fragments in registers: X's traffic falls to MT / CT (MT / 2 CT for the gated
 // product, whose gate and up tiles share them as well).  The 8 waves of a block split K as above; operands are loaded
 // half a chunk at a time (the accumulators of CT tiles take the registers of the other half); the waves' sums of one
-// column tile are added through LDS by the wave that owns the tile (tile ct -> wave ct), in the order of the waves, and
-// that wave runs the tile's epilogue.  Store and gated epilogues only.
-template <int EPI, bool SCALED, typename TC, int MT, int CT, bool XT, bool OT, int STEPS = 2>
+// column tiles are added through LDS in two rounds, in a fixed order, and the four waves that end up with them run the
+// epilogue, each for every fourth (column tile, row tile) unit.  Store and gated epilogues only.
+template <int EPI, bool SCALED, typename TC, int MT, int CT, bool XT, bool OT>
 __global__ __launch_bounds__(512, 1) void gemm_decode_wide_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, const float* __restrict__ ss_in,
     int n_parts, float eps, int M, int N, int K) {
     static_assert(EPI == EPI_STORE || EPI == EPI_GATED, "the wide kernel has no residual epilogue");
-    static_assert(CT <= 8, "a wave owns at most one column tile of a group");
     static_assert((EPI == EPI_GATED ? 2 : 1) * CT * MT <= 24, "the accumulators of a group must fit the registers");
     constexpr int GW = 8;
     constexpr int GATES = EPI == EPI_GATED ? 2 : 1;
     constexpr int NT = GATES * CT;
     constexpr int MP = 16 * MT;
-    __shared__ float red[(GW - 1) * MT * 64 * 4];
+    constexpr int PAIRS = CT * MT;                       // (column tile, row tile) units of the epilogue
+    // the waves' sums meet in two rounds: waves 4..7 hand all of theirs to waves 0..3, then each of these four takes
+    // every fourth unit from the other three.  The second round's buffer lies inside the first's.
+    __shared__ f32x4_t red[4 * NT * MT * 64];
+    static_assert(PAIRS * 3 * GATES <= 4 * NT * MT, "the second round fits the first round's buffer");
     __shared__ float ss_red[GW * 4 * MP];
     __shared__ float row_scale[MP];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int r = lane & 15, g = lane >> 4;
 
-    if (SCALED) {
-        float part[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) part[mt] = 0.f;
-        for (int p = wave * 4 + g; p < n_parts; p += GW * 4)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) part[mt] += ss_in[p * MP + 16 * mt + r];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) ss_red[(wave * 4 + g) * MP + 16 * mt + r] = part[mt];
-        __syncthreads();
-        if (threadIdx.x < MP) {
-            float s = 0.f;
-            for (int i = 0; i < GW * 4; ++i) s += ss_red[i * MP + threadIdx.x];
-            row_scale[threadIdx.x] = 1.0f / sqrtf(s / (float)K + eps);
-        }
-        __syncthreads();
-    }
+    // This thread's share of the rows' sums of squares, all of it under way at once (one round trip before the matrix'
+    // first loads); the waves' shares meet after the first group's products.
+    float ss_part[MT];
+    if (SCALED) gd_ss_share<MT, GW * 4>(ss_in, n_parts, wave * 4 + g, r, ss_part);
 
     // this block's run of column tiles: the tiles dealt evenly over the blocks
     const int tiles = N / 16;
@@ -359,6 +353,7 @@ __global__ __launch_bounds__(512, 1) void gemm_decode_wide_kernel(
     }
     const char* xbase = reinterpret_cast<const char*>(X);
     const int nfull = K / GD_CHUNK;
+    const int my_steps = wave < nfull ? 4 * ((nfull - wave + GW - 1) / GW) : 0;      // steps of 32 of K: this wave's chunks
 
     for (int t0 = t_begin; t0 < t_end; t0 += CT) {
         const int here = min(CT, t_end - t0);            // tiles of this group (the run's last group may have fewer)
@@ -368,76 +363,101 @@ __global__ __launch_bounds__(512, 1) void gemm_decode_wide_kernel(
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)t0 * 4096 + 16u * lane;
-        for (int c = wave; c < nfull; c += GW) {
-            const char* wb = wbase + (size_t)c * chunk_stride;
-            const char* xb = xbase + (size_t)c * (XT ? 4 * MT * 1024 : GD_CHUNK * 2);
+        // One step at a time, the next step's operands asked for before this step's products: a wave has loads under
+        // way while its matrix unit works (against half a chunk loaded and then multiplied: 1-2 %).
+        {
+            bf16x8_t a0[NT], b0[MT], a1[NT], b1[MT];
+#define GDW_LOAD(A, B, STEP)                                                                                         \
+            {                                                                                                        \
+                const int c_ = wave + GW * ((STEP) >> 2), h_ = (STEP) & 3;                                           \
+                const char* wb = wbase + (size_t)c_ * chunk_stride;                                                  \
+                const char* xb = xbase + (size_t)c_ * (XT ? 4 * MT * 1024 : GD_CHUNK * 2);                           \
+                _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) {                                                  \
+                    /* a tile that the group does not have reads the group's first tile again (its sums are dropped) */ \
+                    const int ct = nt % CT < here ? nt % CT : 0;                                                     \
+                    A[nt] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(                            \
+                        wb + (size_t)((nt / CT) * tiles + ct) * 4096 + 1024 * h_));                                  \
+                }                                                                                                    \
+                _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                    \
+                    B[mt] = x_ok[mt] ? *reinterpret_cast<const bf16x8_t*>(xb + xoff[mt] + (XT ? MT * 1024 : 64) * h_) \
+                                     : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};                                             \
+            }
+#define GDW_MFMA(A, B)                                                                                               \
+            _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                        \
+                _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                    \
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[nt], B[mt], acc[nt][mt], 0, 0, 0);
+            if (my_steps > 0) GDW_LOAD(a0, b0, 0)
+            for (int st = 0; st < my_steps; st += 2) {     // (a multiple of 4)
+                GDW_LOAD(a1, b1, st + 1)
+                GDW_MFMA(a0, b0)
+                if (st + 2 < my_steps) GDW_LOAD(a0, b0, st + 2)
+                GDW_MFMA(a1, b1)
+            }
+#undef GDW_LOAD
+#undef GDW_MFMA
+        }
+        // ---- round one: the upper four waves' sums to the lower four -------------------------------------------------
+        if (SCALED && t0 == t_begin) {
 #pragma unroll
-            for (int h = 0; h < 4; h += STEPS) {
-                bf16x8_t a[NT][STEPS], b[MT][STEPS];
+            for (int mt = 0; mt < MT; ++mt) ss_red[(wave * 4 + g) * MP + 16 * mt + r] = ss_part[mt];
+        }
+        if (wave >= 4) {
 #pragma unroll
-                for (int j = 0; j < STEPS; ++j) {
+            for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        // a tile that the group does not have reads the group's first tile again (its sums are dropped)
-                        const int ct = nt % CT < here ? nt % CT : 0;
-                        a[nt][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(
-                            wb + (size_t)((nt / CT) * tiles + ct) * 4096 + 1024 * (h + j)));
-                    }
+                for (int mt = 0; mt < MT; ++mt) red[(((wave - 4) * NT + nt) * MT + mt) * 64 + lane] = acc[nt][mt];
+        }
+        __syncthreads();
+        if (SCALED && t0 == t_begin && threadIdx.x >= 256 && threadIdx.x < 256 + MP) {      // (a wave that has nothing to add now)
+            const int m = threadIdx.x - 256;
+            float s = 0.f;
+            for (int i = 0; i < GW * 4; ++i) s += ss_red[i * MP + m];
+            row_scale[m] = 1.0f / sqrtf(s / (float)K + eps);
+        }
+        if (wave < 4) {
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        b[mt][j] = x_ok[mt] ? *reinterpret_cast<const bf16x8_t*>(xb + xoff[mt] + (XT ? MT * 1024 : 64) * (h + j))
-                                            : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[nt][mt] += red[((wave * NT + nt) * MT + mt) * 64 + lane];
+        }
+        __syncthreads();
+        // ---- round two: unit p = ct MT + mt (its gate and its up tile) belongs to wave p % 4 --------------------------
+        if (wave < 4) {
+#pragma unroll
+            for (int p = 0; p < PAIRS; ++p) {
+                const int owner = p & 3;
+                if (wave != owner) {
+                    const int slot = wave < owner ? wave : wave - 1;
+#pragma unroll
+                    for (int gt = 0; gt < GATES; ++gt) red[((p * 3 + slot) * GATES + gt) * 64 + lane] = acc[gt * CT + p / MT][p % MT];
                 }
-#pragma unroll
-                for (int j = 0; j < STEPS; ++j)
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt)
-                            acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], b[mt][j], acc[nt][mt], 0, 0, 0);
             }
         }
-        // ---- add the waves' sums tile by tile; tile ct (and its up tile) belongs to wave ct ---------------------------
+        __syncthreads();
+        if (wave < 4) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            const int owner = nt % CT;
-            if (wave != owner) {
-                const int slot = wave < owner ? wave : wave - 1;
+            for (int p = 0; p < PAIRS; ++p) {
+                if (wave != (p & 3)) continue;
+                const int ct = p / MT, mt = p % MT;
+                f32x4_t v = acc[ct][mt], up = acc[(GATES - 1) * CT + ct][mt];
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) red[((slot * MT + mt) * 4 + i) * 64 + lane] = acc[nt][mt][i];
-            }
-            __syncthreads();
-            if (wave == owner) {
-#pragma unroll
-                for (int w = 0; w < GW - 1; ++w)
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) acc[nt][mt][i] += red[((w * MT + mt) * 4 + i) * 64 + lane];
-            }
-            __syncthreads();
-        }
-        // ---- epilogue of the tile this wave owns ------------------------------------------------------------------------
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            if (wave != ct || ct >= here) continue;
-            const int n = (t0 + ct) * 16 + 4 * g;
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const int m = 16 * mt + r;
-                if (m >= M) continue;
+                for (int slot = 0; slot < 3; ++slot) {
+                    v += red[((p * 3 + slot) * GATES + 0) * 64 + lane];
+                    if (EPI == EPI_GATED) up += red[((p * 3 + slot) * GATES + GATES - 1) * 64 + lane];
+                }
+                const int n = (t0 + ct) * 16 + 4 * g, m = 16 * mt + r;
+                if (ct >= here || m >= M) continue;
                 const float scale = SCALED ? row_scale[m] : 1.f;
                 TC* out = C + (OT ? operand_order(m, n, MT) : (size_t)m * N + n);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float v = acc[ct][mt][i] * scale;
-                    if (EPI == EPI_GATED) { const float up = acc[CT + ct][mt][i] * scale; v = (v / (1.0f + expf(-v))) * up; }
-                    out[i] = from_f32<TC>(v);
+                    float y = v[i] * scale;
+                    if (EPI == EPI_GATED) { const float u = up[i] * scale; y = (y / (1.0f + expf(-y))) * u; }
+                    out[i] = from_f32<TC>(y);
                 }
             }
         }
+        __syncthreads();                                  // the buffer is free for the next group
     }
 }
 

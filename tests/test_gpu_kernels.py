@@ -121,8 +121,8 @@ def test_linear_with_tiled_weights(M, N, K):
                                             (64, 128, 8320, 8208, 1e-6), (37, 256, 8448, 9008, 1e-5), (20, 128, 8192, 16400, 1e-6),
                                             (48, 128, 128, 151936, 1e-6), (16, 128, 8320, 8208, 1e-6),
                                             # about a column tile per compute unit and a long K: K split over blocks, the
-                                            # group's last block adding the parts (a last group with fewer tiles; 2, 3, 4 parts)
-                                            (64, 4096, 4096, 6144, 1e-6), (40, 4224, 2176, 6176, 1e-5), (20, 5120, 3200, 6160, 1e-6)])
+                                            # group's last block adding the parts (33 to 64 rows; a last group with fewer tiles; 2, 3, 4 parts)
+                                            (64, 4096, 12288, 6144, 1e-6), (40, 4096, 8192, 6128, 1e-5), (52, 5120, 6400, 6160, 1e-6)])
 def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
     """The chain of a decode step's products with the norms folded in: the residual epilogue adds to the stream,
     prepares bf16(h * w) and the parts of sum(h^2); the next products scale their sums by rsqrt(mean(h^2) + eps).
@@ -165,33 +165,37 @@ def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
     h2 = resid.double() + norm64(resid, wn1) @ w_sq.double().t()
     close(resid2, h2, torch.bfloat16, scale=2.0, what="stream after a scaled product")
     assert torch.equal(si2.xw.to_rows(), (resid2 * wn2.float()).bfloat16())
-    # the same chain with row-major hand-over gives the same numbers (both through the kernels with a column tile per
-    # block: the products that split K over blocks add in another order, and are built for operand order only)
-    real_ws = ops.decode_workspace
-    ops.decode_workspace = lambda device: None
+    # the same chain with row-major hand-over: the same numbers where both forms run through the same kernel (up to 16
+    # rows); above that the kernels that walk or split differ by form and add in another order, and each form is held
+    # against float64 by itself
+    same_kernel = M <= 16
+    ops.OPERAND_ORDER = False
     try:
-        resid_t = resid0.clone()
-        si_t = ops.decode_linear_residual(a, ops.tile_weight(w_in), resid_t, wn1, eps)
-        close(resid_t, h, torch.float32, scale=4.0, what="stream after the residual epilogue, K not split")
-        qkv_t = ops.decode_linear(si_t, ops.tile_weight(w_qkv))
-        g_tiled = ops.decode_linear_swiglu(si_t, ops.tile_weight(w_gu), for_product=True)
+        resid_r = resid0.clone()
+        si_r = ops.decode_linear_residual(a, ops.tile_weight(w_in), resid_r, wn1, eps)
+        assert not isinstance(si_r.xw, ops.OperandRows)
+        qkv_r = ops.decode_linear(si_r, ops.tile_weight(w_qkv))
+        g_rows = ops.decode_linear_swiglu(si_r, ops.tile_weight(w_gu), for_product=True)
         w_dn = rnd((H, I), torch.bfloat16, dev, 40, 0.05)
-        ra, rb = resid_t.clone(), resid_t.clone()
-        sa = ops.decode_linear_residual(g_tiled, ops.tile_weight(w_dn), ra, wn2, eps)
-        ops.OPERAND_ORDER = False
-        try:
-            resid_r = resid0.clone()
-            si_r = ops.decode_linear_residual(a, ops.tile_weight(w_in), resid_r, wn1, eps)
-            assert not isinstance(si_r.xw, ops.OperandRows) and torch.equal(si_r.xw, si_t.xw.to_rows()) and torch.equal(resid_r, resid_t)
-            assert torch.equal(ops.decode_linear(si_r, ops.tile_weight(w_qkv)), qkv_t)
-            g_rows = ops.decode_linear_swiglu(si_r, ops.tile_weight(w_gu), for_product=True)
-            sb = ops.decode_linear_residual(g_rows, ops.tile_weight(w_dn), rb, wn2, eps)
-        finally:
-            ops.OPERAND_ORDER = True
+        rb = resid_r.clone()
+        sb = ops.decode_linear_residual(g_rows, ops.tile_weight(w_dn), rb, wn2, eps)
     finally:
-        ops.decode_workspace = real_ws
-    assert isinstance(g_tiled, ops.OperandRows) and torch.equal(g_tiled.to_rows(), g_rows)
-    assert torch.equal(ra, rb) and torch.equal(sa.xw.to_rows(), sb.xw) and torch.equal(sa.ss_parts, sb.ss_parts)
+        ops.OPERAND_ORDER = True
+    close(resid_r, h, torch.float32, scale=4.0, what="stream after the residual epilogue, row-major hand-over")
+    assert torch.equal(si_r.xw, (resid_r * wn1.float()).bfloat16())
+    y_r = norm64(resid_r, wn1) @ w_gu.double().t()
+    close(qkv_r, norm64(resid_r, wn1) @ w_qkv.double().t(), torch.bfloat16, scale=2.0, what="scaled decode_linear, row-major hand-over")
+    close(g_rows, y_r[:, :I] / (1 + torch.exp(-y_r[:, :I])) * y_r[:, I:], torch.bfloat16, scale=2.0, what="gated product, row-major hand-over")
+    close(rb, resid_r.double() + g_rows.double() @ w_dn.double().t(), torch.float32, scale=4.0, what="down product, row-major hand-over")
+    assert torch.equal(sb.xw, (rb * wn2.float()).bfloat16()) and torch.allclose(sb.ss_parts.sum(0)[:M], (rb * rb).sum(1), rtol=1e-5)
+    g_tiled = ops.decode_linear_swiglu(si, ops.tile_weight(w_gu), for_product=True)
+    assert isinstance(g_tiled, ops.OperandRows)
+    if same_kernel:
+        ra = resid.clone()
+        sa = ops.decode_linear_residual(g_tiled, ops.tile_weight(w_dn), ra, wn2, eps)
+        assert torch.equal(resid_r, resid) and torch.equal(si_r.xw, si.xw.to_rows())
+        assert torch.equal(qkv_r, ops.decode_linear(si, ops.tile_weight(w_qkv))) and torch.equal(g_tiled.to_rows(), g_rows)
+        assert torch.equal(ra, rb) and torch.equal(sa.xw.to_rows(), sb.xw) and torch.equal(sa.ss_parts, sb.ss_parts)
     # the down product (its input in operand order) against float64, K split where the shape allows
     rd = resid.clone()
     g_in = ops.decode_linear_swiglu(si, ops.tile_weight(w_gu), for_product=True)
@@ -209,6 +213,36 @@ def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
     out, e = ops.embedding_scaled(ids, table, wn1, eps)
     assert torch.equal(out, ops.embedding(ids, table)) and torch.equal(e.xw.to_rows(), (out * wn1.float()).bfloat16())
     assert torch.allclose(e.ss_parts[0, :len(ids)], (out * out).sum(1), rtol=1e-5) and (len(ids) % 16 == 0 or float(e.ss_parts[0, len(ids):].abs().max()) == 0.0)
+
+
+def test_products_with_k_split_over_blocks_repeat_exactly():
+    """The product whose blocks hand their partial sums to the last block of a column group (long K, about a column
+    tile per compute unit): 40 calls in a row without a wait between them, on changing inputs, give bit for bit what
+    the same inputs gave before, and what float64 gives within the tolerance.  A part read before it was written, or
+    a counter not left at zero, would show as a difference."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    M, N, K = 64, 4096, 12288
+    w = rnd((N, K), torch.bfloat16, dev, 51, 0.02)
+    wt = ops.tile_weight(w)
+    wn = (1 + 0.1 * rnd((N,), torch.float32, dev, 52)).bfloat16()
+    xs = []
+    for i in range(4):
+        x = ops.OperandRows.empty(M, K, dev)
+        x.data.copy_(rnd(tuple(x.data.shape), torch.bfloat16, dev, 60 + i))
+        xs.append(x)
+    first = {}
+    for call in range(40):
+        i = call % 4
+        resid = torch.zeros((M, N), dtype=torch.float32, device=dev)
+        si = ops.decode_linear_residual(xs[i], wt, resid, wn, 1e-6)
+        if i in first:
+            assert torch.equal(resid, first[i][0]) and torch.equal(si.xw.data, first[i][1]) and torch.equal(si.ss_parts, first[i][2]), "call %d" % call
+        else:
+            first[i] = (resid, si.xw.data.clone(), si.ss_parts.clone())
+    for i in range(4):
+        close(first[i][0], xs[i].to_rows().double() @ w.double().t(), torch.float32, scale=4.0, what="input %d" % i)
+    assert int(ops.decode_workspace(dev)[:16384].max()) == 0, "the counters are left at zero"
 
 
 def test_decode_products_refuse_wrong_operands():
