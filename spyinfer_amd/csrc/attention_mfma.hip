@@ -15,7 +15,8 @@
 //                   V^T comes from the cache, where values lie [d][key] within a page: lane
 //                   (d row, g) loads the 8 keys c0 + 8g .. +7 of row d with one 16-byte load.
 // Keys lie [key][d] within a page: lane (key, g) loads 16 bytes K[key][32 kk + 8 g ..].
-// With several parts per tile the partial (O, m, l) go to a workspace and a second kernel merges.
+// With several parts per tile the partial (O, m, l) go to a workspace; the tile's last block merges them (given
+// counters), or a second kernel does.
 //
 // FUSED (steps in which every entry is a single token, head_dim 64, 128 or 256, whole head rotated): the kernel reads
 // the raw q, k, v of the step's product itself.  A query row's values lie in one lane and the three lanes beside it the
@@ -119,7 +120,8 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, bf16_t* kc, bf16_t* vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
-    int n_q, int n_kv, int d, float scale, int window, int splits, float* __restrict__ ws, FusedQKV fz, int out_tiles) {
+    int n_q, int n_kv, int d, float scale, int window, int splits, float* __restrict__ ws, FusedQKV fz, int out_tiles,
+    unsigned* counters) {
     constexpr int KK = DMAX / 32;   // 32-wide chunks of the head dim for Q.K
     constexpr int DT = DMAX / 16;   // 16-row tiles of the head dim for P.V
     extern __shared__ float lds[];   // the waves' O, m, l: AW (head sizes up to 128) or AW - 1 times (DT * 4 + 2) * 64 floats
@@ -485,8 +487,79 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         }
         return;
     }
-    // partial result: ws[((tile * n_kv + hk) * splits + sp)] = { O[16][DMAX], m[16], l[16] }
     float* w = ws + (((size_t)tile * n_kv + hk) * splits + sp) * (16 * (DMAX + 2));
+    if (SPREAD && counters) {
+        // The parts of a (tile, kv head) are merged here, by the block that finishes last (a counter per tile and head,
+        // left at zero), instead of by a second kernel.  The dies' L2s are not coherent inside a kernel: the parts go
+        // through the caches (stores of system scope, waited for before the block counts itself) and are read past them.
+        // A part lies lane for lane: O[(dt 4 + i)][64 lanes], then m[16], l[16].
+        __shared__ unsigned am_last;
+#pragma unroll
+        for (int i = 0; i < MINE; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) __hip_atomic_store(w + ((dt0 + i) * 4 + j) * 64 + lane, mo[i][j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        if (g == 0 && wave == 0) {
+            __hip_atomic_store(w + 16 * DMAX + r16, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            __hip_atomic_store(w + 16 * DMAX + 16 + r16, l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned* c = counters + (size_t)tile * n_kv + hk;
+            const unsigned before = __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            am_last = before == (unsigned)splits - 1u;
+            if (before == (unsigned)splits - 1u) __hip_atomic_store(c, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!am_last) return;
+        constexpr int MAXS = 16;                           // (the caller keeps to it)
+        const float* base = ws + ((size_t)tile * n_kv + hk) * splits * (16 * (DMAX + 2));
+        float pm[MAXS], pl[MAXS];
+        float mn = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < MAXS; ++i) {
+            pm[i] = -INFINITY;
+            pl[i] = 0.f;
+            if (i < splits) {
+                pm[i] = __hip_atomic_load(base + (size_t)i * (16 * (DMAX + 2)) + 16 * DMAX + r16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                pl[i] = __hip_atomic_load(base + (size_t)i * (16 * (DMAX + 2)) + 16 * DMAX + 16 + r16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+        }
+        f32x4_t o[MINE];
+#pragma unroll
+        for (int i = 0; i < MINE; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < MAXS; ++i) mn = fmaxf(mn, pm[i]);
+        float L = 0.f;
+#pragma unroll
+        for (int i = 0; i < MAXS; ++i) {                   // in the order of the parts
+            if (i >= splits) break;
+            const float a = (pm[i] == -INFINITY) ? 0.f : __expf(pm[i] - mn);
+            L += pl[i] * a;
+            const float* pw = base + (size_t)i * (16 * (DMAX + 2));
+#pragma unroll
+            for (int k = 0; k < MINE; ++k)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    o[k][j] += a * __hip_atomic_load(pw + ((dt0 + k) * 4 + j) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+        if (!row_ok) return;
+        const float inv = L > 0.f ? 1.0f / L : 0.f;
+        bf16_t* op = out + ((size_t)(q0 + tq) * n_q + head) * d;
+#pragma unroll
+        for (int i = 0; i < MINE; ++i) {
+            const int dd = (dt0 + i) * 16 + 4 * g;
+            if (dd < d) {
+                uint2 w2;
+                w2.x = pack_bf16x2(o[i][0] * inv, o[i][1] * inv);
+                w2.y = pack_bf16x2(o[i][2] * inv, o[i][3] * inv);
+                if (out_tiles) *reinterpret_cast<uint2*>(out + attention_out_operand_order(q0 + tq, head * d + dd, out_tiles)) = w2;
+                else *reinterpret_cast<uint2*>(op + dd) = w2;
+            }
+        }
+        return;
+    }
+    // partial result for the merge kernel: ws[((tile * n_kv + hk) * splits + sp)] = { O[16][DMAX], m[16], l[16] }
 #pragma unroll
     for (int i = 0; i < MINE; ++i) {
         const int dd = (dt0 + i) * 16 + 4 * g;
@@ -515,7 +588,7 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
                                   const int* tile_row0, int num_tiles, int S, int T, int n_q, int n_kv, int d, float scale,
                                   int window, int splits, float* ws, const void* qkv, const void* qw, const void* kw, int w_dtype,
                                   float eps, const float* cos_t, const float* sin_t, int max_pos, int store, int out_tiles,
-                                  hipStream_t st) {
+                                  unsigned* counters, int n_counters, hipStream_t st) {
     SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
                 "spy_attention_mfma: empty operand");
     SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 256, "spy_attention_mfma: head_dim %d is not a multiple of 16 in 16..256", d);
@@ -539,13 +612,18 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
     }
     const dim3 grid(num_tiles, n_kv, splits);
     const dim3 mgrid(num_tiles, n_kv);
+    // The parts merged by each (tile, kv head)'s last block instead of a second kernel: with counters (zeroed once by the
+    // caller, one per tile and head, left at zero by every call; calls that overlap on one device race on them), up to
+    // 16 parts and head sizes up to 128.
+    unsigned* const cnt = (counters && splits > 1 && splits <= 16 && d <= 128 && (long long)num_tiles * n_kv <= n_counters) ? counters : nullptr;
 #define ATT_LAUNCH(DM, FZ, FL)                                                                                                \
     attention_mfma_kernel<DM, FZ, FL><<<grid, AW * 64, (DM <= 128 ? AW : AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>(  \
         (bf16_t*)out, (const bf16_t*)q, (bf16_t*)kc, (bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,  \
-        tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz, out_tiles)
+        tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz, out_tiles, cnt)
 #define ATT_CASE(DM)                                                                                                          \
     if (qkv) ATT_LAUNCH(DM, true, true); else if (d == DM) ATT_LAUNCH(DM, false, true); else ATT_LAUNCH(DM, false, false);       \
-    if (splits > 1 && qkv)                                                                                                    \
+    if (cnt) {}                                                                                                               \
+    else if (splits > 1 && qkv)                                                                                               \
         attention_merge_kernel<DM, true><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits, 1, out_tiles); \
     else if (splits > 1)                                                                                                      \
         attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits, 1, out_tiles);

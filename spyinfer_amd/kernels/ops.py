@@ -312,11 +312,14 @@ def fused_decode_ok(rows: int, act_dtype, *tiled_weights, max_rows: Optional[int
 
 
 _decode_workspaces = {}
+ATTENTION_COUNTERS = 4096          # counters at the start of the device's workspace (16 KB)
+MERGE_IN_KERNEL = True             # False: the attention's key parts are merged by a second kernel (for measurements)
 
 
 def decode_workspace(device) -> Optional[torch.Tensor]:
-    """The device's workspace of the decode products that split K over blocks (counters that every call leaves at zero,
-    and the blocks' partial sums): made once per device, outside any stream capture, and shared by all calls on the
+    """The device's workspace of the kernels whose blocks meet through memory: the decode products that split K over
+    blocks (counters that every call leaves at zero, and the blocks' partial sums) and the attention whose key parts are
+    merged by a tile's last block (the same counters).  Made once per device, outside any stream capture, and shared by all calls on the
     device, which therefore must not overlap (the engine runs them on one stream).  None while a capture is under way
     and the device has none yet: those products are then not taken."""
     device = torch.device(device)
@@ -647,6 +650,8 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
             ws_floats = hip().lib.spy_attention_mfma_workspace(ctypes.c_int(n_small), ctypes.c_int(n_kv), ctypes.c_int(d),
                                                                ctypes.c_int(splits))
             ws = torch.empty((max(1, ws_floats),), dtype=torch.float32, device=q.device)
+            # with counters the last block of a (tile, kv head) merges its parts; without, a second kernel does
+            counters = decode_workspace(q.device) if splits > 1 and MERGE_IN_KERNEL else None
             if raw is not None:
                 wcode = _code(raw.q_norm_w, "head norm weight") if raw.q_norm_w is not None else F32
                 fused = (_ptr(raw.qkv), _ptr(raw.q_norm_w), _ptr(raw.k_norm_w), ctypes.c_int(wcode), ctypes.c_float(raw.eps),
@@ -657,7 +662,8 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
                          ctypes.c_int(0), ctypes.c_int(0))
             hip().call("spy_attention_mfma", _ptr(out), _ptr(None if raw is not None else q), _ptr(k_cache), _ptr(v_cache), *common,
                        _ptr(small_entry), _ptr(small_row0), ctypes.c_int(n_small), *sizes, ctypes.c_int(splits), _ptr(ws), *fused,
-                       ctypes.c_int(operand.tiles if operand is not None else 0), _Hip.stream())
+                       ctypes.c_int(operand.tiles if operand is not None else 0), _ptr(counters),
+                       ctypes.c_int(0 if counters is None else ATTENTION_COUNTERS), _Hip.stream())
         return operand if operand is not None else out
     hip().call("spy_attention_generic", _ptr(out), _ptr(q), _code(q, "q"), _ptr(k_cache), _ptr(v_cache),
                ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(meta.kv_len), _ptr(meta.block_table),
