@@ -512,36 +512,50 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         }
         __syncthreads();
         if (!am_last) return;
-        constexpr int MAXS = 16;                           // (the caller keeps to it)
-        const float* base = ws + ((size_t)tile * n_kv + hk) * splits * (16 * (DMAX + 2));
+        // All that is read of the parts is asked for before any of it is used, eight parts at a time: one memory round
+        // trip for up to eight parts (a loop that adds as it loads has one per part).
+        constexpr int MAXS = 16, BATCH = 8;                // (the caller keeps to 16 parts)
+        constexpr int PART = 16 * (DMAX + 2);
+        const float* base = ws + ((size_t)tile * n_kv + hk) * splits * PART;
         float pm[MAXS], pl[MAXS];
-        float mn = -INFINITY;
 #pragma unroll
         for (int i = 0; i < MAXS; ++i) {
             pm[i] = -INFINITY;
             pl[i] = 0.f;
             if (i < splits) {
-                pm[i] = __hip_atomic_load(base + (size_t)i * (16 * (DMAX + 2)) + 16 * DMAX + r16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                pl[i] = __hip_atomic_load(base + (size_t)i * (16 * (DMAX + 2)) + 16 * DMAX + 16 + r16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                pm[i] = __hip_atomic_load(base + (size_t)i * PART + 16 * DMAX + r16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                pl[i] = __hip_atomic_load(base + (size_t)i * PART + 16 * DMAX + 16 + r16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
             }
         }
         f32x4_t o[MINE];
 #pragma unroll
         for (int i = 0; i < MINE; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        float mn = -INFINITY, L = 0.f;
 #pragma unroll
-        for (int i = 0; i < MAXS; ++i) mn = fmaxf(mn, pm[i]);
-        float L = 0.f;
+        for (int i0 = 0; i0 < MAXS; i0 += BATCH) {
+            if (i0 >= splits) break;
+            float ov[BATCH][MINE][4];
 #pragma unroll
-        for (int i = 0; i < MAXS; ++i) {                   // in the order of the parts
-            if (i >= splits) break;
-            const float a = (pm[i] == -INFINITY) ? 0.f : __expf(pm[i] - mn);
-            L += pl[i] * a;
-            const float* pw = base + (size_t)i * (16 * (DMAX + 2));
+            for (int i = 0; i < BATCH; ++i)
 #pragma unroll
-            for (int k = 0; k < MINE; ++k)
+                for (int k = 0; k < MINE; ++k)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    o[k][j] += a * __hip_atomic_load(pw + ((dt0 + k) * 4 + j) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    for (int j = 0; j < 4; ++j)
+                        ov[i][k][j] = i0 + i < splits ? __hip_atomic_load(base + (size_t)(i0 + i) * PART + ((dt0 + k) * 4 + j) * 64 + lane,
+                                                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) : 0.f;
+            if (i0 == 0) {
+#pragma unroll
+                for (int i = 0; i < MAXS; ++i) mn = fmaxf(mn, pm[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < BATCH; ++i) {              // in the order of the parts
+                const float a = (pm[i0 + i] == -INFINITY) ? 0.f : __expf(pm[i0 + i] - mn);
+                L += pl[i0 + i] * a;
+#pragma unroll
+                for (int k = 0; k < MINE; ++k)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) o[k][j] += a * ov[i][k][j];
+            }
         }
         if (!row_ok) return;
         const float inv = L > 0.f ? 1.0f / L : 0.f;

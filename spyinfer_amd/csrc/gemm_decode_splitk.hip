@@ -23,6 +23,7 @@
 
 #define SK_COUNTER_BYTES 16384            // 4096 column groups at most
 #define SK_MAX_TILES_PER_BLOCK 16         // CT * MT at most
+#define SK_MAX_PARTS 8                    // parts of K at most
 
 template <int EPI, bool SCALED, typename TC, int MT, int CT, bool XT, bool OT>
 __global__ __launch_bounds__(512, 1) void gemm_decode_splitk_kernel(
@@ -175,20 +176,29 @@ __global__ __launch_bounds__(512, 1) void gemm_decode_splitk_kernel(
     __syncthreads();
     if (!is_last || wave >= 4) return;
     // ---- the last block of the group: the parts in the order of ks, then the epilogue of this wave's units ------------------
+    // (all of this wave's share of the parts is asked for before any of it is used: one memory round trip, where a loop
+    // that adds as it loads has one per part)
+    float pv[MINE][SK_MAX_PARTS][4];
+#pragma unroll
+    for (int p = 0; p < PAIRS; ++p) {
+        if ((p & 3) != wave) continue;
+        const float* q = parts + ((size_t)cg * KS * PAIRS + p) * 256 + lane;
+#pragma unroll
+        for (int k = 0; k < SK_MAX_PARTS; ++k)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                pv[p / 4][k][i] = k < KS ? __hip_atomic_load(q + (size_t)k * PAIRS * 256 + i * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) : 0.f;
+    }
 #pragma unroll
     for (int p = 0; p < PAIRS; ++p) {
         if ((p & 3) != wave) continue;
         const int ct = p / MT, mt = p % MT;
         if (ct >= here) continue;
         f32x4_t v = {0.f, 0.f, 0.f, 0.f};
-        const float* q = parts + ((size_t)cg * KS * PAIRS + p) * 256 + lane;
-        for (int k = 0; k < KS; ++k, q += (size_t)PAIRS * 256) {
-            float t[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) t[i] = __hip_atomic_load(q + i * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        for (int k = 0; k < SK_MAX_PARTS; ++k)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) v[i] += t[i];
-        }
+            for (int i = 0; i < 4; ++i) v[i] += pv[p / 4][k][i];
         const int tile = t0 + ct, n = tile * 16 + 4 * g, m = 16 * mt + r;
         if (SCALED) {
             const float scale = row_scale[m];
@@ -238,7 +248,7 @@ static void sk_shape(int tiles, int nfull, int cus, int* ct_out, int* ks_out) {
         const int groups = (tiles + ct - 1) / ct;
         int ks = cus / groups;
         if (ks > nfull / 16) ks = nfull / 16;
-        if (ks > 16) ks = 16;
+        if (ks > SK_MAX_PARTS) ks = SK_MAX_PARTS;
         if (ks < 2 || groups * ks * 10 < cus * 9) continue;     // (nine in ten compute units at least)
         if (groups * ks > best_blocks) { best_blocks = groups * ks; best_ct = ct; best_ks = ks; }
     }
