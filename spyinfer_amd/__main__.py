@@ -37,6 +37,9 @@ def main(argv=None) -> int:
     ap.add_argument("--max-new-tokens", type=int, default=None)
     ap.add_argument("--ignore-eos", action="store_true")
     ap.add_argument("--prompt-ids", action="append", default=[], help="generate for these token ids and leave (may repeat)")
+    ap.add_argument("--prompt-file", metavar="FILE", help="generate for every line of token ids of this file and leave")
+    ap.add_argument("--random-prompts", metavar="LENGTHS", help="generate for prompts of uniform-random token ids of these "
+                    "lengths (e.g. 5,17,33), drawn with --seed, and leave")
     ap.add_argument("--random-model", metavar="CONFIG_JSON", help="write a random-weights model folder to -m from this "
                     "config.json and --seed, then leave")
     args = ap.parse_args(argv)
@@ -61,7 +64,7 @@ def main(argv=None) -> int:
 
     engine = LLMEngine(args.model_path, dtype=args.dtype, max_num_batched_tokens=args.max_num_batched_tokens,
                        prefill_chunk=args.prefill_chunk, max_num_seqs=args.max_num_seqs, max_model_len=args.max_model_len,
-                       keep_finished_cache=not args.prompt_ids,       # the conversation's further turns compute their new tokens only
+                       keep_finished_cache=False,
                        gpu_memory_utilization=args.gpu_memory_utilization, enforce_eager=args.enforce_eager,
                        kvcache_block_size=args.kvcache_block_size, num_kvcache_blocks=args.num_kvcache_blocks, seed=args.seed)
     params = SamplingParams(temperature=args.temperature, max_new_tokens=args.max_new_tokens, ignore_eos=args.ignore_eos)
@@ -73,14 +76,24 @@ def main(argv=None) -> int:
                     print(out.token, end=" ", flush=True)
         print()
 
-    if args.prompt_ids:
-        ids = [engine.add_request(parse_ids(p), params) for p in args.prompt_ids]
+    prompts = [parse_ids(p) for p in args.prompt_ids]
+    if args.prompt_file:
+        with open(args.prompt_file) as f:
+            prompts += [parse_ids(line) for line in f if line.strip()]
+    if args.random_prompts:
+        import torch
+        g = torch.Generator().manual_seed(args.seed)
+        vocab = engine.model.config.vocab_size
+        prompts += [torch.randint(0, vocab, (n,), generator=g).tolist() for n in parse_ids(args.random_prompts)]
+    if prompts:
+        ids = [engine.add_request(p, params) for p in prompts]
         while engine.has_unfinished_requests():
             engine.step()
         for rid in ids:
             print(" ".join(str(t) for t in engine.get_generated_tokens(rid)))
         return 0
 
+    engine.config.keep_finished_cache = True       # the conversation's further turns compute their new tokens only
     conversation = -1
     while True:
         print("\nUser: ", end="", flush=True)

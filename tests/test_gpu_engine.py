@@ -464,6 +464,16 @@ def test_command_line(folder_a, tmp_path):
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [l for l in r.stdout.strip().splitlines() if l and l[0].isdigit()]
     assert [[int(x) for x in l.split()] for l in lines] == [plain.greedy(p, 5) for p in ps]
+    # the same prompts from a file, one a line; and prompts drawn from --seed by their lengths
+    path = tmp_path / "prompts.txt"
+    path.write_text("".join(",".join(map(str, p)) + "\n" for p in ps) + "\n")
+    r = subprocess.run(base + ["--prompt-file", str(path), "--random-prompts", "6,11", "--seed", "4"], cwd=root, capture_output=True,
+                       text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [[int(x) for x in l.split()] for l in r.stdout.strip().splitlines() if l and l[0].isdigit()]
+    g = torch.Generator().manual_seed(4)
+    drawn = [torch.randint(0, 256, (n,), generator=g).tolist() for n in (6, 11)]
+    assert lines == [plain.greedy(p, 5) for p in ps + drawn]
     talk = "%s\n/new\n%s\n/exit\n" % (",".join(map(str, ps[0])), " ".join(map(str, ps[1])))
     r = subprocess.run(base, cwd=root, input=talk, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-2000:]
