@@ -122,7 +122,9 @@ def test_linear_with_tiled_weights(M, N, K):
                                             (48, 128, 128, 151936, 1e-6), (16, 128, 8320, 8208, 1e-6),
                                             # about a column tile per compute unit and a long K: K split over blocks, the
                                             # group's last block adding the parts (33 to 64 rows; a last group with fewer tiles; 2, 3, 4 parts)
-                                            (64, 4096, 12288, 6144, 1e-6), (40, 4096, 8192, 6128, 1e-5), (52, 5120, 6400, 6160, 1e-6)])
+                                            (64, 4096, 12288, 6144, 1e-6), (40, 4096, 8192, 6128, 1e-5), (52, 5120, 6400, 6160, 1e-6),
+                                            # more than 8 chunks of K for every wave in the loops that ask for the next step's operands ahead
+                                            (40, 9216, 256, 8208, 1e-6), (50, 4096, 36864, 64, 1e-6)])
 def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
     """The chain of a decode step's products with the norms folded in: the residual epilogue adds to the stream,
     prepares bf16(h * w) and the parts of sum(h^2); the next products scale their sums by rsqrt(mean(h^2) + eps).
