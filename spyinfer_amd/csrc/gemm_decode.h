@@ -41,6 +41,30 @@ __device__ __forceinline__ void gd_ss_share(const float* __restrict__ ss_in, int
         for (int mt = 0; mt < MT; ++mt) out[mt] += ss_in[p * MP + 16 * mt + r];
 }
 
+// The residual epilogue for one lane's four columns n .. n + 3 of row m: h = h_old + v goes back to the stream (float32),
+// bf16(h * w_next) to the next product's input (row-major, or in operand order for MT row tiles), and the four lanes of
+// a row add their shares of sum(h^2); lane group 0 writes the row's part to ss_part_row[m].  Rows beyond M write nothing
+// to the stream and the part 0.  wn: the next norm's weight for the four columns, two bfloat16 per word.
+template <bool OT>
+__device__ __forceinline__ void gd_residual_epilogue(const f32x4_t& v, const f32x4_t& h_old, uint2 wn, float* __restrict__ resid_out,
+                                                     bf16_t* __restrict__ xw_out, float* __restrict__ ss_part_row, int m, int n, int g,
+                                                     int M, int N, int MT) {
+    float s = 0.f;
+    if (m < M) {
+        f32x4_t h = h_old;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { h[i] += v[i]; s += h[i] * h[i]; }
+        *reinterpret_cast<f32x4_t*>(resid_out + (size_t)m * N + n) = h;
+        uint2 o;
+        o.x = pack_bf16x2(h[0] * __uint_as_float(wn.x << 16), h[1] * __uint_as_float(wn.x & 0xffff0000u));
+        o.y = pack_bf16x2(h[2] * __uint_as_float(wn.y << 16), h[3] * __uint_as_float(wn.y & 0xffff0000u));
+        *reinterpret_cast<uint2*>(xw_out + (OT ? operand_order(m, n, MT) : (size_t)m * N + n)) = o;
+    }
+    s += __shfl_xor(s, 16, 64);
+    s += __shfl_xor(s, 32, 64);
+    if (g == 0) ss_part_row[m] = s;
+}
+
 struct GdArgs {
     const bf16_t* x; const bf16_t* w; void* c; float* resid; bf16_t* xw_out; const bf16_t* w_next; float* ss_out; const float* ss_in;
     int n_parts; float eps; int M, N, K; bool xt, ot; hipStream_t st;

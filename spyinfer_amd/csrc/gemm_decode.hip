@@ -141,21 +141,7 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     // lane (m = r, g) holds C[m][n_base + 4 g + i]
     const int m = r, n = n_base + 4 * g;
     if (EPI == EPI_RESID) {
-        float s = 0.f;
-        if (m < M) {
-            float* hp = resid_out + (size_t)m * N + n;
-            f32x4_t h = h_old;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { h[i] += acc[0][i]; s += h[i] * h[i]; }
-            *reinterpret_cast<f32x4_t*>(hp) = h;
-            uint2 o;
-            o.x = pack_bf16x2(h[0] * __uint_as_float(wn.x << 16), h[1] * __uint_as_float(wn.x & 0xffff0000u));
-            o.y = pack_bf16x2(h[2] * __uint_as_float(wn.y << 16), h[3] * __uint_as_float(wn.y & 0xffff0000u));
-            *reinterpret_cast<uint2*>(xw_out + (OT ? operand_order(m, n) : (size_t)m * N + n)) = o;
-        }
-        s += __shfl_xor(s, 16, 64);
-        s += __shfl_xor(s, 32, 64);
-        if (g == 0) ss_out[blockIdx.x * 16 + r] = s;     // rows beyond M: 0
+        gd_residual_epilogue<OT>(acc[0], h_old, wn, resid_out, xw_out, ss_out + blockIdx.x * 16, m, n, g, M, N, 1);
         return;
     }
     if (m >= M) return;
@@ -279,20 +265,7 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
                 for (int i = 0; i < 4; ++i) { acc[ct][mt][i] *= scale; if (EPI == EPI_GATED) acc[CT + ct][mt][i] *= scale; }
             }
             if (EPI == EPI_RESID) {
-                float s = 0.f;
-                if (m < M) {
-                    f32x4_t h = h_old;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) { h[i] += acc[ct][mt][i]; s += h[i] * h[i]; }
-                    *reinterpret_cast<f32x4_t*>(resid_out + (size_t)m * N + n) = h;
-                    uint2 o;
-                    o.x = pack_bf16x2(h[0] * __uint_as_float(wn.x << 16), h[1] * __uint_as_float(wn.x & 0xffff0000u));
-                    o.y = pack_bf16x2(h[2] * __uint_as_float(wn.y << 16), h[3] * __uint_as_float(wn.y & 0xffff0000u));
-                    *reinterpret_cast<uint2*>(xw_out + (OT ? operand_order(m, n, MT) : (size_t)m * N + n)) = o;
-                }
-                s += __shfl_xor(s, 16, 64);
-                s += __shfl_xor(s, 32, 64);
-                if (g == 0) ss_out[tile * MP + m] = s;      // rows beyond M: 0
+                gd_residual_epilogue<OT>(acc[ct][mt], h_old, wn, resid_out, xw_out, ss_out + tile * MP, m, n, g, M, N, MT);
                 continue;
             }
             if (m >= M) continue;

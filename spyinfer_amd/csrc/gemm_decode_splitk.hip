@@ -206,21 +206,7 @@ __global__ __launch_bounds__(512, 1) void gemm_decode_splitk_kernel(
             for (int i = 0; i < 4; ++i) v[i] *= scale;
         }
         if (EPI == EPI_RESID) {
-            float s = 0.f;
-            if (m < M) {
-                f32x4_t h = h_old[p / 4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) { h[i] += v[i]; s += h[i] * h[i]; }
-                *reinterpret_cast<f32x4_t*>(resid_out + (size_t)m * N + n) = h;
-                const uint2 w2 = wn[p / 4];
-                uint2 o;
-                o.x = pack_bf16x2(h[0] * __uint_as_float(w2.x << 16), h[1] * __uint_as_float(w2.x & 0xffff0000u));
-                o.y = pack_bf16x2(h[2] * __uint_as_float(w2.y << 16), h[3] * __uint_as_float(w2.y & 0xffff0000u));
-                *reinterpret_cast<uint2*>(xw_out + (OT ? operand_order(m, n, MT) : (size_t)m * N + n)) = o;
-            }
-            s += __shfl_xor(s, 16, 64);
-            s += __shfl_xor(s, 32, 64);
-            if (g == 0) ss_out[tile * MP + m] = s;      // rows beyond M: 0
+            gd_residual_epilogue<OT>(v, h_old[p / 4], wn[p / 4], resid_out, xw_out, ss_out + tile * MP, m, n, g, M, N, MT);
             continue;
         }
         if (m >= M) continue;
