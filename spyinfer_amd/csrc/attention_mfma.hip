@@ -52,9 +52,18 @@ struct FusedQKV {
     int store;              // 0: the new key and value are neither stored nor used (the cache of another call is read)
 };
 
-// This lane's pieces (dims 32 kk + 8 g + e) of a [d] weight vector, as float.
+// This lane's pieces (dims 32 kk + 8 g + e) of a [d] weight vector.  A bfloat16 vector is asked for early and kept as it
+// comes from memory, widened to float only where it is used: widening it at once would wait for it, a memory round trip
+// at the kernel's start.  A float32 vector (a checkpoint that stores its norms so) is read where it is used.
 template <int KK>
-__device__ __forceinline__ void load_weight_pieces(float (&wv)[KK][8], const void* w, int dtype, int g) {
+__device__ __forceinline__ void load_weight_pieces(bf16x8_t (&raw)[KK], const void* w, int dtype, int g) {
+    if (dtype != SPY_F32) {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) raw[kk] = *reinterpret_cast<const bf16x8_t*>(reinterpret_cast<const bf16_t*>(w) + kk * 32 + 8 * g);
+    }
+}
+template <int KK>
+__device__ __forceinline__ void widen_weight_pieces(float (&wv)[KK][8], const bf16x8_t (&raw)[KK], const void* w, int dtype, int g) {
     if (dtype == SPY_F32) {
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
@@ -65,11 +74,9 @@ __device__ __forceinline__ void load_weight_pieces(float (&wv)[KK][8], const voi
         }
     } else {
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            const bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(reinterpret_cast<const bf16_t*>(w) + kk * 32 + 8 * g);
+        for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) wv[kk][e] = bf16_to_f32((bf16_t)v[e]);
-        }
+            for (int e = 0; e < 8; ++e) wv[kk][e] = bf16_to_f32((bf16_t)raw[kk][e]);
     }
 }
 
@@ -194,7 +201,8 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     bf16_t vnew[DT];
     int new_page = -1;
     constexpr int HKF = FUSED ? KK / 2 : 1;
-    float wq[FUSED ? KK : 1][8], wk[FUSED ? KK : 1][8], cs[HKF][8], sn[HKF][8];
+    float cs[HKF][8], sn[HKF][8];
+    bf16x8_t wq_raw[FUSED ? KK : 1], wk_raw[FUSED ? KK : 1];
     const bool normed = FUSED && fz.qw != nullptr, rotated = FUSED && fz.cos_t != nullptr;
     if constexpr (FUSED) {
         if (fz.store) {
@@ -205,9 +213,9 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
             for (int kk = 0; kk < KK; ++kk) knew[kk] = *reinterpret_cast<const bf16x8_t*>(kp_raw + kk * 32 + 8 * g);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) vnew[dt] = vp_raw[dt * 16 + r16];
-            if (normed) load_weight_pieces<KK>(wk, fz.kw, fz.w_dtype, g);
+            if (normed) load_weight_pieces<KK>(wk_raw, fz.kw, fz.w_dtype, g);
         }
-        if (normed) load_weight_pieces<KK>(wq, fz.qw, fz.w_dtype, g);
+        if (normed) load_weight_pieces<KK>(wq_raw, fz.qw, fz.w_dtype, g);
         __builtin_amdgcn_sched_barrier(0);
         has_new = fz.store && n == 1 && newpos >= lo + 32 * b_begin && newpos < lo + 32 * b_end;
     }
@@ -271,9 +279,12 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     if (b_begin + wave < b_end) AM_LOAD_K(b_begin + wave, kpage)
     if constexpr (FUSED) {
         __builtin_amdgcn_sched_barrier(0);
-        norm_rotate<KK>(bq, normed, wq, fz.eps, rotated, cs, sn, d);
+        float wv[KK][8];
+        if (normed) widen_weight_pieces<KK>(wv, wq_raw, fz.qw, fz.w_dtype, g);
+        norm_rotate<KK>(bq, normed, wv, fz.eps, rotated, cs, sn, d);
         if (has_new) {
-            norm_rotate<KK>(knew, normed, wk, fz.eps, rotated, cs, sn, d);
+            if (normed) widen_weight_pieces<KK>(wv, wk_raw, fz.kw, fz.w_dtype, g);
+            norm_rotate<KK>(knew, normed, wv, fz.eps, rotated, cs, sn, d);
             if (new_page < 0 || new_page >= num_pages) has_new = false;   // no page: nothing to store or to use
         }
     }
