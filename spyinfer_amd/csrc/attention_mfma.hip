@@ -128,7 +128,7 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
     int n_q, int n_kv, int d, float scale, int window, int splits, float* __restrict__ ws, FusedQKV fz, int out_tiles,
-    unsigned* counters) {
+    unsigned* counters, int log2p) {
     constexpr int KK = DMAX / 32;   // 32-wide chunks of the head dim for Q.K
     constexpr int DT = DMAX / 16;   // 16-row tiles of the head dim for P.V
     extern __shared__ float lds[];   // the waves' O, m, l: AW (head sizes up to 128) or AW - 1 times (DT * 4 + 2) * 64 floats
@@ -142,6 +142,10 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
 #endif
     const int tile = blockIdx.x, hk = blockIdx.y, sp = blockIdx.z;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: loops over it stay scalar
+    // a key's page and its place inside: a shift and a mask for pages that are a power of two (log2p >= 0), instead of
+    // a division of two dozen instructions per lane, four of them per block of keys
+    auto page_of = [&](int key) { return log2p >= 0 ? key >> log2p : key / P; };
+    auto in_page = [&](int key) { return log2p >= 0 ? key & (P - 1) : key % P; };
     const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
     // FUSED: every entry is one token and has one tile (the host has checked it), so tile t is entry t with query token t:
     // two dependent loads less before the first key can be asked for
@@ -231,8 +235,8 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         if ((B) < b_end) {                                                                                    \
             const int c0_ = lo + 32 * (B);                                                                    \
             const int ka_ = c0_ + 8 * (r16 >> 2) + (r16 & 3), kv_ = c0_ + 8 * g;                              \
-            if (ka_ < kvl) KP = bt[ka_ / P];                                                                  \
-            if (kv_ < kvl) VP = bt[kv_ / P];                                                                  \
+            if (ka_ < kvl) KP = bt[page_of(ka_)];                                                                \
+            if (kv_ < kvl) VP = bt[page_of(kv_)];                                                                \
         }                                                                                                     \
     }
     bf16x8_t ka[KK], kb[KK];
@@ -241,7 +245,7 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     {                                                                                                         \
         const int key_ = lo + 32 * (B) + 8 * (r16 >> 2) + (r16 & 3);                                          \
         const bool ok_ = (KP) >= 0 && (KP) < num_pages;                                                       \
-        const bf16_t* kp_ = kc + (((size_t)(ok_ ? (KP) : 0) * n_kv + hk) * P + key_ % P) * d;                 \
+        const bf16_t* kp_ = kc + (((size_t)(ok_ ? (KP) : 0) * n_kv + hk) * P + in_page(key_)) * d;            \
         _Pragma("unroll") for (int kk = 0; kk < KK; ++kk) {                                                   \
             const int dofs = kk * 32 + 8 * g;                                                                 \
             if (FULL) {                                                                                       \
@@ -260,7 +264,7 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     AM_LOOKUP(b_begin + wave, kpage, vpage)
     AM_LOOKUP(b_begin + wave + AW, kpage_n, vpage_n)
     if constexpr (FUSED) {
-        if (has_new) new_page = bt[newpos / P];
+        if (has_new) new_page = bt[page_of(newpos)];
         if (rotated) {
             const size_t trow = (size_t)min(newpos, fz.max_pos - 1) * (d / 2);
 #pragma unroll
@@ -297,7 +301,7 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         const int key_a = c0 + 8 * (r16 >> 2) + (r16 & 3);      // tile a; tile b is key_a + 4
         const int key_v = c0 + 8 * g;                             // this lane's 8 keys of V
         const bool v_ok = vpage >= 0 && vpage < num_pages;
-        const bf16_t* vp = vc + (((size_t)(v_ok ? vpage : 0) * n_kv + hk) * d) * P + key_v % P;
+        const bf16_t* vp = vc + (((size_t)(v_ok ? vpage : 0) * n_kv + hk) * d) * P + in_page(key_v);
         bf16x8_t vt[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -316,7 +320,7 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
                 if (mine_b) kb[kk] = knew[kk];
             }
             if (mine_a || mine_b) {
-                bf16_t* dst = kc + (((size_t)new_page * n_kv + hk) * P + newpos % P) * d + 8 * g;
+                bf16_t* dst = kc + (((size_t)new_page * n_kv + hk) * P + in_page(newpos)) * d + 8 * g;
 #pragma unroll
                 for (int kk = 0; kk < KK; ++kk) *reinterpret_cast<bf16x8_t*>(dst + kk * 32) = knew[kk];
             }
@@ -328,7 +332,7 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
 #pragma unroll
                     for (int j = 0; j < 8; ++j)
                         if (j == jn) vt[dt][j] = (short)vnew[dt];
-                    vc[(((size_t)new_page * n_kv + hk) * d + dt * 16 + r16) * P + newpos % P] = vnew[dt];
+                    vc[(((size_t)new_page * n_kv + hk) * d + dt * 16 + r16) * P + in_page(newpos)] = vnew[dt];
                 }
             }
         }
@@ -635,6 +639,8 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
     } else {
         SPY_REQUIRE(q, "spy_attention_mfma: no queries");
     }
+    int log2p = -1;                                        // pages of a power of two: shifts instead of divisions
+    if ((P & (P - 1)) == 0) { log2p = 0; while ((1 << log2p) < P) ++log2p; }
     const dim3 grid(num_tiles, n_kv, splits);
     const dim3 mgrid(num_tiles, n_kv);
     // The parts merged by each (tile, kv head)'s last block instead of a second kernel: with counters (zeroed once by the
@@ -644,7 +650,7 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
 #define ATT_LAUNCH(DM, FZ, FL)                                                                                                \
     attention_mfma_kernel<DM, FZ, FL><<<grid, AW * 64, (DM <= 128 ? AW : AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>(  \
         (bf16_t*)out, (const bf16_t*)q, (bf16_t*)kc, (bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,  \
-        tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz, out_tiles, cnt)
+        tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz, out_tiles, cnt, log2p)
 #define ATT_CASE(DM)                                                                                                          \
     if (qkv) ATT_LAUNCH(DM, true, true); else if (d == DM) ATT_LAUNCH(DM, false, true); else ATT_LAUNCH(DM, false, false);       \
     if (cnt) {}                                                                                                               \

@@ -469,6 +469,7 @@ ATT_CASES = [
     (8, 2, 128, 8, [(0, 300), (64, 64), (500, 1)], 130),
     (4, 2, 64, 16, [(900, 70), (1300, 40)], None),                          # few big tiles, many keys: key parts + merge
     (8, 2, 128, 16, [(1500, 33)], 700),
+    (8, 2, 64, 24, [(100, 1), (0, 30), (47, 2), (500, 1)], None),           # pages that are no power of two
 ]
 
 
