@@ -450,6 +450,9 @@ int gd_compute_units() {
 #ifndef GD_WIDE
 #define GD_WIDE 1     // 0: the wide kernel is never taken (for measurements)
 #endif
+#ifndef GD_WIDE_MIN_ROWS
+#define GD_WIDE_MIN_ROWS 9
+#endif
 
 // Column tiles per group of the wide kernel for blocks that walk `per` tiles each with MT row tiles: the CT that moves the
 // fewest bytes through L2, X once per group (MT units per step) and W once per tile (GATES units).
@@ -491,6 +494,10 @@ static bool gd_launch_wide(const GdArgs& a) {
 template <int EPI, bool SCALED, typename TC, bool XT, bool OT>
 static void gd_launch2(const GdArgs& a) {
     constexpr int W = EPI == EPI_GATED ? GD_WAVES_GATED : 8;
+    // (the output head at 9 to 16 rows as well: with a column tile per block its blocks pull as many bytes of X through L2
+    // as of W, 251 us at 16 rows; walking six tiles at a time 222; up to 8 rows the kernel with a tile per block stays,
+    // 187-194 against 206-211 us)
+    if (EPI == EPI_STORE && a.M >= GD_WIDE_MIN_ROWS && a.M <= 16) { if (gd_launch_wide<EPI, SCALED, TC, 1, XT, OT>(a)) return; }
     if (a.M > 48) { if (gd_launch_wide<EPI, SCALED, TC, 4, XT, OT>(a)) return; }
     else if (a.M > 32) { if (gd_launch_wide<EPI, SCALED, TC, 3, XT, OT>(a)) return; }
     else if (a.M > 16) { if (gd_launch_wide<EPI, SCALED, TC, 2, XT, OT>(a)) return; }
