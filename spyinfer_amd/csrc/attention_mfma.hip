@@ -626,8 +626,8 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
     SPY_REQUIRE(splits >= 1 && splits <= 64, "spy_attention_mfma: %d parts (1..64 allowed)", splits);
     SPY_REQUIRE(splits == 1 || ws, "spy_attention_mfma: parts without a workspace");
     SPY_REQUIRE(n_kv <= 65535, "spy_attention_mfma: too many kv heads");
-    SPY_REQUIRE(out_tiles >= 0 && out_tiles <= 4 && (!out_tiles || (T <= 16 * out_tiles && (n_q * d) % 32 == 0 && d % 8 == 0)),
-                "spy_attention_mfma: operand order is for at most 64 rows (%d here) of a width that is a multiple of 32", T);
+    SPY_REQUIRE(out_tiles >= 0 && out_tiles <= 8 && (!out_tiles || (T <= 16 * out_tiles && (n_q * d) % 32 == 0 && d % 8 == 0)),
+                "spy_attention_mfma: operand order is for at most 128 rows (%d here) of a width that is a multiple of 32", T);
     FusedQKV fz = {(const bf16_t*)qkv, qw, kw, w_dtype, eps, cos_t, sin_t, max_pos, store};
     if (qkv) {
         SPY_REQUIRE(T == S && num_tiles == S, "spy_attention_mfma: the fused variant takes single tokens only (%d tokens of %d entries)", T, S);

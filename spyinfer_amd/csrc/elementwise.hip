@@ -86,11 +86,14 @@ __global__ __launch_bounds__(256) void embedding_sumsq_kernel(float* __restrict_
     if (threadIdx.x == 0) ss[t] = s;
 }
 
+// row_tiles: the 16-row tiles that the products reading the result are built with (at least T / 16; ss and the operand
+// order have that many).
 extern "C" int spy_embedding_sumsq(float* out, void* xw, float* ss, const void* table, int table_dtype, const void* w_norm,
-                                   const int* ids, int T, int H, int V, int tiled, hipStream_t st) {
-    SPY_REQUIRE(T > 0 && T <= 64 && H > 0 && V > 0, "spy_embedding_sumsq: T = %d tokens (1..64 allowed)", T);
+                                   const int* ids, int T, int H, int V, int tiled, int row_tiles, hipStream_t st) {
+    SPY_REQUIRE(T > 0 && T <= 128 && H > 0 && V > 0, "spy_embedding_sumsq: T = %d tokens (1..128 allowed)", T);
+    SPY_REQUIRE(row_tiles * 16 >= T && row_tiles <= 8, "spy_embedding_sumsq: %d row tiles for %d tokens", row_tiles, T);
     SPY_REQUIRE(!tiled || H % 32 == 0, "spy_embedding_sumsq: operand order needs a width that is a multiple of 32, not %d", H);
-    SPY_DISPATCH(table_dtype, TW, embedding_sumsq_kernel<TW><<<(T + 15) / 16 * 16, 256, 0, st>>>(out, (bf16_t*)xw, ss, (const TW*)table,
+    SPY_DISPATCH(table_dtype, TW, embedding_sumsq_kernel<TW><<<row_tiles * 16, 256, 0, st>>>(out, (bf16_t*)xw, ss, (const TW*)table,
                                                                                  (const bf16_t*)w_norm, ids, T, H, V, tiled));
     SPY_CHECK_LAUNCH("spy_embedding_sumsq");
     return 0;

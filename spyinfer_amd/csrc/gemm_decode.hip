@@ -288,21 +288,25 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
 // half a chunk at a time (the accumulators of CT tiles take the registers of the other half); the waves' sums of one
 // column tiles are added through LDS in two rounds, in a fixed order, and the four waves that end up with them run the
 // epilogue, each for every fourth (column tile, row tile) unit.  Store and gated epilogues only.
-template <int EPI, bool SCALED, typename TC, int MT, int CT, bool XT, bool OT>
-__global__ __launch_bounds__(512, 1) void gemm_decode_wide_kernel(
+// GW: waves per block.  8 up to four row tiles; 4 beyond (65 to 128 rows), where a wave's sums of a group take up to 192
+// registers and a SIMD has one wave with all 512 of its registers.
+template <int EPI, bool SCALED, typename TC, int MT, int CT, bool XT, bool OT, int GW = 8>
+__global__ __launch_bounds__(GW * 64, 1) void gemm_decode_wide_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, const float* __restrict__ ss_in,
     int n_parts, float eps, int M, int N, int K) {
     static_assert(EPI == EPI_STORE || EPI == EPI_GATED, "the wide kernel has no residual epilogue");
-    static_assert((EPI == EPI_GATED ? 2 : 1) * CT * MT <= 24, "the accumulators of a group must fit the registers");
-    constexpr int GW = 8;
+    static_assert(GW == 8 || GW == 4, "four or eight waves");
+    static_assert((EPI == EPI_GATED ? 2 : 1) * CT * MT <= (GW == 8 ? 24 : 48), "the accumulators of a group must fit the registers");
     constexpr int GATES = EPI == EPI_GATED ? 2 : 1;
     constexpr int NT = GATES * CT;
     constexpr int MP = 16 * MT;
     constexpr int PAIRS = CT * MT;                       // (column tile, row tile) units of the epilogue
-    // the waves' sums meet in two rounds: waves 4..7 hand all of theirs to waves 0..3, then each of these four takes
-    // every fourth unit from the other three.  The second round's buffer lies inside the first's.
-    __shared__ f32x4_t red[4 * NT * MT * 64];
-    static_assert(PAIRS * 3 * GATES <= 4 * NT * MT, "the second round fits the first round's buffer");
+    // the waves' sums meet in two rounds: waves 4..7 (if there are eight) hand all of theirs to waves 0..3, then each of
+    // these four takes every fourth unit from the other three, PB units at a time (72 KB of LDS at most).  The second
+    // round's buffer lies inside the first's.
+    constexpr int PB = PAIRS * 3 * GATES <= 72 ? PAIRS : 72 / (3 * GATES) / 4 * 4;
+    constexpr int RED_TILES = (GW == 8 && 4 * NT * MT > PB * 3 * GATES) ? 4 * NT * MT : PB * 3 * GATES;
+    __shared__ f32x4_t red[RED_TILES * 64];
     __shared__ float ss_red[GW * 4 * MP];
     __shared__ float row_scale[MP];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -359,12 +363,30 @@ __global__ __launch_bounds__(512, 1) void gemm_decode_wide_kernel(
             _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                        \
                 _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                    \
                     acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[nt], B[mt], acc[nt][mt], 0, 0, 0);
-            if (my_steps > 0) GDW_LOAD(a0, b0, 0)
-            for (int st = 0; st < my_steps; st += 2) {     // (a multiple of 4)
-                GDW_LOAD(a1, b1, st + 1)
-                GDW_MFMA(a0, b0)
-                if (st + 2 < my_steps) GDW_LOAD(a0, b0, st + 2)
-                GDW_MFMA(a1, b1)
+            if constexpr (GW == 4 && NT + MT <= 12) {
+                // a wave that has a SIMD's registers to itself keeps three steps' operands under way instead of one (four
+                // waves with one step each would have too few bytes in flight to keep the memory busy), where four steps'
+                // operands fit the 256 registers that loads can write
+                bf16x8_t a2[NT], b2[MT], a3[NT], b3[MT];
+                if (my_steps > 0) { GDW_LOAD(a0, b0, 0) GDW_LOAD(a1, b1, 1) GDW_LOAD(a2, b2, 2) }
+                for (int st = 0; st < my_steps; st += 4) {     // (a multiple of 4)
+                    GDW_LOAD(a3, b3, st + 3)
+                    GDW_MFMA(a0, b0)
+                    if (st + 4 < my_steps) GDW_LOAD(a0, b0, st + 4)
+                    GDW_MFMA(a1, b1)
+                    if (st + 4 < my_steps) GDW_LOAD(a1, b1, st + 5)
+                    GDW_MFMA(a2, b2)
+                    if (st + 4 < my_steps) GDW_LOAD(a2, b2, st + 6)
+                    GDW_MFMA(a3, b3)
+                }
+            } else {
+                if (my_steps > 0) GDW_LOAD(a0, b0, 0)
+                for (int st = 0; st < my_steps; st += 2) {     // (a multiple of 4)
+                    GDW_LOAD(a1, b1, st + 1)
+                    GDW_MFMA(a0, b0)
+                    if (st + 2 < my_steps) GDW_LOAD(a0, b0, st + 2)
+                    GDW_MFMA(a1, b1)
+                }
             }
 #undef GDW_LOAD
 #undef GDW_MFMA
@@ -374,63 +396,67 @@ __global__ __launch_bounds__(512, 1) void gemm_decode_wide_kernel(
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) ss_red[(wave * 4 + g) * MP + 16 * mt + r] = ss_part[mt];
         }
-        if (wave >= 4) {
+        if (GW == 8 && wave >= 4) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) red[(((wave - 4) * NT + nt) * MT + mt) * 64 + lane] = acc[nt][mt];
         }
-        __syncthreads();
-        if (SCALED && t0 == t_begin && threadIdx.x >= 256 && threadIdx.x < 256 + MP) {      // (a wave that has nothing to add now)
-            const int m = threadIdx.x - 256;
+        if (GW == 8 || (SCALED && t0 == t_begin)) __syncthreads();
+        // (the rows' scales: by a wave that has nothing to add now, if there is one)
+        const int t_scale = (int)threadIdx.x - (GW == 8 ? 256 : 0);
+        if (SCALED && t0 == t_begin && t_scale >= 0 && t_scale < MP) {
             float s = 0.f;
-            for (int i = 0; i < GW * 4; ++i) s += ss_red[i * MP + m];
-            row_scale[m] = 1.0f / sqrtf(s / (float)K + eps);
+            for (int i = 0; i < GW * 4; ++i) s += ss_red[i * MP + t_scale];
+            row_scale[t_scale] = 1.0f / sqrtf(s / (float)K + eps);
         }
-        if (wave < 4) {
+        if (GW == 8 && wave < 4) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[nt][mt] += red[((wave * NT + nt) * MT + mt) * 64 + lane];
         }
-        __syncthreads();
+        if (GW == 8 || (SCALED && t0 == t_begin)) __syncthreads();
         // ---- round two: unit p = ct MT + mt (its gate and its up tile) belongs to wave p % 4 --------------------------
-        if (wave < 4) {
 #pragma unroll
-            for (int p = 0; p < PAIRS; ++p) {
-                const int owner = p & 3;
-                if (wave != owner) {
-                    const int slot = wave < owner ? wave : wave - 1;
+        for (int p0 = 0; p0 < PAIRS; p0 += PB) {
+            if (wave < 4) {
 #pragma unroll
-                    for (int gt = 0; gt < GATES; ++gt) red[((p * 3 + slot) * GATES + gt) * 64 + lane] = acc[gt * CT + p / MT][p % MT];
+                for (int p = p0; p < p0 + PB && p < PAIRS; ++p) {
+                    const int owner = p & 3;
+                    if (wave != owner) {
+                        const int slot = wave < owner ? wave : wave - 1;
+#pragma unroll
+                        for (int gt = 0; gt < GATES; ++gt) red[(((p - p0) * 3 + slot) * GATES + gt) * 64 + lane] = acc[gt * CT + p / MT][p % MT];
+                    }
                 }
             }
-        }
-        __syncthreads();
-        if (wave < 4) {
+            __syncthreads();
+            if (wave < 4) {
 #pragma unroll
-            for (int p = 0; p < PAIRS; ++p) {
-                if (wave != (p & 3)) continue;
-                const int ct = p / MT, mt = p % MT;
-                f32x4_t v = acc[ct][mt], up = acc[(GATES - 1) * CT + ct][mt];
+                for (int p = p0; p < p0 + PB && p < PAIRS; ++p) {
+                    if (wave != (p & 3)) continue;
+                    const int ct = p / MT, mt = p % MT;
+                    f32x4_t v = acc[ct][mt], up = acc[(GATES - 1) * CT + ct][mt];
 #pragma unroll
-                for (int slot = 0; slot < 3; ++slot) {
-                    v += red[((p * 3 + slot) * GATES + 0) * 64 + lane];
-                    if (EPI == EPI_GATED) up += red[((p * 3 + slot) * GATES + GATES - 1) * 64 + lane];
-                }
-                const int n = (t0 + ct) * 16 + 4 * g, m = 16 * mt + r;
-                if (ct >= here || m >= M) continue;
-                const float scale = SCALED ? row_scale[m] : 1.f;
-                TC* out = C + (OT ? operand_order(m, n, MT) : (size_t)m * N + n);
+                    for (int slot = 0; slot < 3; ++slot) {
+                        v += red[(((p - p0) * 3 + slot) * GATES + 0) * 64 + lane];
+                        if (EPI == EPI_GATED) up += red[(((p - p0) * 3 + slot) * GATES + GATES - 1) * 64 + lane];
+                    }
+                    const int n = (t0 + ct) * 16 + 4 * g, m = 16 * mt + r;
+                    if (ct >= here || m >= M) continue;
+                    const float scale = SCALED ? row_scale[m] : 1.f;
+                    TC* out = C + (OT ? operand_order(m, n, MT) : (size_t)m * N + n);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float y = v[i] * scale;
-                    if (EPI == EPI_GATED) { const float u = up[i] * scale; y = (y / (1.0f + expf(-y))) * u; }
-                    out[i] = from_f32<TC>(y);
+                    for (int i = 0; i < 4; ++i) {
+                        float y = v[i] * scale;
+                        if (EPI == EPI_GATED) { const float u = up[i] * scale; y = (y / (1.0f + expf(-y))) * u; }
+                        out[i] = from_f32<TC>(y);
+                    }
                 }
             }
+            __syncthreads();                              // the buffer is free for the next units, or the next group
         }
-        __syncthreads();                                  // the buffer is free for the next group
     }
 }
 
@@ -472,15 +498,23 @@ static bool gd_launch_wide(const GdArgs& a) {
     if constexpr (EPI == EPI_RESID || !SCALED || !XT) return false;
     else {
         constexpr int GATES = EPI == EPI_GATED ? 2 : 1;
+        constexpr int GW = MT > 4 ? 4 : 8;               // beyond four row tiles: four waves with a SIMD's registers each
         // a group's accumulators (GATES * CT * MT tiles of four registers) leave room for its operands up to 24 tiles
-        constexpr int MAX_CT = 24 / (GATES * MT) < 6 ? 24 / (GATES * MT) : 6;
+        // (48 for a wave that has a SIMD to itself)
+        constexpr int ROOM = GW == 8 ? 24 : 48;
+        constexpr int MAX_CT = ROOM / (GATES * MT) < 6 ? ROOM / (GATES * MT) : 6;
         const int cus = gd_compute_units(), tiles = a.N / 16;
-        if (!GD_WIDE || tiles < 2 * cus) return false;       // fewer than two tiles per CU: one tile per block, two blocks per CU
-        const int ct = wide_ct((tiles + cus - 1) / cus, MT, GATES, MAX_CT);
+        // fewer than two tiles per CU: one tile per block, two blocks per CU (beyond four row tiles the gated product has
+        // no other kernel: it walks here whatever the width, two column tiles at a time at least)
+        const bool only = MT > 4 && EPI == EPI_GATED;
+        if (!GD_WIDE || (tiles < 2 * cus && !only)) return false;
+        int ct = wide_ct((tiles + cus - 1) / cus, MT, GATES, MAX_CT);
+        if (only && ct < 2) ct = 2;
+        const int blocks = tiles < cus ? tiles : cus;
 #define GD_WIDE_CASE(C)                                                                                               \
         if constexpr (C <= MAX_CT) {                                                                                  \
             if (ct == C) {                                                                                            \
-                gemm_decode_wide_kernel<EPI, SCALED, TC, MT, C, XT, OT><<<cus, 512, 0, a.st>>>(                        \
+                gemm_decode_wide_kernel<EPI, SCALED, TC, MT, C, XT, OT, GW><<<blocks, GW * 64, 0, a.st>>>(                \
                     a.x, a.w, (TC*)a.c, a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K);                                    \
                 return true;                                                                                          \
             }                                                                                                         \
@@ -491,45 +525,60 @@ static bool gd_launch_wide(const GdArgs& a) {
     }
 }
 
+// false: this combination is not built for the call's number of rows (beyond 64 rows only what a decode step has is built)
 template <int EPI, bool SCALED, typename TC, bool XT, bool OT>
-static void gd_launch2(const GdArgs& a) {
+static bool gd_launch2(const GdArgs& a) {
     constexpr int W = EPI == EPI_GATED ? GD_WAVES_GATED : 8;
     // (the output head at 9 to 16 rows as well: with a column tile per block its blocks pull as many bytes of X through L2
     // as of W, 251 us at 16 rows; walking six tiles at a time 222; up to 8 rows the kernel with a tile per block stays,
     // 187-194 against 206-211 us)
-    if (EPI == EPI_STORE && a.M >= GD_WIDE_MIN_ROWS && a.M <= 16) { if (gd_launch_wide<EPI, SCALED, TC, 1, XT, OT>(a)) return; }
-    if (a.M > 48) { if (gd_launch_wide<EPI, SCALED, TC, 4, XT, OT>(a)) return; }
-    else if (a.M > 32) { if (gd_launch_wide<EPI, SCALED, TC, 3, XT, OT>(a)) return; }
-    else if (a.M > 16) { if (gd_launch_wide<EPI, SCALED, TC, 2, XT, OT>(a)) return; }
+    if (EPI == EPI_STORE && a.M >= GD_WIDE_MIN_ROWS && a.M <= 16) { if (gd_launch_wide<EPI, SCALED, TC, 1, XT, OT>(a)) return true; }
+    if (a.M > 96) { if (gd_launch_wide<EPI, SCALED, TC, 8, XT, OT>(a)) return true; }
+    else if (a.M > 64) { if (gd_launch_wide<EPI, SCALED, TC, 6, XT, OT>(a)) return true; }
+    else if (a.M > 48) { if (gd_launch_wide<EPI, SCALED, TC, 4, XT, OT>(a)) return true; }
+    else if (a.M > 32) { if (gd_launch_wide<EPI, SCALED, TC, 3, XT, OT>(a)) return true; }
+    else if (a.M > 16) { if (gd_launch_wide<EPI, SCALED, TC, 2, XT, OT>(a)) return true; }
 #define GD_ARGS a.x, a.w, (TC*)a.c, a.resid, a.xw_out, a.w_next, a.ss_out, a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K
     // Two column tiles per block where that leaves enough blocks (measured, 64 rows: qkv of 6144 columns 26.8 -> 20.5
     // us; with 4096 columns, 128 blocks, 15.4 -> 19.4 us; the gated product 53 -> 61 us: its block has one wave per SIMD then)
     const bool two = EPI == EPI_STORE && a.N % 32 == 0 && a.N / 32 >= 192;
+    // beyond four row tiles: blocks of eight waves (a wave per row tile runs the epilogue), one column tile; built for
+    // what a decode step has: inputs in operand order, the residual product of a plain input with its output in operand
+    // order, the stored product of a normed input
+    constexpr bool TALL = XT && ((EPI == EPI_RESID && !SCALED && OT) || (EPI == EPI_STORE && SCALED));
     if (a.M <= 16) gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
 #define GD_ROWS(MT)                                                                                                  \
     if constexpr (EPI == EPI_STORE) {                                                                                \
         if (two) gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 2, W, XT, OT><<<a.N / 32, W * 64, 0, a.st>>>(GD_ARGS);   \
         else gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 1, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);      \
     } else gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 1, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS)
+#define GD_ROWS_TALL(MT)                                                                                             \
+    if constexpr (TALL) gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 1, 8, XT, OT><<<a.N / 16, 512, 0, a.st>>>(GD_ARGS); \
+    else return false;
     else if (a.M <= 32) { GD_ROWS(2); }
     else if (a.M <= 48) { GD_ROWS(3); }
-    else { GD_ROWS(4); }
+    else if (a.M <= 64) { GD_ROWS(4); }
+    else if (a.M <= 96) { GD_ROWS_TALL(6) }
+    else { GD_ROWS_TALL(8) }
+#undef GD_ROWS_TALL
 #undef GD_ROWS
 #undef GD_ARGS
+    return true;
 }
 
 template <int EPI, bool SCALED, typename TC>
-static void gd_launch(const GdArgs& a) {
+static bool gd_launch(const GdArgs& a) {
     constexpr bool CAN_OT = EPI != EPI_STORE && sizeof(TC) == 2;      // operand order is for bfloat16 that a product reads next
-    if (a.xt) { if (CAN_OT && a.ot) gd_launch2<EPI, SCALED, TC, true, CAN_OT>(a); else gd_launch2<EPI, SCALED, TC, true, false>(a); }
-    else { if (CAN_OT && a.ot) gd_launch2<EPI, SCALED, TC, false, CAN_OT>(a); else gd_launch2<EPI, SCALED, TC, false, false>(a); }
+    if (a.xt) return (CAN_OT && a.ot) ? gd_launch2<EPI, SCALED, TC, true, CAN_OT>(a) : gd_launch2<EPI, SCALED, TC, true, false>(a);
+    return (CAN_OT && a.ot) ? gd_launch2<EPI, SCALED, TC, false, CAN_OT>(a) : gd_launch2<EPI, SCALED, TC, false, false>(a);
 }
 
 // Bytes of the device's workspace for the products that split K over blocks: zeroed once by the caller, then handed to
 // every call on that device (ws; none: those products are not taken).  Calls on one device that overlap race on it.
 extern "C" int64_t spy_gemm_decode_workspace() { return gd_splitk_workspace_bytes(); }
 
-// x: bfloat16 [M, K], M <= 64; MP = M rounded up to a multiple of 16.  scaled != 0: x = bf16(h * w_norm) and ss_in
+// x: bfloat16 [M, K], M <= 128; MP = 16 times the row tiles the kernel is built with (M rounded up to 16 up to 64 rows, 96
+// or 128 beyond).  scaled != 0: x = bf16(h * w_norm) and ss_in
 // [n_parts, MP] holds the parts of sum(h^2); the result is multiplied by rsqrt(sum / K + eps).
 // epi 0: C [M, N] (c_dtype);  epi 1: W = [gate | up], C [M, N] = silu(gate) * up;  epi 2: resid [M, N] += result,
 // xw_out [M, N] = bf16(resid * w_next), ss_out [N / 16, MP] = every block's part of the rows' sums of squares.
@@ -537,7 +586,7 @@ extern "C" int64_t spy_gemm_decode_workspace() { return gd_splitk_workspace_byte
 extern "C" int spy_gemm_decode(const void* X, int scaled, const float* ss_in, int n_parts, float eps, const void* Wt, int epi,
                                void* C, int c_dtype, float* resid, void* xw_out, const void* w_next, float* ss_out, int M, int N,
                                int K, int x_tiled, int out_tiled, void* ws, int64_t ws_bytes, hipStream_t st) {
-    SPY_REQUIRE(M > 0 && M <= 64, "spy_gemm_decode: M = %d rows (1..64 allowed)", M);
+    SPY_REQUIRE(M > 0 && M <= 128, "spy_gemm_decode: M = %d rows (1..128 allowed)", M);
     SPY_REQUIRE(N > 0 && N % 16 == 0 && K > 0 && K % 128 == 0, "spy_gemm_decode: N = %d must be a multiple of 16 and K = %d of 128", N, K);
     SPY_REQUIRE(epi >= 0 && epi <= 2, "spy_gemm_decode: unknown epilogue %d", epi);
     SPY_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)Wt % 16) == 0, "spy_gemm_decode: operands must be 16-byte aligned");
@@ -556,14 +605,17 @@ extern "C" int spy_gemm_decode(const void* X, int scaled, const float* ss_in, in
         SPY_CHECK_LAUNCH("spy_gemm_decode");
         return 0;
     }
-    if (epi == EPI_RESID) { if (scaled) gd_launch<EPI_RESID, true, bf16_t>(a); else gd_launch<EPI_RESID, false, bf16_t>(a); }
+    bool built;
+    if (epi == EPI_RESID) built = scaled ? gd_launch<EPI_RESID, true, bf16_t>(a) : gd_launch<EPI_RESID, false, bf16_t>(a);
     else if (epi == EPI_GATED) {
-        if (scaled) { if (f32) gd_launch<EPI_GATED, true, float>(a); else gd_launch<EPI_GATED, true, bf16_t>(a); }
-        else { if (f32) gd_launch<EPI_GATED, false, float>(a); else gd_launch<EPI_GATED, false, bf16_t>(a); }
+        if (scaled) built = f32 ? gd_launch<EPI_GATED, true, float>(a) : gd_launch<EPI_GATED, true, bf16_t>(a);
+        else built = f32 ? gd_launch<EPI_GATED, false, float>(a) : gd_launch<EPI_GATED, false, bf16_t>(a);
     } else {
-        if (scaled) { if (f32) gd_launch<EPI_STORE, true, float>(a); else gd_launch<EPI_STORE, true, bf16_t>(a); }
-        else { if (f32) gd_launch<EPI_STORE, false, float>(a); else gd_launch<EPI_STORE, false, bf16_t>(a); }
+        if (scaled) built = f32 ? gd_launch<EPI_STORE, true, float>(a) : gd_launch<EPI_STORE, true, bf16_t>(a);
+        else built = f32 ? gd_launch<EPI_STORE, false, float>(a) : gd_launch<EPI_STORE, false, bf16_t>(a);
     }
+    SPY_REQUIRE(built, "spy_gemm_decode: %d rows: beyond 64 rows the product is built for inputs in operand order only, as the stored or "
+                "gated product of a normed input or the residual product of a plain input with its output in operand order", M);
     SPY_CHECK_LAUNCH("spy_gemm_decode");
     return 0;
 }

@@ -1,4 +1,4 @@
-// Decode products of 33 to 64 rows for matrices with about one column tile of 16 per compute unit (o, down, qkv).
+// Decode products of 33 to 128 rows for matrices with about one column tile of 16 per compute unit (o, down, qkv).
 //
 // With a column tile per block every block pulls all of X through L2, MT row tiles against one tile of W: MT times the
 // bytes of W, and the L2's throughput bounds the product, not the matrix' way from memory.  Sharing the X fragments
@@ -22,23 +22,24 @@
 #include <math.h>
 
 #define SK_COUNTER_BYTES 16384            // 4096 column groups at most
-#define SK_MAX_TILES_PER_BLOCK 16         // CT * MT at most
+#define SK_MAX_TILES_PER_BLOCK 32         // CT * MT at most
 #define SK_MAX_PARTS 8                    // parts of K at most
 
-template <int EPI, bool SCALED, typename TC, int MT, int CT, bool XT, bool OT>
-__global__ __launch_bounds__(512, 1) void gemm_decode_splitk_kernel(
+// GW: waves per block, 8 up to four row tiles, 4 beyond (a wave then has a SIMD's registers to itself).
+template <int EPI, bool SCALED, typename TC, int MT, int CT, bool XT, bool OT, int GW = 8>
+__global__ __launch_bounds__(GW * 64, 1) void gemm_decode_splitk_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, float* __restrict__ resid_out,
     bf16_t* __restrict__ xw_out, const bf16_t* __restrict__ w_next, float* __restrict__ ss_out, const float* __restrict__ ss_in,
     int n_parts, float eps, int M, int N, int K, int KS, unsigned* counters, float* parts) {
     static_assert(EPI == EPI_STORE || EPI == EPI_RESID, "store and residual epilogues");
-    static_assert(CT * MT <= SK_MAX_TILES_PER_BLOCK, "the sums must fit the registers and the workspace");
-    constexpr int GW = 8;
+    static_assert(GW == 8 || GW == 4, "four or eight waves");
+    static_assert(CT * MT <= (GW == 8 ? 16 : SK_MAX_TILES_PER_BLOCK), "the sums must fit the registers and the workspace");
     constexpr int MP = 16 * MT;
     constexpr int PAIRS = CT * MT;                       // (column tile, row tile) units: p = ct MT + mt, owned by wave p % 4
     constexpr int MINE = (PAIRS + 3) / 4;                // units of a wave at most
     // the waves' sums meet in two rounds: waves 4..7 hand all of theirs to waves 0..3, then each of these four takes
     // every fourth unit from the other three.  The second round's buffer lies inside the first's.
-    __shared__ f32x4_t red[4 * PAIRS * 64];
+    __shared__ f32x4_t red[(GW == 8 ? 4 : 3) * PAIRS * 64];
     __shared__ float ss_red[SCALED ? GW * 4 * MP : 1];
     __shared__ float row_scale[SCALED ? MP : 1];
     __shared__ unsigned is_last;
@@ -108,12 +109,28 @@ __global__ __launch_bounds__(512, 1) void gemm_decode_splitk_kernel(
         _Pragma("unroll") for (int ct = 0; ct < CT; ++ct)                                                            \
             _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                        \
                 acc[ct][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[ct], B[mt], acc[ct][mt], 0, 0, 0);
-        if (my_steps > 0) SK_LOAD(a0, b0, 0)
-        for (int st = 0; st < my_steps; st += 2) {         // (a multiple of 4)
-            SK_LOAD(a1, b1, st + 1)
-            SK_MFMA(a0, b0)
-            if (st + 2 < my_steps) SK_LOAD(a0, b0, st + 2)
-            SK_MFMA(a1, b1)
+        if constexpr (GW == 4) {
+            // (a wave that has a SIMD's registers to itself keeps three steps' operands under way instead of one)
+            bf16x8_t a2[CT], b2[MT], a3[CT], b3[MT];
+            if (my_steps > 0) { SK_LOAD(a0, b0, 0) SK_LOAD(a1, b1, 1) SK_LOAD(a2, b2, 2) }
+            for (int st = 0; st < my_steps; st += 4) {     // (a multiple of 4)
+                SK_LOAD(a3, b3, st + 3)
+                SK_MFMA(a0, b0)
+                if (st + 4 < my_steps) SK_LOAD(a0, b0, st + 4)
+                SK_MFMA(a1, b1)
+                if (st + 4 < my_steps) SK_LOAD(a1, b1, st + 5)
+                SK_MFMA(a2, b2)
+                if (st + 4 < my_steps) SK_LOAD(a2, b2, st + 6)
+                SK_MFMA(a3, b3)
+            }
+        } else {
+            if (my_steps > 0) SK_LOAD(a0, b0, 0)
+            for (int st = 0; st < my_steps; st += 2) {     // (a multiple of 4)
+                SK_LOAD(a1, b1, st + 1)
+                SK_MFMA(a0, b0)
+                if (st + 2 < my_steps) SK_LOAD(a0, b0, st + 2)
+                SK_MFMA(a1, b1)
+            }
         }
 #undef SK_LOAD
 #undef SK_MFMA
@@ -123,26 +140,26 @@ __global__ __launch_bounds__(512, 1) void gemm_decode_splitk_kernel(
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) ss_red[(wave * 4 + g) * MP + 16 * mt + r] = ss_part[mt];
     }
-    if (wave >= 4) {
+    if (GW == 8 && wave >= 4) {
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) red[(((wave - 4) * CT + ct) * MT + mt) * 64 + lane] = acc[ct][mt];
     }
-    __syncthreads();
-    if (SCALED && threadIdx.x >= 256 && threadIdx.x < 256 + MP) {      // (a wave that has nothing to add now)
-        const int m = threadIdx.x - 256;
+    if (GW == 8 || SCALED) __syncthreads();
+    const int t_scale = (int)threadIdx.x - (GW == 8 ? 256 : 0);        // (a wave that has nothing to add now, if there is one)
+    if (SCALED && t_scale >= 0 && t_scale < MP) {
         float s = 0.f;
-        for (int i = 0; i < GW * 4; ++i) s += ss_red[i * MP + m];
-        row_scale[m] = 1.0f / sqrtf(s / (float)K + eps);
+        for (int i = 0; i < GW * 4; ++i) s += ss_red[i * MP + t_scale];
+        row_scale[t_scale] = 1.0f / sqrtf(s / (float)K + eps);
     }
-    if (wave < 4) {
+    if (GW == 8 && wave < 4) {
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) acc[ct][mt] += red[((wave * CT + ct) * MT + mt) * 64 + lane];
     }
-    __syncthreads();
+    if (GW == 8 || SCALED) __syncthreads();
     // ---- round two: unit p to wave p % 4 ---------------------------------------------------------------------------------
     if (wave < 4) {
 #pragma unroll
@@ -253,9 +270,10 @@ static bool sk_launch(const GdArgs& a) {
     if (a.ws_bytes < gd_splitk_workspace_bytes()) return false;
     unsigned* counters = reinterpret_cast<unsigned*>(a.ws);
     float* parts = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws) + SK_COUNTER_BYTES);
+    constexpr int GW = MT > 4 ? 4 : 8;
 #define SK_CASE(C)                                                                                                      \
     if (ct == C) {                                                                                                      \
-        gemm_decode_splitk_kernel<EPI, SCALED, TC, MT, C, XT, OT><<<groups * ks, 512, 0, a.st>>>(                        \
+        gemm_decode_splitk_kernel<EPI, SCALED, TC, MT, C, XT, OT, GW><<<groups * ks, GW * 64, 0, a.st>>>(                \
             a.x, a.w, (TC*)a.c, a.resid, a.xw_out, a.w_next, a.ss_out, a.ss_in, a.n_parts, a.eps, a.M, a.N, a.K, ks, counters, parts); \
         return true;                                                                                                    \
     }
@@ -266,6 +284,11 @@ static bool sk_launch(const GdArgs& a) {
 
 template <int EPI, bool SCALED, typename TC, bool XT, bool OT>
 static bool sk_rows(const GdArgs& a) {
+    if constexpr (XT) {                                   // (beyond 64 rows: inputs in operand order only)
+        if (a.M > 96) return sk_launch<EPI, SCALED, TC, 8, XT, OT>(a);
+        if (a.M > 64) return sk_launch<EPI, SCALED, TC, 6, XT, OT>(a);
+    }
+    if (a.M > 64) return false;
     if (a.M > 48) return sk_launch<EPI, SCALED, TC, 4, XT, OT>(a);
     return sk_launch<EPI, SCALED, TC, 3, XT, OT>(a);
 }
@@ -274,7 +297,7 @@ static bool sk_rows(const GdArgs& a) {
 // order) with its output in operand order, and the stored bfloat16 product of a normed input in operand order.
 bool gd_splitk_try(const GdArgs& a, int epi, bool scaled, bool f32_out) {
     // (up to 32 rows the kernels with a column tile per block are as fast: down 23.5 against 23.6 us at 32 rows)
-    if (!GD_SPLITK || a.ws == nullptr || a.M <= 32 || a.M > 64 || a.N % 16 != 0 || a.K % GD_CHUNK != 0) return false;
+    if (!GD_SPLITK || a.ws == nullptr || a.M <= 32 || a.M > 128 || a.N % 16 != 0 || a.K % GD_CHUNK != 0) return false;
     if (a.N / 16 >= 2 * gd_compute_units()) return false;           // many columns: the kernels that walk column tiles
     if (epi == EPI_RESID && !scaled && a.ot) {
         return a.xt ? sk_rows<EPI_RESID, false, bf16_t, true, true>(a) : sk_rows<EPI_RESID, false, bf16_t, false, true>(a);

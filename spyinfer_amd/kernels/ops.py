@@ -158,7 +158,7 @@ _LIBRARY_F32_OUT = True      # torch.mm(..., out_dtype=float32) exists in this t
 #: library product of prefill.
 TILED_WEIGHTS = True
 #: Most rows that the decode products (``decode_linear`` and its kin) take.
-FUSED_DECODE_MAX_ROWS = 64
+FUSED_DECODE_MAX_ROWS = 128
 
 
 def default_fold_rows(weight_elements: int) -> int:
@@ -253,10 +253,16 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, tiled: Optional[torc
 
 # --------------------------------------------------------------------------
 # Decode-time products with the norm and the residual sum folded in
+def row_tiles(rows: int) -> int:
+    """Row tiles of 16 that the decode products are built with for ``rows`` rows: as many as the rows need up to four
+    (64 rows); beyond, six (65 to 96 rows) or eight (97 to 128)."""
+    return -(-rows // 16) if rows <= 64 else (6 if rows <= 96 else 8)
+
+
 class OperandRows:
-    """Rows of bfloat16 [M, K], M <= 64, in the order the MFMA operand wants them: ``data`` is [K/32 steps, MT row
-    tiles, 64 lanes, 8] with lane 16 g + r of row tile t and step s holding x[16 t + r][32 s + 8 g ..]; MT = ceil(M / 16);
-    rows M.. of the last tile hold anything.  The decode products write their outputs for each other this way (an
+    """Rows of bfloat16 [M, K], M <= 128, in the order the MFMA operand wants them: ``data`` is [K/32 steps, MT row
+    tiles, 64 lanes, 8] with lane 16 g + r of row tile t and step s holding x[16 t + r][32 s + 8 g ..]; MT = row_tiles(M);
+    rows from M on hold anything.  The decode products write their outputs for each other this way (an
     operand is then one load of 1 KiB in one piece)."""
     __slots__ = ("data", "rows", "width")
 
@@ -265,13 +271,13 @@ class OperandRows:
 
     @property
     def tiles(self) -> int:
-        return -(-self.rows // 16)
+        return row_tiles(self.rows)
 
     @staticmethod
     def empty(rows: int, width: int, device) -> "OperandRows":
         _check(0 < rows <= FUSED_DECODE_MAX_ROWS and width % 32 == 0,
                "operand order takes 1..%d rows of a width that is a multiple of 32" % FUSED_DECODE_MAX_ROWS)
-        return OperandRows(torch.empty((width // 32, -(-rows // 16), 64, 8), dtype=torch.bfloat16, device=device), rows, width)
+        return OperandRows(torch.empty((width // 32, row_tiles(rows), 64, 8), dtype=torch.bfloat16, device=device), rows, width)
 
     def to_rows(self) -> torch.Tensor:
         """The same values as an ordinary [M, K] tensor (for tests; not used by the engine)."""
@@ -307,6 +313,8 @@ def fused_decode_ok(rows: int, act_dtype, *tiled_weights, max_rows: Optional[int
         max_rows = default_fold_rows(sum(t.numel() for t in tiled_weights if t is not None))
     if rows > max_rows:
         return False
+    if rows > 64 and not (OPERAND_ORDER and all(t is not None and t.shape[0] % 32 == 0 for t in tiled_weights)):
+        return False                 # beyond 64 rows the products are built for hand-over in operand order only
     return all(t is not None and t.dtype == torch.bfloat16 and t.shape[0] % 16 == 0 and t.shape[1] % 128 == 0
                for t in tiled_weights)
 
@@ -349,7 +357,7 @@ def _gemm_decode(x, tiled: torch.Tensor, epi: int, n_out: int, out, resid, xw_ou
         _check(xs.dtype == torch.bfloat16 and xs.dim() == 2 and xs.shape[1] == K, "decode product: x must be bfloat16 [M, %d]" % K)
         M = xs.shape[0]
     out_tiled = isinstance(out, OperandRows) or isinstance(xw_out, OperandRows)
-    mp = -(-M // 16) * 16
+    mp = 16 * row_tiles(M)
     _check(ss is None or ss.shape[1] == mp, "decode product: the parts of the sums of squares must have %d columns" % mp)
     _check(ss_out is None or tuple(ss_out.shape) == (n_out // 16, mp), "decode product: the new parts must be [N / 16, %d]" % mp)
     for o in (out, xw_out):
@@ -409,7 +417,7 @@ def decode_linear_residual(x, tiled: torch.Tensor, resid: torch.Tensor, next_nor
            "decode_linear_residual: the stream must be float32 [M, %d]" % N)
     _check(next_norm_weight.dtype == torch.bfloat16 and next_norm_weight.shape == (N,),
            "decode_linear_residual: the next norm's weight must be bfloat16 [%d]" % N)
-    ss = torch.empty((N // 16, -(-M // 16) * 16), dtype=torch.float32, device=resid.device)
+    ss = torch.empty((N // 16, 16 * row_tiles(M)), dtype=torch.float32, device=resid.device)
     if _operand_order_ok(N):
         xw = OperandRows.empty(M, N, resid.device)
     else:
@@ -429,10 +437,10 @@ def embedding_scaled(ids: torch.Tensor, table: torch.Tensor, norm_weight: torch.
     out = torch.empty((T, H), dtype=torch.float32, device=table.device)
     tiled = _operand_order_ok(H)
     xw = OperandRows.empty(T, H, table.device) if tiled else torch.empty((T, H), dtype=torch.bfloat16, device=table.device)
-    ss = torch.empty((1, -(-T // 16) * 16), dtype=torch.float32, device=table.device)
+    ss = torch.empty((1, 16 * row_tiles(T)), dtype=torch.float32, device=table.device)
     hip().call("spy_embedding_sumsq", _ptr(out), _ptr(xw.data if tiled else xw), _ptr(ss), _ptr(table), _code(table, "embedding table"),
                _ptr(norm_weight), _ptr(ids), ctypes.c_int(T), ctypes.c_int(H), ctypes.c_int(V), ctypes.c_int(1 if tiled else 0),
-               _Hip.stream())
+               ctypes.c_int(row_tiles(T)), _Hip.stream())
     return out, ScaledInput(xw, ss, eps, norm)
 
 

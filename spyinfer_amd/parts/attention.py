@@ -139,6 +139,10 @@ class PagedAttention(Mixer):
 
     # ---- step ------------------------------------------------------------
     def can_fold(self, batch):
+        # (beyond 64 rows the products take their inputs in operand order only, which the attention hands over when every
+        # entry is a single token)
+        if batch.T > 64 and batch.max_q_len != 1:
+            return False
         return ops.fused_decode_ok(batch.T, batch.act_dtype, self.w_qkv_tiled, self.w_o_tiled, max_rows=self.fold_rows)
 
     def _attend(self, x, batch, cache, store, for_product=False):

@@ -366,9 +366,9 @@ def test_folded_decode_steps(tmp_path_factory):
     assert torch.allclose(mixed[1:3], ref4[[1, 4]], **TOL["bfloat16"])
 
 
-@pytest.mark.parametrize("requests", [19, 37, 57, 64, 70])
+@pytest.mark.parametrize("requests", [19, 37, 57, 64, 70, 100, 130])
 def test_folded_decode_steps_of_many_requests(tmp_path_factory, requests):
-    """Decode steps of 17 to 64 requests take the folded products with two to four row tiles (70 requests: the library's); their logits equal, up to
+    """Decode steps of 17 to 128 requests take the folded products with two to eight row tiles (130 requests: the library's); their logits equal, up to
     bfloat16 rounding, those of the same steps with the norms as kernels of their own, from graphs as well, and the last
     step's equal the plain implementation's.  Parts may be built to fold up to fewer rows (48 here): the embedding then still prepares the first norm's input, which the unfolded block does not use."""
     from spyinfer_amd.engine.batch import StepEntry
@@ -382,7 +382,7 @@ def test_folded_decode_steps_of_many_requests(tmp_path_factory, requests):
     ps = prompts(400, [3 + (7 * i) % 23 for i in range(requests)], 5)
     runs, calls = [], []
     real = ops.decode_linear_residual
-    assert ops.default_fold_rows(1 << 20) == 64
+    assert ops.default_fold_rows(1 << 20) == 128
     for folded, eager, fold_rows in ((True, True, None), (True, False, None), (False, True, None), (True, True, 48)):
         ops.FUSED_DECODE = folded
         for layer in model.layers:

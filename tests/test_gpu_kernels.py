@@ -217,6 +217,70 @@ def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
     assert torch.allclose(e.ss_parts[0, :len(ids)], (out * out).sum(1), rtol=1e-5) and (len(ids) % 16 == 0 or float(e.ss_parts[0, len(ids):].abs().max()) == 0.0)
 
 
+def _operand_rows(x):
+    """[M, K] bfloat16 -> ops.OperandRows with the same values (rows beyond M: zeros)."""
+    from spyinfer_amd.kernels import ops
+    M, K = x.shape
+    out = ops.OperandRows.empty(M, K, x.device)
+    mt = out.tiles
+    pad = torch.zeros((16 * mt, K), dtype=x.dtype, device=x.device)
+    pad[:M] = x
+    out.data.view(K // 32, mt, 4, 16, 8).copy_(pad.view(mt, 16, K // 32, 4, 8).permute(2, 0, 3, 1, 4))
+    assert torch.equal(out.to_rows(), x)
+    return out
+
+
+@pytest.mark.parametrize("M,H,I,NQKV,eps", [(80, 4096, 12288, 6144, 1e-6), (128, 4096, 12288, 6144, 1e-6), (65, 5120, 6400, 6160, 1e-5),
+                                            (100, 256, 384, 8208, 1e-6), (97, 128, 8320, 151936, 1e-6), (128, 4096, 36864, 64, 1e-6)])
+def test_decode_products_beyond_64_rows(M, H, I, NQKV, eps):
+    """65 to 128 rows (six or eight row tiles; inputs in operand order only): the chain residual product -> stored and
+    gated products of the normed rows -> residual product of the gated result, each against float64; widths with a
+    column tile per compute unit (K split over blocks), with many (blocks that walk), and small ones."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    resid0 = rnd((M, H), torch.float32, dev, 31, 1.5)
+    wn1 = (1 + 0.1 * rnd((H,), torch.float32, dev, 32)).bfloat16()
+    wn2 = (1 + 0.1 * rnd((H,), torch.float32, dev, 33)).bfloat16()
+    w_in = rnd((H, I), torch.bfloat16, dev, 34, 0.05)
+    w_qkv = rnd((NQKV, H), torch.bfloat16, dev, 35, 0.05)
+    w_gu = rnd((2 * I, H), torch.bfloat16, dev, 36, 0.05)
+    w_dn = rnd((H, I), torch.bfloat16, dev, 40, 0.05)
+    a = rnd((M, I), torch.bfloat16, dev, 37)
+
+    def norm64(h, w):
+        h = h.double()
+        return h * torch.rsqrt((h * h).mean(1, keepdim=True) + eps) * w.double()
+
+    assert ops.row_tiles(M) == (6 if M <= 96 else 8)
+    resid = resid0.clone()
+    si = ops.decode_linear_residual(_operand_rows(a), ops.tile_weight(w_in), resid, wn1, eps)
+    close(resid, resid0.double() + a.double() @ w_in.double().t(), torch.float32, scale=4.0, what="stream after the residual epilogue")
+    assert isinstance(si.xw, ops.OperandRows) and torch.equal(si.xw.to_rows(), (resid * wn1.float()).bfloat16())
+    ss = si.ss_parts.sum(0)
+    assert ss.shape[0] == 16 * ops.row_tiles(M) and torch.allclose(ss[:M], (resid * resid).sum(1), rtol=1e-5) and (M == ss.shape[0] or float(ss[M:].abs().max()) == 0.0)
+    for od in (torch.bfloat16, torch.float32):
+        close(ops.decode_linear(si, ops.tile_weight(w_qkv), od), norm64(resid, wn1) @ w_qkv.double().t(), torch.bfloat16, scale=2.0,
+              what="scaled decode_linear")
+    y = norm64(resid, wn1) @ w_gu.double().t()
+    gated = y[:, :I] / (1 + torch.exp(-y[:, :I])) * y[:, I:]
+    close(ops.decode_linear_swiglu(si, ops.tile_weight(w_gu)), gated, torch.bfloat16, scale=2.0, what="gated product, row-major result")
+    g = ops.decode_linear_swiglu(si, ops.tile_weight(w_gu), for_product=True)
+    assert isinstance(g, ops.OperandRows)
+    close(g.to_rows(), gated, torch.bfloat16, scale=2.0, what="gated product, result in operand order")
+    rd = resid.clone()
+    sd = ops.decode_linear_residual(g, ops.tile_weight(w_dn), rd, wn2, eps)
+    close(rd, resid.double() + g.to_rows().double() @ w_dn.double().t(), torch.float32, scale=4.0, what="stream after the down product")
+    assert torch.equal(sd.xw.to_rows(), (rd * wn2.float()).bfloat16()) and torch.allclose(sd.ss_parts.sum(0)[:M], (rd * rd).sum(1), rtol=1e-5)
+    # what is not built beyond 64 rows is refused, not computed wrongly: a row-major input
+    with pytest.raises(ops.KernelError, match="operand order"):
+        ops.decode_linear_residual(a, ops.tile_weight(w_in), resid.clone(), wn1, eps)
+    table = rnd((50, H), torch.bfloat16, dev, 39)
+    ids = torch.randint(0, 50, (M,), generator=torch.Generator().manual_seed(41)).int().to(dev)
+    out, e = ops.embedding_scaled(ids, table, wn1, eps)
+    assert torch.equal(out, ops.embedding(ids, table)) and torch.equal(e.xw.to_rows(), (out * wn1.float()).bfloat16())
+    assert torch.allclose(e.ss_parts[0, :M], (out * out).sum(1), rtol=1e-5) and (M == e.ss_parts.shape[1] or float(e.ss_parts[0, M:].abs().max()) == 0.0)
+
+
 def test_products_with_k_split_over_blocks_repeat_exactly():
     """The product whose blocks hand their partial sums to the last block of a column group (long K, about a column
     tile per compute unit): 40 calls in a row without a wait between them, on changing inputs, give bit for bit what
@@ -588,6 +652,7 @@ FUSED_CASES = [
     (8, 8, 256, 32, [300, 63, 64], 50, True, False),
     (16, 1, 64, 8, [99, 7], None, True, True),
     (6, 2, 128, 16, [33], 8, False, False),
+    (8, 2, 128, 16, [(37 * i) % 700 for i in range(100)], None, True, True),      # 100 single tokens: seven row tiles of output
 ]
 
 

@@ -130,3 +130,49 @@ def test_steps_at_real_widths(widths, sharp):
         assert folded[0] == 8 * 2 * 2, "the bfloat16 steps of single tokens ran %d folded products" % folded[0]
     finally:
         ops.decode_linear_residual = real
+
+
+def test_decode_steps_of_65_to_128_requests_at_real_widths():
+    """Decode steps of 100 and of 70 requests (eight and six row tiles of the folded products, which take their inputs in
+    operand order only there) at the 8B widths: bfloat16 against float32 on the same weights, float32 against the plain
+    implementation, and the folded products really ran."""
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.kernels import ops
+    from tests.plain.qwen3_plain import PlainQwen3
+    dev = require_gpu()
+    R = 100
+    (r16, r32), raw, w16 = _runners(dev, R, 400, WIDTHS[0])
+    plain = PlainQwen3(None, config=raw, weights=w16)
+    g = torch.Generator().manual_seed(11)
+    prompts = [torch.randint(0, RAW["vocab_size"], (3 + (7 * i) % 40,), generator=g).tolist() for i in range(R)]
+    seqs = [list(p) for p in prompts]
+    folded = [0]
+    real = ops.decode_linear_residual
+    ops.decode_linear_residual = lambda *a, **k: (folded.__setitem__(0, folded[0] + 1), real(*a, **k))[1]
+
+    def both(entries_of):
+        outs = []
+        for runner, cs in zip((r16, r32), caches):
+            entries = entries_of(cs)
+            for e in entries:
+                runner.manager.reserve(e.cache, len(e.tokens))
+            outs.append(runner.step(entries))
+        return outs
+
+    try:
+        caches = [[runner.manager.admit(i) for i in range(R)] for runner in (r16, r32)]
+        outs = both(lambda cs: [StepEntry(c, p, [len(p) - 1]) for c, p in zip(cs, prompts)])
+        _close(outs[0], outs[1], "prompts")
+        assert folded[0] == 0
+        for live, steps in ((R, 2), (70, 2)):
+            for s in range(steps):
+                toks = torch.randint(0, RAW["vocab_size"], (live,), generator=g).tolist()
+                for q, t in zip(seqs, toks):
+                    q.append(t)
+                outs = both(lambda cs: [StepEntry(c, [t], [0]) for c, t in zip(cs[:live], toks)])
+                _close(outs[0], outs[1], "%d requests, step %d" % (live, s))
+            for i in (0, live // 2, live - 1):
+                _plain_close(outs[1][i], plain.forward(seqs[i])[-1], "%d requests, request %d" % (live, i))
+        assert folded[0] == 4 * 2 * 2, "the bfloat16 steps of single tokens ran %d folded products" % folded[0]
+    finally:
+        ops.decode_linear_residual = real
