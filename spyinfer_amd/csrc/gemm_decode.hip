@@ -498,7 +498,10 @@ static bool gd_launch_wide(const GdArgs& a) {
     if constexpr (EPI == EPI_RESID || !SCALED || !XT) return false;
     else {
         constexpr int GATES = EPI == EPI_GATED ? 2 : 1;
-        constexpr int GW = MT > 4 ? 4 : 8;               // beyond four row tiles: four waves with a SIMD's registers each
+#ifndef GD_GW4_FROM
+#define GD_GW4_FROM 5        // (four waves from three row tiles on, measured at 40 to 64 rows: gate/up 41-43 us against 35-37)
+#endif
+        constexpr int GW = MT >= GD_GW4_FROM ? 4 : 8;    // beyond four row tiles: four waves with a SIMD's registers each
         // a group's accumulators (GATES * CT * MT tiles of four registers) leave room for its operands up to 24 tiles
         // (48 for a wave that has a SIMD to itself)
         constexpr int ROOM = GW == 8 ? 24 : 48;
