@@ -74,6 +74,9 @@ struct GdArgs {
 // Compute units of the current device (asked for once per device).
 int gd_compute_units();
 
+// The product whose blocks walk runs of column tiles (gemm_decode_wide.hip): true if it has launched the call.
+bool gd_wide_try(const GdArgs& a, int epi, bool scaled, bool f32_out);
+
 // The product with K split over blocks (gemm_decode_splitk.hip): true if it has launched the call.
 bool gd_splitk_try(const GdArgs& a, int epi, bool scaled, bool f32_out);
 long long gd_splitk_workspace_bytes();
