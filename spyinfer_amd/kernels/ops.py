@@ -164,10 +164,9 @@ FUSED_DECODE_MAX_ROWS = 128
 def default_fold_rows(weight_elements: int) -> int:
     """Most rows of a step for which a part with ``weight_elements`` matrix elements should run its products with the
     norms and residual sums folded in (above: the library product with norm kernels of their own), where the part's
-    builder names no limit.  Measured on MI355X: such products beat the library's by 16 % at 32 rows and are level with
-    it at 64 rows, where the step still gains by the norm and SwiGLU kernels it does not run: 1.5 % at the Qwen3-8B
-    shape, 1.7 % at the 32B shape (5.5 % at 56 rows) since the gated product walks runs of column tiles.  So: as many
-    rows as the decode products take, whatever the size."""
+    builder names no limit.  Measured on MI355X at the Qwen3-8B shape: a step of 32 / 64 requests takes 4.4 / 5.8 ms with
+    them against 5.9 / 7.4 with the library's products, one of 65 / 96 / 128 requests 7.0 / 7.9 / 9.5 against 7.9 / 9.0
+    / 10.3.  So: as many rows as the decode products take, whatever the size."""
     return FUSED_DECODE_MAX_ROWS
 
 
@@ -395,7 +394,7 @@ def decode_linear(x, tiled: torch.Tensor, out_dtype: torch.dtype = torch.bfloat1
 
 
 def decode_linear_swiglu(x, tiled_gate_up: torch.Tensor, for_product: bool = False):
-    """silu(x . Wgate^T) * (x . Wup^T) for at most 16 rows; ``tiled_gate_up [2 I, K]`` = tiles of [Wgate | Wup].
+    """silu(x . Wgate^T) * (x . Wup^T) for at most 128 rows (beyond 64: a normed input in operand order only); ``tiled_gate_up [2 I, K]`` = tiles of [Wgate | Wup].
     ``for_product``: the result goes into another decode product only, and may come as OperandRows."""
     _check(tiled_gate_up.shape[0] % 32 == 0, "decode_linear_swiglu: [2 I, K] with I a multiple of 16 expected")
     I = tiled_gate_up.shape[0] // 2
@@ -409,7 +408,7 @@ def decode_linear_swiglu(x, tiled_gate_up: torch.Tensor, for_product: bool = Fal
 
 def decode_linear_residual(x, tiled: torch.Tensor, resid: torch.Tensor, next_norm_weight: torch.Tensor,
                            eps: float, norm=None) -> ScaledInput:
-    """resid += x . w^T (float32, in place) for at most 16 rows -> the ScaledInput of the norm that reads the
+    """resid += x . w^T (float32, in place) for at most 128 rows (beyond 64: x in operand order only) -> the ScaledInput of the norm that reads the
     stream next: bfloat16(resid * next_norm_weight) and the parts [N / 16, 16] of the new rows' sums of squares."""
     N = tiled.shape[0]
     M = _rows_of(x)
