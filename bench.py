@@ -30,6 +30,9 @@ MODEL_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_a
                 bos_token_id=151643, eos_token_id=151645)
 # the larger shapes; the default stays the 8B shape
 SHAPES = {
+    # the size of model that the reference's own run script names (run.sh:2): 28 narrow layers, where a step is many short kernels
+    "0.6b": ("Qwen3-0.6B shape", dict(MODEL_8B, num_hidden_layers=28, hidden_size=1024, num_attention_heads=16, intermediate_size=3072,
+                                      tie_word_embeddings=True)),
     "8b": ("Qwen3-8B shape", MODEL_8B),
     "14b": ("Qwen3-14B shape", dict(MODEL_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)),
     "32b": ("Qwen3-32B shape", dict(MODEL_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)),
