@@ -52,6 +52,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,32,64", help="further decode batch sizes to report (empty: none)")
     ap.add_argument("--enforce-eager", action="store_true")
+    ap.add_argument("--weight-copies", default="both", choices=["both", "tiled"], help="EngineConfig.weight_copies")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes of the model")
     ap.add_argument("--serve", type=int, default=0, metavar="N",
@@ -67,6 +68,7 @@ def main() -> int:
     from spyinfer_amd.config.registry import architecture_of
     from spyinfer_amd.engine.batch import StepEntry
     from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.engine.runner import bind_weights
     from spyinfer_amd.kernels import ops
     from spyinfer_amd.sampling import SamplingParams
     from spyinfer_amd.weights.random_init import random_tensors_on_device
@@ -83,7 +85,7 @@ def main() -> int:
     model = arch.build(cfg)
     run_dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
     weights = random_tensors_on_device(model.weight_specs(), args.seed, run_dtype, dev)
-    model.bind(weights, dev)
+    bind_weights(model, weights, dev, args.weight_copies)
     del weights
     torch.cuda.empty_cache()
 
@@ -94,7 +96,8 @@ def main() -> int:
     eng = LLMEngine.__new__(LLMEngine)
     eng._init_with_model(model, dev, dtype=args.dtype, max_model_len=args.context, kvcache_block_size=page,
                          num_kvcache_blocks=max(pages_per_req * max_batch, -(-args.prefill_tokens // page)) + 8, max_num_seqs=max_batch,
-                         max_num_batched_tokens=max(16384, args.prefill_tokens), enforce_eager=args.enforce_eager, seed=args.seed)
+                         max_num_batched_tokens=max(16384, args.prefill_tokens), enforce_eager=args.enforce_eager, seed=args.seed,
+                         weight_copies=args.weight_copies)
     g = torch.Generator().manual_seed(args.seed)
 
     def prompts(n, length):

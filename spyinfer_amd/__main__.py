@@ -32,6 +32,8 @@ def main(argv=None) -> int:
     ap.add_argument("--enforce-eager", action="store_true")
     ap.add_argument("--kvcache-block-size", type=int, default=16)
     ap.add_argument("--num-kvcache-blocks", type=int, default=None)
+    ap.add_argument("--weight-copies", default="both", choices=["both", "tiled"],
+                    help="tiled: matrices are kept in tiles only (half the weights' memory, prompts a sixth slower)")
     ap.add_argument("--temperature", type=float, default=0.0)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--max-new-tokens", type=int, default=None)
@@ -66,7 +68,8 @@ def main(argv=None) -> int:
                        prefill_chunk=args.prefill_chunk, max_num_seqs=args.max_num_seqs, max_model_len=args.max_model_len,
                        keep_finished_cache=False,
                        gpu_memory_utilization=args.gpu_memory_utilization, enforce_eager=args.enforce_eager,
-                       kvcache_block_size=args.kvcache_block_size, num_kvcache_blocks=args.num_kvcache_blocks, seed=args.seed)
+                       kvcache_block_size=args.kvcache_block_size, num_kvcache_blocks=args.num_kvcache_blocks, seed=args.seed,
+                       weight_copies=args.weight_copies)
     params = SamplingParams(temperature=args.temperature, max_new_tokens=args.max_new_tokens, ignore_eos=args.ignore_eos)
 
     def stream(rid):

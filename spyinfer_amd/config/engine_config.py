@@ -35,6 +35,11 @@ class EngineConfig:
     #: True: a finished request keeps its pages and slot for a further turn (append_to_request), as the reference's do
     #: until they are removed (llm_engine.cpp:40-73); they are the first to go when pages or slots are short
     keep_finished_cache: bool = False
+    #: "both": every bfloat16 matrix is held as rows (for the library's products of many rows) and in tiles (for the
+    #: products of few rows).  "tiled": in tiles only, which halves the weights' memory; a step of more than 64 rows
+    #: then restores each matrix's rows into a scratch tensor ahead of its product (a prompt portion of 2048 tokens
+    #: takes about a sixth longer).  Matrices without a tiled form (float32, odd shapes) keep their rows either way.
+    weight_copies: str = "both"
 
     def validate(self) -> None:
         if self.dtype not in ("bfloat16", "float32"):
@@ -44,5 +49,7 @@ class EngineConfig:
                 raise ValueError("%s must be positive" % name)
         if self.num_kvcache_blocks is not None and self.num_kvcache_blocks <= 0:
             raise ValueError("num_kvcache_blocks must be positive")
+        if self.weight_copies not in ("both", "tiled"):
+            raise ValueError("weight_copies must be 'both' or 'tiled', got %r" % (self.weight_copies,))
         if not (0.0 < self.gpu_memory_utilization <= 1.0):
             raise ValueError("gpu_memory_utilization must be in (0, 1]")

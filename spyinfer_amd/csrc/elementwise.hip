@@ -300,6 +300,41 @@ extern "C" int spy_swiglu(const void* in, void* out, int dtype, int T, int I, hi
 }
 
 // ---------------------------------------------------------------------------------------------
+// A matrix [N, K] back from the order the decode products read it ([K/128 chunks][N/16 tiles][4 steps][g = 4][r = 16][8])
+// into rows, for the library's products of many rows when only that copy of the matrix is kept.  A block moves
+// UNTILE_TILES tiles of 16 rows x 128 columns (4 KiB each, one piece of the source); thread (r, step, g) of a tile
+// writes 16 bytes of row r, so that 16 neighbouring lanes write 256 bytes of one row.
+#define UNTILE_TILES 4
+__global__ __launch_bounds__(256) void untile_weight_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ tiled, int N, int K,
+                                                            size_t n_tiles) {
+    typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+    const int r = threadIdx.x >> 4, sg = threadIdx.x & 15;
+    const size_t col_tiles = (size_t)(N / 16);
+    for (size_t t = (size_t)blockIdx.x * UNTILE_TILES; t < n_tiles; t += (size_t)gridDim.x * UNTILE_TILES) {
+        u32x4_t v[UNTILE_TILES];
+#pragma unroll
+        for (int i = 0; i < UNTILE_TILES; ++i)
+            if (t + i < n_tiles) v[i] = *reinterpret_cast<const u32x4_t*>(tiled + ((t + i) * 256 + sg * 16 + r) * 8);
+#pragma unroll
+        for (int i = 0; i < UNTILE_TILES; ++i) {
+            if (t + i < n_tiles) {
+                const size_t chunk = (t + i) / col_tiles, tile = (t + i) % col_tiles;
+                *reinterpret_cast<u32x4_t*>(out + (tile * 16 + r) * (size_t)K + chunk * 128 + sg * 8) = v[i];
+            }
+        }
+    }
+}
+
+extern "C" int spy_untile_weight(void* out, const void* tiled, int N, int K, hipStream_t st) {
+    SPY_REQUIRE(N > 0 && K > 0 && N % 16 == 0 && K % 128 == 0, "spy_untile_weight: [%d, %d] is not made of tiles of 16 x 128", N, K);
+    const size_t n_tiles = (size_t)(N / 16) * (size_t)(K / 128);
+    const size_t want = (n_tiles + UNTILE_TILES - 1) / UNTILE_TILES;
+    untile_weight_kernel<<<(unsigned)(want > 65536 ? 65536 : want), 256, 0, st>>>((bf16_t*)out, (const bf16_t*)tiled, N, K, n_tiles);
+    SPY_CHECK_LAUNCH("spy_untile_weight");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
 // One wave per (token, head of q|k|v), QK_WAVES heads per block.  q, k: optional RMS norm over the head,
 // then half-split rotation of the first `rot` dims: y[j] = x[j] c - x[j+rot/2] s; y[j+rot/2] = x[j] s + x[j+rot/2] c.
 // A lane holds both members of its pairs, so the rotation needs no exchange between lanes.

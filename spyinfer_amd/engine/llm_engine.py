@@ -67,7 +67,7 @@ class LLMEngine:
             raise TypeError("unknown engine option(s): %s; known: %s" % (", ".join(bad), ", ".join(sorted(known))))
         config = EngineConfig(model=model_path, **params)
         config.validate()
-        self._init_with_model(load_model(model_path, config.dtype, torch.device(device)), device, **params)
+        self._init_with_model(load_model(model_path, config.dtype, torch.device(device), config.weight_copies), device, **params)
         self.config.model = model_path
 
     def _init_with_model(self, model, device, **params) -> None:

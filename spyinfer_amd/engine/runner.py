@@ -33,12 +33,23 @@ def resolve_dtype(name) -> torch.dtype:
     return DTYPES[name]
 
 
-def load_model(folder: str, dtype, device) -> DecoderModel:
+def bind_weights(model: DecoderModel, weights, device, weight_copies: str = "both") -> None:
+    """``model.bind`` with the engine's choice of the forms in which matrices are kept (EngineConfig.weight_copies)."""
+    from ..kernels import ops
+    before = ops.ROW_MAJOR_WEIGHTS
+    ops.ROW_MAJOR_WEIGHTS = weight_copies != "tiled"
+    try:
+        model.bind(weights, device)
+    finally:
+        ops.ROW_MAJOR_WEIGHTS = before
+
+
+def load_model(folder: str, dtype, device, weight_copies: str = "both") -> DecoderModel:
     """config.json -> architecture -> model of parts, weights bound by name."""
     arch, cfg = load_model_config(folder)
     model = arch.build(cfg)
     weights = load_weights(folder, model.weight_specs(), resolve_dtype(dtype), device)
-    model.bind(weights, device)
+    bind_weights(model, weights, device, weight_copies)
     return model
 
 

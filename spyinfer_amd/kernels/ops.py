@@ -65,7 +65,7 @@ class _Hip:
         self.lib.spy_last_error.restype = ctypes.c_char_p
         for name in ("spy_embedding", "spy_add_rmsnorm", "spy_rmsnorm", "spy_gemm", "spy_qknorm_rope_store",
                      "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_prefill",
-                     "spy_attention_prefill_workspace", "spy_swiglu",
+                     "spy_attention_prefill_workspace", "spy_swiglu", "spy_untile_weight",
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
                      "spy_gemm_decode", "spy_gemm_decode_workspace", "spy_embedding_sumsq", "spy_sample_static"):
             if not hasattr(self.lib, name):
@@ -182,6 +182,70 @@ def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
     return w.view(N // 16, 16, K // 128, 4, 4, 8).permute(2, 0, 3, 4, 1, 5).contiguous().view(N, K)
 
 
+#: False while a model's weights are bound: a bfloat16 matrix that has a tiled copy is kept in that form only
+#: (``weight_forms``), which halves the weights' device memory; a product of many rows then restores the rows into a
+#: scratch tensor first (``TiledOnly.rows``), which costs a sixth more time in a prompt portion of 2048 tokens.
+ROW_MAJOR_WEIGHTS = True
+#: most rows that a product takes straight from the tiled copy when the rows of the matrix are not kept
+TILED_ONLY_DIRECT_ROWS = 64
+_untile_scratch = {}          # device -> the tensor that restored rows go to outside graph capture
+
+
+def untile_weight(tiled: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The matrix [N, K] whose ``tile_weight`` is ``tiled``, into ``out`` if one is brought."""
+    _dev(tiled, out)
+    _check(tiled.dtype == torch.bfloat16 and tiled.dim() == 2, "untile_weight: a bfloat16 matrix from tile_weight expected")
+    N, K = tiled.shape
+    out = _result(out, N, K, torch.bfloat16, tiled.device)
+    hip().call("spy_untile_weight", _ptr(out), _ptr(tiled), ctypes.c_int(N), ctypes.c_int(K), _Hip.stream())
+    return out
+
+
+class TiledOnly:
+    """Stands where a product expects the matrix [N, K] of which only the tiled copy is kept: it has the matrix's
+    shape, dtype and device, and ``rows()`` restores the matrix for the library's product.  Outside graph capture the
+    rows go to one scratch tensor per device, which every matrix uses in turn and which holds them until the next
+    call (the steps run on one stream); inside a capture they go to a tensor of the graph's own pool."""
+    __slots__ = ("tiled",)
+
+    shape = property(lambda self: self.tiled.shape)
+    dtype = property(lambda self: self.tiled.dtype)
+    device = property(lambda self: self.tiled.device)
+    is_cuda = property(lambda self: self.tiled.is_cuda)
+
+    def dim(self) -> int:
+        return 2
+
+    def is_contiguous(self) -> bool:
+        return True
+
+    def __init__(self, tiled: torch.Tensor):
+        self.tiled = tiled
+        self._scratch()            # made now, while the weights are bound, so that the memory left for the cache counts it
+
+    def _scratch(self) -> torch.Tensor:
+        t = self.tiled
+        buf = _untile_scratch.get(t.device)
+        if buf is None or buf.numel() < t.numel():
+            buf = _untile_scratch[t.device] = torch.empty((t.numel(),), dtype=torch.bfloat16, device=t.device)
+        return buf[:t.numel()].view(t.shape)
+
+    def rows(self) -> torch.Tensor:
+        if torch.cuda.is_current_stream_capturing():
+            return untile_weight(self.tiled)
+        return untile_weight(self.tiled, self._scratch())
+
+
+def weight_forms(w: torch.Tensor, keep_rows: bool = False):
+    """(matrix, tiled copy or None) as a part keeps them for ``linear``: both forms, or, with ROW_MAJOR_WEIGHTS off and
+    a tiled copy at hand, the tiled copy alone (the first member is then a TiledOnly).  ``keep_rows``: the rows are
+    needed for something else than products (an embedding table) and stay."""
+    tiled = tile_weight(w)
+    if tiled is not None and not ROW_MAJOR_WEIGHTS and not keep_rows:
+        return TiledOnly(tiled), tiled
+    return w, tiled
+
+
 def _result(out: Optional[torch.Tensor], M: int, N: int, dtype: torch.dtype, device) -> torch.Tensor:
     """The [M, N] result tensor of a product: ``out`` if the caller brought one (checked), else a new one."""
     if out is None:
@@ -210,9 +274,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     if M == 0:
         return out
     all_bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-    if all_bf16 and tiled is not None and M <= SKINNY_MAX_ROWS:
+    if isinstance(w, TiledOnly):
+        _check(x.dtype == torch.bfloat16, "linear: a matrix kept in tiles only takes bfloat16 rows")
+        tiled = w.tiled
+    if all_bf16 and tiled is not None and M <= (TILED_ONLY_DIRECT_ROWS if isinstance(w, TiledOnly) else SKINNY_MAX_ROWS):
         _check(tiled.shape == w.shape, "linear: the tiled copy does not fit the matrix")
         return decode_linear(x, tiled, out_dtype, out)
+    if isinstance(w, TiledOnly):
+        w = w.rows()
     global _LIBRARY_F32_OUT
     if all_bf16 and out_dtype == torch.float32 and M > SKINNY_MAX_ROWS and _LIBRARY_F32_OUT:
         try:

@@ -112,8 +112,8 @@ class PagedAttention(Mixer):
         # one product for q, k and v: rows [q heads | k heads | v heads]
         self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
         del q, k, v
-        self.w_o = weights[prefix + ".o_proj.weight"]
-        self.w_qkv_tiled, self.w_o_tiled = ops.tile_weight(self.w_qkv), ops.tile_weight(self.w_o)
+        self.w_qkv, self.w_qkv_tiled = ops.weight_forms(self.w_qkv)
+        self.w_o, self.w_o_tiled = ops.weight_forms(weights.pop(prefix + ".o_proj.weight"))
         if self.qk_norm_eps is not None:
             self.q_norm, self.k_norm = weights[prefix + ".q_norm.weight"], weights[prefix + ".k_norm.weight"]
             if self.q_norm.dtype != self.k_norm.dtype:

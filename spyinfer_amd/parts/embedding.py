@@ -36,7 +36,7 @@ class LMHead(Part):
     def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding = None, fold_rows: int = 32):
         """``fold_rows``: most rows for which the head runs as a decode product with the final norm folded in.  Above,
         the library's product after a norm kernel is faster for a large matrix (measured with 151936 x 4096: 229 / 253 us
-        at 24 / 32 rows against the library's 264 / 269, but 323 against 260 at 48)."""
+        at 24 / 32 rows against the library's 264 / 269, but 266 / 283 against 261 / 269 at 48 / 64)."""
         self.vocab_size, self.hidden_size, self.tied_to = vocab_size, hidden_size, tied_to
         self.fold_rows = fold_rows
         self.weight = None
@@ -48,11 +48,16 @@ class LMHead(Part):
         return [WeightSpec(prefix + ".weight", (self.vocab_size, self.hidden_size))]
 
     def bind(self, prefix, weights):
-        self.weight = self.tied_to.weight if self.tied_to is not None else weights[prefix + ".weight"]
-        self.weight_tiled = ops.tile_weight(self.weight)
+        if self.tied_to is not None:
+            self.weight, self.weight_tiled = ops.weight_forms(self.tied_to.weight, keep_rows=True)   # the table's rows are looked up
+        else:
+            self.weight, self.weight_tiled = ops.weight_forms(weights.pop(prefix + ".weight"))
 
     def can_fold(self, batch):
-        return ops.fused_decode_ok(batch.T, batch.act_dtype, self.weight_tiled, max_rows=self.fold_rows)
+        # without the matrix's rows there is no library product to prefer: the folded product stands as far as it is built
+        # for a plain input's rows (measured with 151936 x 4096 at 64 rows: 283 us against the library's 269 and a norm kernel)
+        rows = max(self.fold_rows, ops.TILED_ONLY_DIRECT_ROWS) if isinstance(self.weight, ops.TiledOnly) else self.fold_rows
+        return ops.fused_decode_ok(batch.T, batch.act_dtype, self.weight_tiled, max_rows=rows)
 
     def logits(self, resid, pending, final_norm, batch, out=None):
         """The end of a forward pass: ``final_norm`` of the stream (``pending`` as a block leaves it: None, an addend

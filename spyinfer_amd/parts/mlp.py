@@ -32,10 +32,10 @@ class GatedMLP(FeedForward):
             g, u = g.float(), u.float()
         self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
         del g, u
-        self.w_down = weights[prefix + ".down_proj.weight"]
         # tiles 0 .. I/16 - 1 of the tiled copy are gate rows, the rest up rows: what the fused SwiGLU kernel expects
-        self.w_gate_up_tiled = ops.tile_weight(self.w_gate_up) if self.intermediate_size % 16 == 0 else None
-        self.w_down_tiled = ops.tile_weight(self.w_down)
+        if self.intermediate_size % 16 == 0:
+            self.w_gate_up, self.w_gate_up_tiled = ops.weight_forms(self.w_gate_up)
+        self.w_down, self.w_down_tiled = ops.weight_forms(weights.pop(prefix + ".down_proj.weight"))
 
     def can_fold(self, batch):
         return ops.fused_decode_ok(batch.T, batch.act_dtype, self.w_gate_up_tiled, self.w_down_tiled, max_rows=self.fold_rows)

@@ -77,3 +77,7 @@ def test_engine_config():
         EngineConfig(dtype="float16").validate()
     with pytest.raises(ValueError):
         EngineConfig(kvcache_block_size=0).validate()
+    assert c.weight_copies == "both"
+    EngineConfig(weight_copies="tiled").validate()
+    with pytest.raises(ValueError):
+        EngineConfig(weight_copies="rows").validate()

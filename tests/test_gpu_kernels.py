@@ -111,6 +111,61 @@ def test_linear_with_tiled_weights(M, N, K):
     assert ops.tile_weight(rnd((24, 128), torch.bfloat16, dev, 1)) is None and ops.tile_weight(rnd((32, 96), torch.bfloat16, dev, 1)) is None
 
 
+@pytest.mark.parametrize("N,K", [(16, 128), (48, 384), (4112, 1280), (24576, 4096)])
+def test_untile_weight_restores_the_rows(N, K):
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    w = rnd((N, K), torch.bfloat16, dev, 23, 0.05)
+    assert torch.equal(ops.untile_weight(ops.tile_weight(w)), w)
+
+
+def test_linear_with_a_matrix_kept_in_tiles_only(monkeypatch):
+    """``weight_forms`` with the rows switched off keeps the tiled copy alone; ``linear`` then gives, for any number of
+    rows, what it gives with both forms: the same kernel on the same values up to 16 rows and beyond 64 (there the
+    library, on the restored rows), the decode kernel instead of the library between; also inside a captured graph,
+    where the restored rows may not go to the scratch tensor that calls outside share."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    N, K = 1040, 640
+    w = rnd((N, K), torch.bfloat16, dev, 31, 0.05)
+    both = ops.weight_forms(w)
+    assert both[0] is w and both[1] is not None
+    monkeypatch.setattr(ops, "ROW_MAJOR_WEIGHTS", False)
+    only, tiled = ops.weight_forms(w)
+    assert isinstance(only, ops.TiledOnly) and only.shape == w.shape and torch.equal(tiled, both[1])
+    kept, _ = ops.weight_forms(w, keep_rows=True)
+    assert kept is w
+    odd = rnd((24, 128), torch.bfloat16, dev, 1)                # no tiled form: the rows stay
+    assert ops.weight_forms(odd)[0] is odd and ops.weight_forms(odd)[1] is None
+    small = ops.weight_forms(rnd((32, 128), torch.bfloat16, dev, 2))[0]
+    for M in (1, 16, 17, 40, 64, 65, 300):
+        x = rnd((M, K), torch.bfloat16, dev, 32 + M)
+        for od in (torch.bfloat16, torch.float32):
+            a, b = ops.linear(x, only, od, tiled=tiled), ops.linear(x, w, od, tiled=both[1])
+            close(a, x.double() @ w.double().t(), torch.bfloat16, scale=1.0, what="linear, tiles only, %d rows" % M)
+            if M <= 16 or M > 64:
+                assert torch.equal(a, b), "%d rows: another result than with both forms" % M
+        ops.linear(x[:, :128].contiguous(), small)                # a smaller matrix takes its turn in the scratch tensor
+    I = N // 2
+    x = rnd((200, K), torch.bfloat16, dev, 50)
+    assert torch.equal(ops.linear_swiglu(x, only, tiled), ops.linear_swiglu(x, w, both[1]))
+    # captured: replays with other inputs, the scratch tensor used by calls in between
+    xs = torch.zeros((200, K), dtype=torch.bfloat16, device=dev)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        ops.linear(xs, only)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = ops.linear(xs, only)
+    for seed in (60, 61, 62):
+        xs.copy_(rnd((200, K), torch.bfloat16, dev, seed))
+        ops.linear(xs[:, :128].contiguous(), small)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, ops.linear(xs, w)), "replay with input %d" % seed
+
+
 @pytest.mark.parametrize("M,H,I,NQKV,eps", [(1, 128, 256, 192, 1e-6), (7, 256, 384, 400, 1e-5), (16, 4096, 1024, 6144, 1e-6),
                                             (3, 5120, 128, 64, 1e-2), (17, 256, 128, 96, 1e-6), (32, 1024, 2048, 320, 1e-5),
                                             (41, 128, 384, 400, 1e-6), (64, 256, 128, 6144, 1e-6), (57, 128, 384, 6176, 1e-5),

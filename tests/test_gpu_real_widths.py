@@ -25,9 +25,9 @@ RAW = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_act="s
 WIDTHS = [(4096, 32, 8, 128, 12288), (5120, 40, 8, 128, 17408), (2048, 32, 4, 64, 6144)]
 
 
-def _runners(dev, requests, pages, widths, sharp=False):
+def _runners(dev, requests, pages, widths, sharp=False, dtypes=("bfloat16", "float32"), weight_copies=("both", "both")):
     from spyinfer_amd.config.registry import architecture_of
-    from spyinfer_amd.engine.runner import ModelRunner
+    from spyinfer_amd.engine.runner import ModelRunner, bind_weights
     from spyinfer_amd.weights.random_init import random_tensors_on_device
     raw = dict(RAW, hidden_size=widths[0], num_attention_heads=widths[1], num_key_value_heads=widths[2], head_dim=widths[3],
                intermediate_size=widths[4])
@@ -35,7 +35,7 @@ def _runners(dev, requests, pages, widths, sharp=False):
     cfg = arch.config_cls.from_dict(raw)
     out = []
     w16 = None
-    for dtype in ("bfloat16", "float32"):
+    for dtype, copies in zip(dtypes, weight_copies):
         model = arch.build(cfg)
         if w16 is None:
             w16 = random_tensors_on_device(model.weight_specs(), 5, torch.bfloat16, dev, norm_std=0.05)
@@ -44,7 +44,7 @@ def _runners(dev, requests, pages, widths, sharp=False):
                     if k.endswith("q_norm.weight") or k.endswith("k_norm.weight"):
                         w16[k] = (w16[k].float() * 2.0).to(torch.bfloat16)
         weights = w16 if dtype == "bfloat16" else {k: (v.float() if v.dtype == torch.bfloat16 else v) for k, v in w16.items()}
-        model.bind(dict(weights), dev)       # a copy: parts take the matrices they fuse out of the dictionary
+        bind_weights(model, dict(weights), dev, copies)       # a copy: parts take matrices out of the dictionary
         out.append(ModelRunner(model, dtype, dev, 16, pages, requests, enforce_eager=True, max_model_len=1024))
     return out, raw, w16
 
@@ -176,3 +176,44 @@ def test_decode_steps_of_65_to_128_requests_at_real_widths():
         assert folded[0] == 4 * 2 * 2, "the bfloat16 steps of single tokens ran %d folded products" % folded[0]
     finally:
         ops.decode_linear_residual = real
+
+
+def test_steps_with_matrices_kept_in_tiles_only():
+    """EngineConfig.weight_copies = "tiled" at the 8B widths, in bfloat16 against the same model with both forms: no
+    bfloat16 matrix keeps its rows; steps of many rows (the library's products on restored rows) and of single tokens
+    (the folded products) give the same logits bit for bit; a step of 40 rows, where the decode kernel stands in for
+    the library, the same within the bfloat16 tolerance."""
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    runners, raw, w16 = _runners(dev, 4, 64, WIDTHS[0], dtypes=("bfloat16", "bfloat16"), weight_copies=("both", "tiled"))
+    layer = runners[1].model.layers[0]
+    for m in (layer.mixer.w_qkv, layer.mixer.w_o, layer.ffn.w_gate_up, layer.ffn.w_down):
+        assert isinstance(m, ops.TiledOnly)
+    assert isinstance(runners[1].model.lm_head.weight, torch.Tensor)      # 4099 rows have no tiled form: they stay
+    assert not isinstance(runners[0].model.layers[0].mixer.w_o, ops.TiledOnly)
+    g = torch.Generator().manual_seed(13)
+    prompts = [torch.randint(0, RAW["vocab_size"], (n,), generator=g).tolist() for n in (300, 170, 20, 5)]
+    caches = [[runner.manager.admit(i) for i in range(4)] for runner in runners]
+
+    def both(entries_of):
+        outs = []
+        for runner, cs in zip(runners, caches):
+            entries = entries_of(cs)
+            for e in entries:
+                runner.manager.reserve(e.cache, len(e.tokens))
+            outs.append(runner.step(entries))
+        return outs
+
+    outs = both(lambda cs: [StepEntry(c, p, [0, len(p) - 1]) for c, p in zip(cs, prompts)])
+    assert torch.equal(outs[0], outs[1]), "prompts: other logits than with both forms"
+    more = torch.randint(0, RAW["vocab_size"], (40,), generator=g).tolist()
+    outs = both(lambda cs: [StepEntry(cs[0], more, [0, 39])])
+    _close(outs[1], outs[0], "a portion of 40 tokens")
+    for step in range(2):
+        toks = torch.randint(0, RAW["vocab_size"], (4,), generator=g).tolist()
+        outs = both(lambda cs: [StepEntry(c, [t], [0]) for c, t in zip(cs, toks)])
+        if step == 0:
+            _close(outs[1], outs[0], "single tokens after the portion")       # request 0's keys differ by rounding now
+            assert torch.equal(outs[0][1:], outs[1][1:])
+    assert torch.isfinite(outs[1]).all()
