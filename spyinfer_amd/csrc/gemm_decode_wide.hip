@@ -195,7 +195,7 @@ __global__ __launch_bounds__(GW * 64, 1) void gemm_decode_wide_kernel(
 static int wide_ct(int per, int MT, int gates, int max_ct) {
     int best = 1, best_cost = 1 << 30;
     for (int ct = 1; ct <= max_ct; ++ct) {
-        if (ct == 5) continue;                      // (not built)
+        if (ct == 5 || ct == 7 || (ct > 8 && ct != 12)) continue;   // (not built)
         const int cost = ((per + ct - 1) / ct) * MT + per * gates;
         if (cost < best_cost) { best = ct; best_cost = cost; }
     }
@@ -211,11 +211,15 @@ static bool gd_launch_wide(const GdArgs& a) {
 #ifndef GD_GW4_FROM
 #define GD_GW4_FROM 5        // (four waves from three row tiles on, measured at 40 to 64 rows: gate/up 41-43 us against 35-37)
 #endif
-        constexpr int GW = MT >= GD_GW4_FROM ? 4 : 8;    // beyond four row tiles: four waves with a SIMD's registers each
+#ifndef GD_GW4_STORE_FROM
+#define GD_GW4_STORE_FROM 3  // (the stored product, whose four-wave blocks take up to twelve column tiles at a time: the output head of
+#endif                       // 151936 x 4096 at 48 / 64 / 96 rows 253 / 267 / 288 us against 266 / 283 / 307 with eight waves and six tiles)
+        // beyond four row tiles (the stored product: beyond two): four waves with a SIMD's registers each
+        constexpr int GW = MT >= (EPI == EPI_STORE ? GD_GW4_STORE_FROM : GD_GW4_FROM) ? 4 : 8;
         // a group's accumulators (GATES * CT * MT tiles of four registers) leave room for its operands up to 24 tiles
         // (48 for a wave that has a SIMD to itself)
         constexpr int ROOM = GW == 8 ? 24 : 48;
-        constexpr int MAX_CT = ROOM / (GATES * MT) < 6 ? ROOM / (GATES * MT) : 6;
+        constexpr int MAX_CT = ROOM / (GATES * MT) < (GW == 4 ? 12 : 6) ? ROOM / (GATES * MT) : (GW == 4 ? 12 : 6);
         const int cus = gd_compute_units(), tiles = a.N / 16;
         // fewer than two tiles per CU: one tile per block, two blocks per CU (beyond four row tiles the gated product has
         // no other kernel: it walks here whatever the width, two column tiles at a time at least)
@@ -232,7 +236,7 @@ static bool gd_launch_wide(const GdArgs& a) {
                 return true;                                                                                          \
             }                                                                                                         \
         }
-        GD_WIDE_CASE(2) GD_WIDE_CASE(3) GD_WIDE_CASE(4) GD_WIDE_CASE(6)
+        GD_WIDE_CASE(2) GD_WIDE_CASE(3) GD_WIDE_CASE(4) GD_WIDE_CASE(6) GD_WIDE_CASE(8) GD_WIDE_CASE(12)
 #undef GD_WIDE_CASE
         return false;                                          // one tile at a time: the kernel with a tile per block stands
     }

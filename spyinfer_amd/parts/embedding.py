@@ -33,10 +33,11 @@ class TokenEmbedding(Part):
 
 
 class LMHead(Part):
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding = None, fold_rows: int = 32):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding = None, fold_rows: int = 64):
         """``fold_rows``: most rows for which the head runs as a decode product with the final norm folded in.  Above,
-        the library's product after a norm kernel is faster for a large matrix (measured with 151936 x 4096: 229 / 253 us
-        at 24 / 32 rows against the library's 264 / 269, but 266 / 283 against 261 / 269 at 48 / 64)."""
+        the library's product after a norm kernel is faster for a large matrix (measured with 151936 x 4096: 235 / 246 /
+        253 / 267 us at 24 / 32 / 48 / 64 rows against the library's 263 / 270 / 258 / 268 and a norm kernel of 6, but
+        281 / 288 / 367 against 274 / 280 / 293 at 80 / 96 / 128)."""
         self.vocab_size, self.hidden_size, self.tied_to = vocab_size, hidden_size, tied_to
         self.fold_rows = fold_rows
         self.weight = None
@@ -54,9 +55,9 @@ class LMHead(Part):
             self.weight, self.weight_tiled = ops.weight_forms(weights.pop(prefix + ".weight"))
 
     def can_fold(self, batch):
-        # without the matrix's rows there is no library product to prefer: the folded product stands as far as it is built
-        # for a plain input's rows (measured with 151936 x 4096 at 64 rows: 283 us against the library's 269 and a norm kernel)
-        rows = max(self.fold_rows, ops.TILED_ONLY_DIRECT_ROWS) if isinstance(self.weight, ops.TiledOnly) else self.fold_rows
+        # without the matrix's rows the library's product would have them restored first (more bytes than the product
+        # itself reads): the folded product stands as far as it is built
+        rows = ops.FUSED_DECODE_MAX_ROWS if isinstance(self.weight, ops.TiledOnly) else self.fold_rows
         return ops.fused_decode_ok(batch.T, batch.act_dtype, self.weight_tiled, max_rows=rows)
 
     def logits(self, resid, pending, final_norm, batch, out=None):
