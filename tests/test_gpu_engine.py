@@ -279,6 +279,47 @@ def test_greedy_bfloat16_follows_plain(folder_a):
     assert same >= 40
 
 
+def test_entry_point_with_matrices_in_tiles_only(tmp_path):
+    """``weight_copies="tiled"`` through the entry point, with a small configuration whose matrices all have a tiled form
+    (widths that are multiples of 128): no matrix of a layer keeps its rows, prompts of more than 64 tokens run through
+    the restored rows, and the tokens are those of the engine that keeps both forms; they follow the plain
+    implementation as far as its logits do not nearly tie."""
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.sampling import SamplingParams
+    from spyinfer_amd.weights import write_random_model
+    require_gpu()
+    raw = dict(TINY_A, hidden_size=128, num_attention_heads=4, num_key_value_heads=2, head_dim=32, intermediate_size=256,
+               vocab_size=512, tie_word_embeddings=False, num_hidden_layers=2)
+    folder = write_random_model(str(tmp_path / "m"), raw, 71, torch.bfloat16, **INIT)
+    ps = prompts(512, [5, 90, 33, 70], 3)
+    sp = SamplingParams(max_new_tokens=12, ignore_eos=True)
+    kw = dict(dtype="bfloat16", max_model_len=128, num_kvcache_blocks=40, max_num_seqs=8)
+    both = LLMEngine(folder, **kw).generate(ps, sp)
+    eng = LLMEngine(folder, weight_copies="tiled", **kw)
+    layer = eng.model.layers[0]
+    for m in (layer.mixer.w_qkv, layer.mixer.w_o, layer.ffn.w_gate_up, layer.ffn.w_down, eng.model.lm_head.weight):
+        assert isinstance(m, ops.TiledOnly)
+    assert isinstance(eng.model.embed.weight, torch.Tensor)
+    got = eng.generate(ps, sp)
+    assert got == both
+    plain = PlainQwen3(folder)
+    same = 0
+    for p, g in zip(ps, got):
+        toks = list(p)
+        for t in g:
+            logits = plain.forward(toks)[-1]
+            best = int(torch.argmax(logits))
+            if t != best:
+                assert float(logits[best] - logits[t]) < 0.1, "a bfloat16 token differs where the plain logits are apart"
+                break
+            same += 1
+            toks.append(t)
+    assert same >= 24
+    with pytest.raises(ValueError):
+        LLMEngine(folder, weight_copies="rows", **kw)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_graph_replays_equal_eager_steps(folder_c, dtype):
     """Decode steps from a captured graph, replayed many times with the program's own work between
