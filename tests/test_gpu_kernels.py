@@ -175,6 +175,9 @@ def test_linear_with_a_matrix_kept_in_tiles_only(monkeypatch):
                                             # tiles, several at a time, the last group of a run with fewer
                                             (64, 128, 8320, 8208, 1e-6), (37, 256, 8448, 9008, 1e-5), (20, 128, 8192, 16400, 1e-6),
                                             (48, 128, 128, 151936, 1e-6), (16, 128, 8320, 8208, 1e-6),
+                                            # stored products of very many columns at three and four row tiles: four-wave
+                                            # blocks with twelve and eight column tiles at a time, a last group with fewer
+                                            (64, 512, 128, 40000, 1e-6), (40, 1024, 128, 49168, 1e-5),
                                             # about a column tile per compute unit and a long K: K split over blocks, the
                                             # group's last block adding the parts (33 to 64 rows; a last group with fewer tiles; 2, 3, 4 parts)
                                             (64, 4096, 12288, 6144, 1e-6), (40, 4096, 8192, 6128, 1e-5), (52, 5120, 6400, 6160, 1e-6),
