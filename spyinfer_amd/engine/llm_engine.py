@@ -100,10 +100,7 @@ class LLMEngine:
         self.run_ahead = True
 
     def _pages_from_free_memory(self) -> int:
-        if self.device.type == "cuda":
-            free, _total = torch.cuda.mem_get_info(self.device)
-        else:
-            free = 1 << 30
+        free, _total = torch.cuda.mem_get_info(self.device)
         return pages_for_memory(free, self.config, self.model)
 
     # ---- requests --------------------------------------------------------

@@ -77,7 +77,7 @@ class ModelRunner:
         self.manager = CacheManager(model.cache_specs(), page_size, num_pages, max_num_seqs)
         self.storage = CacheStorage(self.manager, self.act_dtype, self.device)
         self.steps_run = 0
-        self.use_graphs = (not enforce_eager) and self.device.type == "cuda"
+        self.use_graphs = not enforce_eager
         limit = max_model_len or model.max_positions or num_pages * page_size
         self.fixed_max_blocks = min(-(-limit // page_size), max(1, num_pages))
         #: captured steps by shape; at most ``max_graphs``, further shapes run kernel by kernel.  A captured step is
@@ -134,8 +134,7 @@ class ModelRunner:
             raise ValueError("a request would reach %d tokens, the model's positions end at %d"
                              % (batch.max_kv_len, self.model.max_positions))
         self.model.plan(batch)
-        if self.device.type == "cuda":
-            self._pack(batch)
+        self._pack(batch)
         if graphable:
             batch.graph_key()
         return PreparedStep(batch, graphable)
@@ -157,10 +156,7 @@ class ModelRunner:
         if graphable:
             logits = self._step_graph(batch, token_source)
         else:
-            if self.device.type == "cuda":
-                self._upload(batch, None)
-            else:
-                batch.upload()
+            self._upload(batch, None)
             if token_source is not None:
                 batch.token_ids.copy_(token_source)
             logits = self.model.forward(batch, self.storage)

@@ -57,12 +57,17 @@ class Sampler:
         R = logits.shape[0]
         if R == 0:
             return None
-        host = torch.empty((2, R), dtype=torch.float32, pin_memory=self.device.type == "cuda")
+        host = self._host_buffer(R)
         flat = host.numpy()
         flat[0] = temperatures
         flat[1] = [uniform_for(s, i) if t > 0 else 0.0 for s, i, t in zip(seeds, indices, temperatures)]
         dev = host.to(self.device, non_blocking=True)
         return ops.sample(logits, dev[0], dev[1])
+
+    @staticmethod
+    def _host_buffer(R: int) -> torch.Tensor:
+        """Pinned host memory [2, R] for the rows' temperatures and uniform numbers (its copy to the device does not wait)."""
+        return torch.empty((2, R), dtype=torch.float32, pin_memory=True)
 
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
                indices: Sequence[int]) -> List[int]:

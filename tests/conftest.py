@@ -2,6 +2,7 @@ import os
 import sys
 
 import pytest
+import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
@@ -34,6 +35,21 @@ def emu_ops(monkeypatch):
     monkeypatch.setattr(ops, "fused_decode_ok", lambda *a, **k: False)
     monkeypatch.setattr(ops, "fused_attention_ok", lambda *a, **k: False)
     monkeypatch.setattr(ops, "hip", lambda: None)
+    # what the engine does with the device beside the operations: transfers through pinned memory, HIP graphs, the
+    # device's free memory
+    from spyinfer_amd.engine.llm_engine import LLMEngine, pages_for_memory
+    from spyinfer_amd.engine.runner import ModelRunner
+    from spyinfer_amd.sampling.sampler import Sampler
+    runner_init = ModelRunner.__init__
+
+    def init_without_graphs(self, *args, **kwargs):
+        kwargs["enforce_eager"] = True
+        runner_init(self, *args, **kwargs)
+    monkeypatch.setattr(ModelRunner, "__init__", init_without_graphs)
+    monkeypatch.setattr(ModelRunner, "_pack", lambda self, batch: None)
+    monkeypatch.setattr(ModelRunner, "_upload", lambda self, batch, dev_buf, bind=True: batch.upload())
+    monkeypatch.setattr(LLMEngine, "_pages_from_free_memory", lambda self: pages_for_memory(1 << 30, self.config, self.model))
+    monkeypatch.setattr(Sampler, "_host_buffer", staticmethod(lambda R: torch.empty((2, R), dtype=torch.float32)))
 
 
 @pytest.fixture(autouse=True)
