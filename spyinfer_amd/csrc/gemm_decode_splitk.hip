@@ -237,6 +237,12 @@ long long gd_splitk_workspace_bytes() {
     return SK_COUNTER_BYTES + (long long)gd_compute_units() * SK_MAX_TILES_PER_BLOCK * 1024;
 }
 
+#ifndef SK_MIN_CHUNKS
+#define SK_MIN_CHUNKS 12    // chunks of K that a part has at least (three for every two waves of eight)
+#endif
+#ifndef SK_MIN_FILL
+#define SK_MIN_FILL 90      // per cent of the compute units that must get a block
+#endif
 #ifndef SK_STORE_FROM
 #define SK_STORE_FROM 64    // rows beyond which the stored product splits K
 #endif
@@ -244,18 +250,19 @@ long long gd_splitk_workspace_bytes() {
 #define GD_SPLITK 1       // 0: never taken (for measurements)
 #endif
 
-// Column tiles per block and parts of K: the pair that gives the most compute units a block, each of a part's 8 waves
-// at least two chunks of K (with one, the way of the parts through memory costs more than X's traffic: the o product
-// of 4096 x 4096 at 64 rows took 17.3 us against 15.1 with a column tile per block; down, 4096 x 12288, 27.6 against
-// 35.1, and qkv, 6144 x 4096 in two parts, 18.6 against 19.3); among equals the most column tiles.
+// Column tiles per block and parts of K: the pair that gives the most compute units a block, a part with at least 12
+// chunks of K for its 8 waves (with one chunk per wave the way of the parts through memory costs more than X's traffic:
+// the o product of 4096 x 4096 at 64 rows took 17.3 us in four parts against 15.1 with a column tile per block; with 13
+// chunks a part, 5120 x 5120 in three parts, 20.1 against 28.3; down, 4096 x 12288, 27.6 against 35.1, and qkv,
+// 6144 x 4096 in two parts, 18.6 against 19.3); among equals the most column tiles.
 static void sk_shape(int tiles, int nfull, int cus, int* ct_out, int* ks_out) {
     int best_ct = 0, best_ks = 0, best_blocks = 0;
     for (int ct = 4; ct >= 3; --ct) {
         const int groups = (tiles + ct - 1) / ct;
         int ks = cus / groups;
-        if (ks > nfull / 16) ks = nfull / 16;
+        if (ks > nfull / SK_MIN_CHUNKS) ks = nfull / SK_MIN_CHUNKS;
         if (ks > SK_MAX_PARTS) ks = SK_MAX_PARTS;
-        if (ks < 2 || groups * ks * 10 < cus * 9) continue;     // (nine in ten compute units at least)
+        if (ks < 2 || groups * ks * 100 < cus * SK_MIN_FILL) continue;     // (nine in ten compute units at least)
         if (groups * ks > best_blocks) { best_blocks = groups * ks; best_ct = ct; best_ks = ks; }
     }
     *ct_out = best_ct;
