@@ -183,6 +183,9 @@ def test_linear_with_a_matrix_kept_in_tiles_only(monkeypatch):
                                             (64, 4096, 12288, 6144, 1e-6), (40, 4096, 8192, 6128, 1e-5), (52, 5120, 6400, 6160, 1e-6),
                                             # (three parts of 13, 13 and 14 chunks for eight waves each)
                                             (64, 5120, 5120, 6160, 1e-6),
+                                            # gated products with five pairs of column tiles per compute unit: four-wave blocks
+                                            # that take a block's run as one group of six (four and three row tiles)
+                                            (64, 1024, 17408, 96, 1e-6), (40, 256, 17408, 96, 1e-5),
                                             # more than 8 chunks of K for every wave in the loops that ask for the next step's operands ahead
                                             (40, 9216, 256, 8208, 1e-6), (50, 4096, 36864, 64, 1e-6)])
 def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
