@@ -243,6 +243,9 @@ long long gd_splitk_workspace_bytes() {
 #ifndef SK_MIN_FILL
 #define SK_MIN_FILL 90      // per cent of the compute units that must get a block
 #endif
+#ifndef SK_EVEN_FILL
+#define SK_EVEN_FILL 85     // per cent of the blocks' turns that a tile per block must fill to stand up to 32 rows
+#endif
 #ifndef SK_STORE_FROM
 #define SK_STORE_FROM 64    // rows beyond which the stored product splits K
 #endif
@@ -300,15 +303,28 @@ static bool sk_rows(const GdArgs& a) {
     }
     if (a.M > 64) return false;
     if (a.M > 48) return sk_launch<EPI, SCALED, TC, 4, XT, OT>(a);
-    return sk_launch<EPI, SCALED, TC, 3, XT, OT>(a);
+    if (a.M > 32) return sk_launch<EPI, SCALED, TC, 3, XT, OT>(a);
+    if constexpr (EPI == EPI_RESID) {                     // (one and two row tiles: the residual product only)
+        if (a.M > 16) return sk_launch<EPI, SCALED, TC, 2, XT, OT>(a);
+        return sk_launch<EPI, SCALED, TC, 1, XT, OT>(a);
+    }
+    return false;
 }
 
 // Built for the combinations that a decode step has: the residual product of a plain input (row-major or in operand
 // order) with its output in operand order, and the stored bfloat16 product of a normed input in operand order.
 bool gd_splitk_try(const GdArgs& a, int epi, bool scaled, bool f32_out) {
-    // (up to 32 rows the kernels with a column tile per block are as fast: down 23.5 against 23.6 us at 32 rows)
-    if (!GD_SPLITK || a.ws == nullptr || a.M <= 32 || a.M > 128 || a.N % 16 != 0 || a.K % GD_CHUNK != 0) return false;
-    if (a.N / 16 >= 2 * gd_compute_units()) return false;           // many columns: the kernels that walk column tiles
+    if (!GD_SPLITK || a.ws == nullptr || a.M > 128 || a.N % 16 != 0 || a.K % GD_CHUNK != 0) return false;
+    const int cus = gd_compute_units(), tiles = a.N / 16;
+    if (tiles >= 2 * cus) return false;                             // many columns: the kernels that walk column tiles
+    // Up to 32 rows the kernels with a column tile per block are as fast where their blocks fill the compute units evenly
+    // (256 tiles: down, 4096 x 12288, 23.5 against 23.6 us at 32 rows).  Where the last turn of blocks is short (320 tiles
+    // on 256 compute units: some units stream two tiles, the others one), equal parts for all pay from the first row on:
+    // down of 5120 x 25600 55.9 / 65.6 / 77.0 us at 8 / 16 / 24 rows with a tile per block, against 50.7 at 40 rows here.
+    if (a.M <= 32) {
+        const int turns = (tiles + cus - 1) / cus;
+        if (tiles * 100 >= turns * cus * SK_EVEN_FILL) return false;
+    }
     if (epi == EPI_RESID && !scaled && a.ot) {
         return a.xt ? sk_rows<EPI_RESID, false, bf16_t, true, true>(a) : sk_rows<EPI_RESID, false, bf16_t, false, true>(a);
     }

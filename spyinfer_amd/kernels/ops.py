@@ -436,7 +436,7 @@ def _gemm_decode(x, tiled: torch.Tensor, epi: int, n_out: int, out, resid, xw_ou
     xw_t = xw_out.data if isinstance(xw_out, OperandRows) else xw_out
     _dev(xs, ss, tiled, out_t, resid, xw_t, w_next, ss_out)
     _check(0 < M <= FUSED_DECODE_MAX_ROWS, "decode product: %d rows (1..%d allowed)" % (M, FUSED_DECODE_MAX_ROWS))
-    ws = decode_workspace(xs.device) if M > 16 else None
+    ws = decode_workspace(xs.device)
     hip().call("spy_gemm_decode", _ptr(xs), ctypes.c_int(0 if ss is None else 1), _ptr(ss), ctypes.c_int(0 if ss is None else ss.shape[0]),
                ctypes.c_float(eps), _ptr(tiled), ctypes.c_int(epi), _ptr(out_t), ctypes.c_int(0 if out_t is None else _code(out_t, "out")),
                _ptr(resid), _ptr(xw_t), _ptr(w_next), _ptr(ss_out), ctypes.c_int(M), ctypes.c_int(n_out), ctypes.c_int(K),

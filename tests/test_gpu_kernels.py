@@ -183,6 +183,8 @@ def test_linear_with_a_matrix_kept_in_tiles_only(monkeypatch):
                                             (64, 4096, 12288, 6144, 1e-6), (40, 4096, 8192, 6128, 1e-5), (52, 5120, 6400, 6160, 1e-6),
                                             # (three parts of 13, 13 and 14 chunks for eight waves each)
                                             (64, 5120, 5120, 6160, 1e-6),
+                                            # 320 column tiles for 256 compute units: K split over blocks from the first row on
+                                            (8, 5120, 5120, 96, 1e-6), (24, 5120, 6400, 96, 1e-5), (1, 5120, 3200, 64, 1e-6),
                                             # gated products with five pairs of column tiles per compute unit: four-wave blocks
                                             # that take a block's run as one group of six (four and three row tiles)
                                             (64, 1024, 17408, 96, 1e-6), (40, 256, 17408, 96, 1e-5),
@@ -233,7 +235,10 @@ def test_decode_products_with_folded_norm(M, H, I, NQKV, eps):
     # the same chain with row-major hand-over: the same numbers where both forms run through the same kernel (up to 16
     # rows); above that the kernels that walk or split differ by form and add in another order, and each form is held
     # against float64 by itself
-    same_kernel = M <= 16
+    # (and where a tile per block fills the compute units evenly: with 320 column tiles for 256 units the products that hand
+    # over in operand order split K over blocks from the first row on)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    same_kernel = M <= 16 and ((H // 16) % cus == 0 or H // 16 < cus // 4)
     ops.OPERAND_ORDER = False
     try:
         resid_r = resid0.clone()
