@@ -33,6 +33,10 @@ SHAPES = {
     # the size of model that the reference's own run script names (run.sh:2): 28 narrow layers, where a step is many short kernels
     "0.6b": ("Qwen3-0.6B shape", dict(MODEL_8B, num_hidden_layers=28, hidden_size=1024, num_attention_heads=16, intermediate_size=3072,
                                       tie_word_embeddings=True)),
+    "1.7b": ("Qwen3-1.7B shape", dict(MODEL_8B, num_hidden_layers=28, hidden_size=2048, num_attention_heads=16, intermediate_size=6144,
+                                      tie_word_embeddings=True)),
+    "4b": ("Qwen3-4B shape", dict(MODEL_8B, num_hidden_layers=36, hidden_size=2560, num_attention_heads=32, intermediate_size=9728,
+                                  tie_word_embeddings=True)),
     "8b": ("Qwen3-8B shape", MODEL_8B),
     "14b": ("Qwen3-14B shape", dict(MODEL_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)),
     "32b": ("Qwen3-32B shape", dict(MODEL_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)),

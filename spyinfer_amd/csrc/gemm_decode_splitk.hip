@@ -321,9 +321,11 @@ bool gd_splitk_try(const GdArgs& a, int epi, bool scaled, bool f32_out) {
     // (256 tiles: down, 4096 x 12288, 23.5 against 23.6 us at 32 rows).  Where the last turn of blocks is short (320 tiles
     // on 256 compute units: some units stream two tiles, the others one), equal parts for all pay from the first row on:
     // down of 5120 x 25600 55.9 / 65.6 / 77.0 us at 8 / 16 / 24 rows with a tile per block, against 50.7 at 40 rows here.
+    // (Fewer tiles than units and few rows: no unit streams two tiles, and the parts' way through memory costs what the
+    // idle units would save: down of 2560 x 9728, 160 tiles, 13.5 against 12.4 us at 8 rows, 13.4 against 14.9 at 16.)
     if (a.M <= 32) {
         const int turns = (tiles + cus - 1) / cus;
-        if (tiles * 100 >= turns * cus * SK_EVEN_FILL) return false;
+        if (tiles * 100 >= turns * cus * SK_EVEN_FILL || (a.M <= 8 && turns == 1)) return false;
     }
     if (epi == EPI_RESID && !scaled && a.ot) {
         return a.xt ? sk_rows<EPI_RESID, false, bf16_t, true, true>(a) : sk_rows<EPI_RESID, false, bf16_t, false, true>(a);
