@@ -27,21 +27,33 @@
 
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 
+#ifndef GD_HALVES
+#define GD_HALVES 1       // 0: blocks of three halves of column tiles are never taken (for measurements)
+#endif
 #ifndef GD_WAVES_GATED
 #define GD_WAVES_GATED 4
 #endif
 
-template <int EPI, bool SCALED, typename TC, int GD_WAVES, bool XT, bool OT>
+// H3: a block has three halves of column tiles (24 columns) instead of one tile: tile t whole and the lower half of
+// tile t + 1, or the upper half of tile t and tile t + 1 whole, in turn.  For a matrix of one and a half column tiles per
+// compute unit (qkv of 6144 columns on 256 units) every unit then streams the same number of bytes; with a tile per
+// block half of the units stream two tiles and the others one.  A half tile is the lanes r < 8 (or r >= 8) of every
+// fragment of W, 128 bytes in one piece each, and the columns 4 g + i of the lane groups g < 2 (g >= 2) of the result.
+// The stored product only.
+template <int EPI, bool SCALED, typename TC, int GD_WAVES, bool XT, bool OT, bool H3 = false>
 __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, float* __restrict__ resid_out,
     bf16_t* __restrict__ xw_out, const bf16_t* __restrict__ w_next, float* __restrict__ ss_out, const float* __restrict__ ss_in,
     int n_parts, float eps, int M, int N, int K) {
-    constexpr int NT = EPI == EPI_GATED ? 2 : 1;
+    static_assert(!H3 || EPI == EPI_STORE, "halves of column tiles: the stored product only");
+    constexpr int NT = (EPI == EPI_GATED || H3) ? 2 : 1;
     __shared__ float red[(GD_WAVES - 1) * NT * 64 * 4];
     __shared__ float ss_red[GD_WAVES * 4 * 16];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int r = lane & 15, g = lane >> 4;
-    const int n_base = blockIdx.x * 16;
+    const int tile0 = H3 ? (3 * (int)blockIdx.x) >> 1 : (int)blockIdx.x;      // the block's (first) column tile
+    const bool lower = (blockIdx.x & 1) == 0;                                   // H3: tile0 whole and half of the next, or the reverse
+    const int n_base = tile0 * 16;
     const bool x_ok = r < M;                       // lanes whose row of X does not exist load nothing
 
     // Loads whose values are needed only after the product are issued now, so that they are on their way while
@@ -67,11 +79,13 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     f32x4_t acc[NT], acc2[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) { acc[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f}; acc2[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f}; }
-    const size_t chunk_stride = (size_t)(NT * N / 16) * 4096;         // bytes of one chunk of all tiles
-    const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)blockIdx.x * 4096;
+    const size_t chunk_stride = (size_t)((EPI == EPI_GATED ? 2 : 1) * N / 16) * 4096;         // bytes of one chunk of all tiles
+    const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)tile0 * 4096;
     unsigned woff[NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) woff[nt] = (unsigned)(nt * N / 16) * 4096u + 16u * lane;
+    for (int nt = 0; nt < NT; ++nt) woff[nt] = (H3 ? (unsigned)nt : (unsigned)(nt * N / 16)) * 4096u + 16u * lane;
+    // H3: the lanes of a fragment of tile nt that this block reads
+    const bool w_on[2] = {!H3 || lower || r >= 8, !H3 || !lower || r < 8};
     const char* xbase = reinterpret_cast<const char*>(X);
     const unsigned xoff = XT ? 16u * lane : (unsigned)min(r, M - 1) * (unsigned)K * 2u + 16u * g;
 
@@ -81,8 +95,11 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
         const char* wb_ = wbase + (size_t)(CHUNK) * chunk_stride;                                        \
         const char* xb_ = xbase + (size_t)(CHUNK) * (XT ? 4096 : GD_CHUNK * 2) + xoff;                   \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                  \
-            _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                            \
-                A[nt][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wb_ + woff[nt] + 1024 * j));                \
+            _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) {                                          \
+                if (!H3) A[nt][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wb_ + woff[nt] + 1024 * j));      \
+                else A[nt][j] = w_on[nt] ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wb_ + woff[nt] + 1024 * j)) \
+                                         : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};                                                       \
+            }                                                                                            \
             B[j] = x_ok ? *reinterpret_cast<const bf16x8_t*>(xb_ + (XT ? 1024 : 64) * j) : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}; \
         }                                                                                                \
     }
@@ -145,6 +162,18 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
         return;
     }
     if (m >= M) return;
+    if constexpr (H3) {
+        // tile0: all columns (lower) or those of its upper half; the next tile: its lower half, or all
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+            const bool mine = nt == 0 ? (lower || g >= 2) : (!lower || g < 2);
+            if (!mine) continue;
+            TC* out = C + (size_t)m * N + n + 16 * nt;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[i] = from_f32<TC>(acc[nt][i]);
+        }
+        return;
+    }
     TC* out = C + (OT ? operand_order(m, n) : (size_t)m * N + n);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -159,11 +188,13 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
 // of sum(h^2) have 16 MT rows each: ss[n][16 MT].
 // CT: column tiles of 16 per block.  Every block reads all of X, from L2, and with MT row tiles that is MT times the
 // bytes of its W tile: with two column tiles the X fragments in registers serve both, and X's traffic halves.
-template <int EPI, bool SCALED, typename TC, int MT, int CT, int GD_WAVES, bool XT, bool OT>
+// H3 (with CT = 2, the stored product): three halves of column tiles per block, as in gemm_decode_kernel.
+template <int EPI, bool SCALED, typename TC, int MT, int CT, int GD_WAVES, bool XT, bool OT, bool H3 = false>
 __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, float* __restrict__ resid_out,
     bf16_t* __restrict__ xw_out, const bf16_t* __restrict__ w_next, float* __restrict__ ss_out, const float* __restrict__ ss_in,
     int n_parts, float eps, int M, int N, int K) {
+    static_assert(!H3 || (EPI == EPI_STORE && CT == 2), "halves of column tiles: the stored product, two tiles a block");
     constexpr int NT = (EPI == EPI_GATED ? 2 : 1) * CT;      // W tiles per block: [gate tiles | up tiles] for the gated product
     constexpr int MP = 16 * MT;
     __shared__ f32x4_t red[(GD_WAVES - 1) * NT * MT * 64];
@@ -190,7 +221,10 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     const size_t chunk_stride = (size_t)((EPI == EPI_GATED ? 2 : 1) * N / 16) * 4096;
-    const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)blockIdx.x * (CT * 4096);
+    const int tile0 = H3 ? (3 * (int)blockIdx.x) >> 1 : (int)blockIdx.x * CT;       // the block's first column tile
+    const bool lower = (blockIdx.x & 1) == 0;                // H3: tile0 whole and the lower half of the next, or the reverse
+    const bool w_on[2] = {!H3 || lower || r >= 8, !H3 || !lower || r < 8};
+    const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)tile0 * 4096;
     unsigned woff[NT], xoff[MT];
     bool x_ok[MT];
 #pragma unroll
@@ -207,8 +241,11 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
         const char* wb = wbase + (size_t)(CHUNK) * chunk_stride;                                                     \
         const char* xb = xbase + (size_t)(CHUNK) * (XT ? 4 * MT * 1024 : GD_CHUNK * 2);                              \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                              \
-            _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                        \
-                A[nt][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wb + woff[nt] + 1024 * j));                             \
+            _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) {                                                      \
+                if (!H3) A[nt][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wb + woff[nt] + 1024 * j));                    \
+                else A[nt][j] = w_on[nt & 1] ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wb + woff[nt] + 1024 * j))          \
+                                             : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};                                                                 \
+            }                                                                                                        \
             _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                        \
                 B[mt][j] = x_ok[mt] ? *reinterpret_cast<const bf16x8_t*>(xb + xoff[mt] + (XT ? MT * 1024 : 64) * j)  \
                                     : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};                                              \
@@ -259,7 +296,8 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
         }
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
-            const int tile = blockIdx.x * CT + ct, n = tile * 16 + 4 * g;
+            const int tile = tile0 + ct, n = tile * 16 + 4 * g;
+            if (H3 && !(ct == 0 ? (lower || g >= 2) : (!lower || g < 2))) continue;      // the other block's half of the tile
             if (SCALED) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) { acc[ct][mt][i] *= scale; if (EPI == EPI_GATED) acc[CT + ct][mt][i] *= scale; }
@@ -301,14 +339,30 @@ static bool gd_launch2(const GdArgs& a) {
     // Two column tiles per block where that leaves enough blocks (measured, 64 rows: qkv of 6144 columns 26.8 -> 20.5
     // us; with 4096 columns, 128 blocks, 15.4 -> 19.4 us; the gated product 53 -> 61 us: its block has one wave per SIMD then)
     const bool two = EPI == EPI_STORE && a.N % 32 == 0 && a.N / 32 >= 192;
+    // one and a half column tiles per compute unit: three halves of tiles per block (the stored product of a normed input)
+    bool halves_rows = false;
+    if constexpr (EPI == EPI_STORE && SCALED && XT && !OT && sizeof(TC) == 2) {
+        const int cus_ = gd_compute_units();
+        halves_rows = GD_HALVES && a.N % 48 == 0 && (a.N / 24) % cus_ == 0 && (a.N / 16) % cus_ != 0;
+    }
     // beyond four row tiles: blocks of eight waves (a wave per row tile runs the epilogue), one column tile; built for
     // what a decode step has: inputs in operand order, the residual product of a plain input with its output in operand
     // order, the stored product of a normed input
     constexpr bool TALL = XT && ((EPI == EPI_RESID && !SCALED && OT) || (EPI == EPI_STORE && SCALED));
-    if (a.M <= 16) gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
+    if (a.M <= 16) {
+        // one and a half column tiles per compute unit: three halves of tiles per block
+        bool halves = false;
+        if constexpr (EPI == EPI_STORE && SCALED && XT && !OT && sizeof(TC) == 2) {
+            const int cus = gd_compute_units();
+            halves = GD_HALVES && a.N % 48 == 0 && (a.N / 24) % cus == 0 && (a.N / 16) % cus != 0;
+            if (halves) gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT, true><<<a.N / 24, W * 64, 0, a.st>>>(GD_ARGS);
+        }
+        if (!halves) gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
+    }
 #define GD_ROWS(MT)                                                                                                  \
     if constexpr (EPI == EPI_STORE) {                                                                                \
-        if (two) gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 2, W, XT, OT><<<a.N / 32, W * 64, 0, a.st>>>(GD_ARGS);   \
+        if (halves_rows) gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 2, W, XT, OT, true><<<a.N / 24, W * 64, 0, a.st>>>(GD_ARGS); \
+        else if (two) gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 2, W, XT, OT><<<a.N / 32, W * 64, 0, a.st>>>(GD_ARGS);   \
         else gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 1, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);      \
     } else gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 1, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS)
 #define GD_ROWS_TALL(MT)                                                                                             \
