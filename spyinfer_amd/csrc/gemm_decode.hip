@@ -40,18 +40,20 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 // block half of the units stream two tiles and the others one.  A half tile is the lanes r < 8 (or r >= 8) of every
 // fragment of W, 128 bytes in one piece each, and the columns 4 g + i of the lane groups g < 2 (g >= 2) of the result.
 // The stored product only.
-template <int EPI, bool SCALED, typename TC, int GD_WAVES, bool XT, bool OT, bool H3 = false>
+// HT: 0, or the number of half tiles of a block, 3 or 5 (two and a half tiles per unit: qkv of 10240 columns).
+template <int EPI, bool SCALED, typename TC, int GD_WAVES, bool XT, bool OT, int HT = 0>
 __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, float* __restrict__ resid_out,
     bf16_t* __restrict__ xw_out, const bf16_t* __restrict__ w_next, float* __restrict__ ss_out, const float* __restrict__ ss_in,
     int n_parts, float eps, int M, int N, int K) {
-    static_assert(!H3 || EPI == EPI_STORE, "halves of column tiles: the stored product only");
-    constexpr int NT = (EPI == EPI_GATED || H3) ? 2 : 1;
+    constexpr bool H3 = HT != 0;
+    static_assert(!H3 || (EPI == EPI_STORE && (HT == 3 || HT == 5)), "three or five halves of column tiles, the stored product only");
+    constexpr int NT = H3 ? (HT + 1) / 2 : (EPI == EPI_GATED ? 2 : 1);
     __shared__ float red[(GD_WAVES - 1) * NT * 64 * 4];
     __shared__ float ss_red[GD_WAVES * 4 * 16];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int r = lane & 15, g = lane >> 4;
-    const int tile0 = H3 ? (3 * (int)blockIdx.x) >> 1 : (int)blockIdx.x;      // the block's (first) column tile
+    const int tile0 = H3 ? (HT * (int)blockIdx.x) >> 1 : (int)blockIdx.x;     // the block's (first) column tile
     const bool lower = (blockIdx.x & 1) == 0;                                   // H3: tile0 whole and half of the next, or the reverse
     const int n_base = tile0 * 16;
     const bool x_ok = r < M;                       // lanes whose row of X does not exist load nothing
@@ -84,8 +86,11 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     unsigned woff[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) woff[nt] = (H3 ? (unsigned)nt : (unsigned)(nt * N / 16)) * 4096u + 16u * lane;
-    // H3: the lanes of a fragment of tile nt that this block reads
-    const bool w_on[2] = {!H3 || lower || r >= 8, !H3 || !lower || r < 8};
+    // halves: the lanes of a fragment of tile nt that this block reads (its first tile's upper half only, or its last
+    // tile's lower half only)
+    bool w_on[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) w_on[nt] = !H3 || (nt == 0 ? (lower || r >= 8) : (nt == NT - 1 ? (!lower || r < 8) : true));
     const char* xbase = reinterpret_cast<const char*>(X);
     const unsigned xoff = XT ? 16u * lane : (unsigned)min(r, M - 1) * (unsigned)K * 2u + 16u * g;
 
@@ -165,8 +170,8 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
     if constexpr (H3) {
         // tile0: all columns (lower) or those of its upper half; the next tile: its lower half, or all
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-            const bool mine = nt == 0 ? (lower || g >= 2) : (!lower || g < 2);
+        for (int nt = 0; nt < NT; ++nt) {
+            const bool mine = nt == 0 ? (lower || g >= 2) : (nt == NT - 1 ? (!lower || g < 2) : true);
             if (!mine) continue;
             TC* out = C + (size_t)m * N + n + 16 * nt;
 #pragma unroll
@@ -354,8 +359,14 @@ static bool gd_launch2(const GdArgs& a) {
         bool halves = false;
         if constexpr (EPI == EPI_STORE && SCALED && XT && !OT && sizeof(TC) == 2) {
             const int cus = gd_compute_units();
-            halves = GD_HALVES && a.N % 48 == 0 && (a.N / 24) % cus == 0 && (a.N / 16) % cus != 0;
-            if (halves) gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT, true><<<a.N / 24, W * 64, 0, a.st>>>(GD_ARGS);
+            const bool uneven = GD_HALVES && (a.N / 16) % cus != 0;
+            if (uneven && a.N % 48 == 0 && (a.N / 24) % cus == 0) {
+                gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT, 3><<<a.N / 24, W * 64, 0, a.st>>>(GD_ARGS);
+                halves = true;
+            } else if (uneven && a.N % 80 == 0 && (a.N / 40) % cus == 0) {
+                gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT, 5><<<a.N / 40, W * 64, 0, a.st>>>(GD_ARGS);
+                halves = true;
+            }
         }
         if (!halves) gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
     }

@@ -183,6 +183,8 @@ def test_linear_with_a_matrix_kept_in_tiles_only(monkeypatch):
                                             (64, 4096, 12288, 6144, 1e-6), (40, 4096, 8192, 6128, 1e-5), (52, 5120, 6400, 6160, 1e-6),
                                             # (three parts of 13, 13 and 14 chunks for eight waves each)
                                             (64, 5120, 5120, 6160, 1e-6),
+                                            # two and a half column tiles per compute unit: blocks of five halves of tiles
+                                            (8, 256, 128, 10240, 1e-6), (16, 128, 128, 10240, 1e-5),
                                             # 320 column tiles for 256 compute units: K split over blocks from the first row on
                                             (8, 5120, 5120, 96, 1e-6), (24, 5120, 6400, 96, 1e-5), (1, 5120, 3200, 64, 1e-6),
                                             # gated products with five pairs of column tiles per compute unit: four-wave blocks
