@@ -177,6 +177,26 @@ class CacheManager:
                     table[i] = -1
                     rc.versions[g.index] += 1
 
+    def rewind(self, rc: RequestCache, num_tokens: int) -> bool:
+        """Count only the first ``num_tokens`` tokens as cached again, so that the later ones are computed anew into
+        the pages they already have (a further turn of a request whose last token was stored by a step run ahead
+        needs that token's logits once more).  False, and nothing changed, if that cannot be done: a state of fixed
+        size has taken the tokens in for good, or a window has given back a page that a query at ``num_tokens`` reads."""
+        if not (0 <= num_tokens <= rc.num_tokens):
+            raise ValueError("rewind to %d tokens, %d are cached" % (num_tokens, rc.num_tokens))
+        if num_tokens == rc.num_tokens:
+            return True
+        if self.state_groups:
+            return False
+        for g in self.page_groups:
+            table = rc.tables[g.index]
+            last = -(-rc.num_tokens // g.page_size)
+            if any(table[i] < 0 for i in range(g.first_needed_page(num_tokens), last)):
+                return False
+        rc.reserved += rc.num_tokens - num_tokens
+        rc.num_tokens = num_tokens
+        return True
+
     def release(self, rc: RequestCache) -> None:
         """The request ends (or is preempted): everything it holds goes back."""
         if not rc.live:

@@ -155,6 +155,13 @@ class Scheduler:
         while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs:
             seq = self.waiting[0]
             kept = seq.cache is not None and seq.cache.live        # a further turn of a request whose cache is parked
+            if kept and seq.cache.num_tokens >= len(seq) and not self.manager.rewind(seq.cache, len(seq) - 1):
+                # The turn brings no token that is not cached yet (a step run ahead stored the last one, and the turn
+                # is empty), but its first new token is sampled from the last token's logits: that token runs again.
+                # Where the cache cannot step back, it is given up and the history computed anew.
+                self._unpark(seq)
+                self.manager.release(seq.cache)
+                seq.cache, kept = None, False
             if not kept and not self.manager.can_admit() and not self._reclaim_parked():
                 break
             cache = seq.cache if kept else self.manager.admit(seq.id)

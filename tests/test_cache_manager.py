@@ -148,3 +148,35 @@ def test_a_cache_kind_from_outside_forms_groups_of_its_own():
     m.check()
     with pytest.raises(TypeError, match="CacheKind"):
         CacheManager([object()], 8, 4, 2)
+
+
+def test_rewind_steps_back_where_the_cache_allows_it():
+    m = CacheManager([PagedKV(1, 8)], page_size=4, num_pages=4, max_num_seqs=2)
+    rc = m.admit("a")
+    m.reserve(rc, 8)
+    m.commit(rc, 8)
+    table = list(rc.tables[0])
+    assert m.rewind(rc, 7) and rc.num_tokens == 7 and rc.reserved == 1 and rc.tables[0] == table
+    assert m.pages_needed(rc, 1) == [0]
+    m.reserve(rc, 1)
+    m.commit(rc, 1)
+    assert rc.num_tokens == 8 and rc.reserved == 0
+    m.check()
+    with pytest.raises(ValueError):
+        m.rewind(rc, 9)
+    # a window that has given back the page which the earlier position reads: no way back
+    w = CacheManager([PagedKV(1, 8, window=4)], page_size=4, num_pages=4, max_num_seqs=2)
+    rc = w.admit("a")
+    w.reserve(rc, 7)
+    w.commit(rc, 7)                 # the next query (position 7) reads keys 4..7: page 0 is back
+    assert rc.tables[0][0] == -1
+    assert not w.rewind(rc, 6) and rc.num_tokens == 7          # position 6 reads keys 3..6
+    w.reserve(rc, 1)
+    w.commit(rc, 1)
+    assert w.rewind(rc, 7) and rc.num_tokens == 7               # position 7 reads keys 4..7, all there
+    # a state of fixed size has taken its tokens in for good
+    s = CacheManager([PagedKV(1, 8), FixedState((4,))], page_size=4, num_pages=4, max_num_seqs=2)
+    rc = s.admit("a")
+    s.reserve(rc, 5)
+    s.commit(rc, 5)
+    assert not s.rewind(rc, 4) and rc.num_tokens == 5 and s.rewind(rc, 5)

@@ -201,3 +201,48 @@ def test_refused_turn_leaves_the_request_as_it_was_and_draws_go_on(folder_a, emu
         eng.remove_request(rid)
         eng.runner.manager.check()
         assert eng.runner.manager.num_free_pages() == [8] and eng.runner.manager.slots.num_free == eng.config.max_num_seqs
+
+
+def test_a_turn_without_new_tokens_after_an_end_token_met_while_a_step_ran_ahead(folder_a, emu_ops):
+    """A request ends at its end token while the next step is already in flight: that step has stored the end token's
+    key and value, so a kept cache covers every token of the request.  A further turn that brings no tokens (the
+    reference's append_to_request takes an empty message, src/engine/llm_engine.cpp:40-73) still has to sample from the
+    last token's logits: the cache steps back by one token.  Tokens equal those of an engine that keeps nothing, the
+    other requests go on, and nothing is lost."""
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    plain = PlainQwen3(folder_a)
+    ps = prompts(256, [14, 6], seed=11)
+    g0 = plain.greedy(ps[0], 10)
+    k = max(i for i in range(10) if g0[i] not in g0[:i])
+    assert k >= 2                                       # met after steps of decoded tokens alone: one was in flight
+    eos = g0[k]
+
+    def run(keep, turn):
+        eng = LLMEngine(folder_a, dtype="float32", device="cpu", max_model_len=96, num_kvcache_blocks=24, keep_finished_cache=keep)
+        eng.eos_token_id = eos
+        rid = eng.add_request(ps[0], SamplingParams(max_new_tokens=20))
+        other = eng.add_request(ps[1], SamplingParams(max_new_tokens=40, ignore_eos=True))
+        while not eng.is_request_finished(rid):
+            eng.step()
+        assert eng.finish_reason(rid) == "eos" and eng.get_generated_tokens(rid) == g0[:k + 1]
+        seq = eng._sequences[rid]
+        if keep:
+            assert seq.cache is not None and seq.cache.num_tokens == len(seq)      # the step in flight stored the end token
+        eng.append_to_request(rid, turn, SamplingParams(max_new_tokens=4, ignore_eos=True))
+        steps = 0
+        while eng.has_unfinished_requests():
+            eng.step()
+            steps += 1
+            assert steps < 200, "the engine is wedged"
+        out = eng.get_generated_tokens(rid), eng.get_generated_tokens(other)
+        eng.remove_request(rid)
+        eng.remove_request(other)
+        eng.runner.manager.check()
+        assert eng.runner.manager.num_free_pages() == [24]
+        return out
+
+    for turn in ([], [9]):
+        kept, fresh = run(True, turn), run(False, turn)
+        assert kept == fresh
+        assert kept[0] == plain.greedy(ps[0] + g0[:k + 1] + turn, 4)
+        assert kept[1] == plain.greedy(ps[1], 40)
