@@ -93,13 +93,24 @@ class RequestCache:
         return [p for p in self.tables[group] if p >= 0]
 
 
+def window_pages(window: int, page_size: int, step_tokens: int = 1) -> int:
+    """Most pages that one request holds in a group whose layers read the last ``window`` keys only, while it runs
+    ``step_tokens`` tokens in a step: the keys that the step's first query reads and the step's own, which begin and
+    end anywhere in a page."""
+    return -(-(window - 1 + step_tokens) // page_size) + 1
+
+
 class CacheManager:
-    def __init__(self, cache_specs: Sequence[Optional[object]], page_size: int, num_pages: int, max_num_seqs: int):
+    def __init__(self, cache_specs: Sequence[Optional[object]], page_size: int, num_pages: int, max_num_seqs: int,
+                 max_step_tokens: Optional[int] = None):
         """``cache_specs[i]`` is the need of layer cache ``i`` (None = nothing).
-        Every page group gets a pool of ``num_pages`` pages of ``page_size`` tokens."""
+        Every page group gets a pool of ``num_pages`` pages of ``page_size`` tokens; a group with a window gets no
+        more than ``max_num_seqs`` requests can hold at once when none runs more than ``max_step_tokens`` tokens in a
+        step (if that is given)."""
         if page_size <= 0:
             raise ValueError("page_size must be positive")
         self.page_size = page_size
+        self.max_step_tokens = max_step_tokens
         self.page_groups: List[PageGroup] = []
         self.state_groups: List[StateGroup] = []
         self.location: Dict[int, tuple] = {}   # cache id -> ("paged"|"state", group index, index in group)
@@ -112,7 +123,8 @@ class CacheManager:
             if spec.paged:
                 grp = next((g for g in self.page_groups if g.spec == spec), None)
                 if grp is None:
-                    grp = PageGroup(len(self.page_groups), spec, [], page_size, PagePool(num_pages))
+                    grp = PageGroup(len(self.page_groups), spec, [], page_size,
+                                    PagePool(self.pages_of_group(spec, page_size, num_pages, max_num_seqs, max_step_tokens)))
                     self.page_groups.append(grp)
             else:
                 grp = next((g for g in self.state_groups if g.spec == spec), None)
@@ -123,6 +135,13 @@ class CacheManager:
             grp.cache_ids.append(cid)
         self.slots = SlotPool(max_num_seqs)
         self.requests: Dict[object, RequestCache] = {}
+
+    @staticmethod
+    def pages_of_group(spec: CacheKind, page_size: int, num_pages: int, max_num_seqs: int, max_step_tokens: Optional[int]) -> int:
+        """Pages in the pool of a group of kind ``spec`` when ``num_pages`` are offered to every group."""
+        if spec.window is None or max_step_tokens is None:
+            return num_pages
+        return max(1, min(num_pages, max_num_seqs * window_pages(spec.window, page_size, max_step_tokens)))
 
     # ---- admission -------------------------------------------------------
     def can_admit(self) -> bool:
@@ -226,10 +245,21 @@ class CacheManager:
         return [g.pool.num_free for g in self.page_groups]
 
     def max_tokens_per_request(self) -> int:
-        """Most tokens one request alone can hold (the smallest group decides)."""
-        if not self.page_groups:
-            return 1 << 62
-        return min(g.pool.num_pages for g in self.page_groups) * self.page_size
+        """Most tokens one request alone can reach (the smallest group decides).  A group with a window gives back the
+        pages that the window has passed, so with room for the window and one token more it sets no limit."""
+        limit = 1 << 62
+        for g in self.page_groups:
+            if g.spec.window is not None and g.pool.num_pages >= window_pages(g.spec.window, g.page_size):
+                continue
+            limit = min(limit, g.pool.num_pages * g.page_size)
+        return limit
+
+    def max_reservable(self, rc: RequestCache, n_tokens: int) -> int:
+        """The most tokens up to ``n_tokens`` for which ``rc`` could get pages now."""
+        for g in self.page_groups:
+            room = (len(rc.tables[g.index]) + g.pool.num_free) * g.page_size - rc.num_tokens
+            n_tokens = min(n_tokens, room)
+        return max(0, n_tokens)
 
     def check(self) -> None:
         """Invariant: every page is either free or in exactly one live table; same for slots."""

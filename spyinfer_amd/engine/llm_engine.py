@@ -14,7 +14,8 @@ import torch
 from ..config.engine_config import EngineConfig
 from ..sampling.sampler import Sampler, SamplingParams
 from .batch import StepEntry
-from .runner import ModelRunner, load_model
+from ..cache.manager import CacheManager
+from .runner import ModelRunner, load_model, resolve_dtype
 from .scheduler import Scheduler
 from .sequence import Sequence, SequenceStatus
 
@@ -41,22 +42,46 @@ class _Flight(NamedTuple):
 
 
 def pages_for_memory(free_bytes: int, config: EngineConfig, model) -> int:
-    """Pages of the cache pool when ``free_bytes`` of device memory are free (num_kvcache_blocks not given): the share
-    ``gpu_memory_utilization`` of what is left after the memory that captured decode steps will hold over the run
-    (``ModelRunner.graph_memory_bound``; nothing with enforce_eager), less a tenth for the activations of one full
-    step; never more than max_num_seqs requests of max_model_len tokens need."""
+    """Pages of the cache pool when ``free_bytes`` of device memory are free (num_kvcache_blocks not given).  From the
+    free memory go first the memory that captured decode steps will hold over the run
+    (``ModelRunner.graph_memory_bound``; nothing with enforce_eager); of the rest the share ``gpu_memory_utilization``
+    less a tenth (the activations of one full step, the library's workspace) is the cache's.  The slots of per-request
+    state are allocated whatever the pool's size, ``max_num_seqs`` of them in every layer cache that has any: they come
+    off first, and if they alone do not fit, that is an error here and not an allocation failure later.  Groups of
+    layers with a window get no more pages than their requests can hold (``CacheManager.pages_of_group``); what they
+    leave goes to the other groups.  Never more pages than max_num_seqs requests of max_model_len tokens need."""
     page = config.kvcache_block_size
-    per_page = ModelRunner.bytes_per_page(model, page, config.dtype)
-    if per_page == 0:
-        return 1
+    dtype = resolve_dtype(config.dtype)
+    specs = [s for s in model.cache_specs() if s is not None]
     blocks = -(-config.max_model_len // page)
     graphs = 0
     if not config.enforce_eager:
-        groups = len({s for s in model.cache_specs() if s is not None and s.paged})
+        groups = len({s for s in specs if s.paged})
         graphs = ModelRunner.graph_logits_bytes(config.max_num_seqs, model.vocab_size) \
             + ModelRunner.MAX_GRAPHS * ModelRunner.graph_metadata_bytes(config.max_num_seqs, groups, blocks)
-    pages = int(max(0, free_bytes - graphs) * config.gpu_memory_utilization * 0.9) // per_page
-    return max(1, min(pages, blocks * config.max_num_seqs))
+    budget = int(max(0, free_bytes - graphs) * config.gpu_memory_utilization * 0.9)
+    state = config.max_num_seqs * sum(s.page_bytes(page, dtype) for s in specs if not s.paged)
+    if state > budget:
+        raise ValueError("the per-request state of max_num_seqs = %d requests takes %d bytes of device memory; %d are at hand "
+                         "for the cache: lower max_num_seqs" % (config.max_num_seqs, state, budget))
+    budget -= state
+    per_kind = {}
+    for s in specs:
+        if s.paged:
+            per_kind[s] = per_kind.get(s, 0) + s.page_bytes(page, dtype)
+    if not per_kind:
+        return 1                                   # no layer keeps anything in pages
+    cap = blocks * config.max_num_seqs
+    pages = 0
+    while per_kind:
+        pages = min(cap, budget // sum(per_kind.values()))
+        full = [k for k in per_kind if CacheManager.pages_of_group(k, page, max(1, pages), config.max_num_seqs,
+                                                                   config.max_num_batched_tokens) < pages]
+        if not full:
+            break
+        for k in full:          # these groups take what their windows need; the others share what is left
+            budget -= per_kind.pop(k) * CacheManager.pages_of_group(k, page, pages, config.max_num_seqs, config.max_num_batched_tokens)
+    return max(1, pages)
 
 
 class LLMEngine:

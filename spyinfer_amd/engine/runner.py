@@ -74,7 +74,7 @@ class ModelRunner:
         self.act_dtype = resolve_dtype(dtype)
         self.device = torch.device(device)
         self.max_num_batched_tokens = max_num_batched_tokens
-        self.manager = CacheManager(model.cache_specs(), page_size, num_pages, max_num_seqs)
+        self.manager = CacheManager(model.cache_specs(), page_size, num_pages, max_num_seqs, max_num_batched_tokens)
         self.storage = CacheStorage(self.manager, self.act_dtype, self.device)
         self.steps_run = 0
         self.use_graphs = not enforce_eager
@@ -134,6 +134,8 @@ class ModelRunner:
             raise ValueError("a request would reach %d tokens, the model's positions end at %d"
                              % (batch.max_kv_len, self.model.max_positions))
         self.model.plan(batch)
+        # the parts have the last word: a part that reads the step from the host cannot be replayed from a recording
+        graphable = graphable and self.model.capturable(batch)
         self._pack(batch)
         if graphable:
             batch.graph_key()

@@ -138,7 +138,11 @@ class Scheduler:
                     continue
                 victim = max(self.running, key=lambda s: s.admit_order)
                 if victim is seq and len(self.running) == 1:
-                    raise RuntimeError("request %d cannot get pages although it runs alone; the pool is too small" % seq.id)
+                    # alone, nobody to take pages from: a smaller portion (a window gives pages back as it moves on)
+                    n = self.manager.max_reservable(seq.cache, n)
+                    if n == 0:
+                        raise RuntimeError("request %d cannot get pages although it runs alone; the pool is too small" % seq.id)
+                    break
                 for x in out:
                     if x.seq is victim:    # a victim scheduled earlier in this step leaves it and returns its budget
                         budget += x.num_tokens
@@ -168,7 +172,9 @@ class Scheduler:
             n = min(len(seq) - cache.num_tokens, budget, self.prefill_chunk)
             while not self.manager.can_reserve(cache, n) and self._reclaim_parked(spare=seq):
                 pass
-            if not self.manager.can_reserve(cache, n):
+            if not self.manager.can_reserve(cache, n) and not self.running and not out:
+                n = self.manager.max_reservable(cache, n)     # nothing runs that could end and free pages: a smaller portion
+            if n == 0 or not self.manager.can_reserve(cache, n):
                 if not kept:
                     self.manager.release(cache)
                 break

@@ -188,7 +188,7 @@ def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
 ROW_MAJOR_WEIGHTS = True
 #: most rows that a product takes straight from the tiled copy when the rows of the matrix are not kept
 TILED_ONLY_DIRECT_ROWS = 64
-_untile_scratch = {}          # device -> the tensor that restored rows go to outside graph capture
+_untile_scratch = {}          # device -> the newest tensor that restored rows go to
 
 
 def untile_weight(tiled: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -203,10 +203,12 @@ def untile_weight(tiled: torch.Tensor, out: Optional[torch.Tensor] = None) -> to
 
 class TiledOnly:
     """Stands where a product expects the matrix [N, K] of which only the tiled copy is kept: it has the matrix's
-    shape, dtype and device, and ``rows()`` restores the matrix for the library's product.  Outside graph capture the
-    rows go to one scratch tensor per device, which every matrix uses in turn and which holds them until the next
-    call (the steps run on one stream); inside a capture they go to a tensor of the graph's own pool."""
-    __slots__ = ("tiled",)
+    shape, dtype and device, and ``rows()`` restores the matrix for the library's product into a scratch tensor of the
+    device, which the matrices use in turn and which holds the rows until the next call (the steps run on one stream).
+    A matrix keeps the scratch tensor it was made with: if a larger matrix makes a larger one later, the older matrices
+    go on with theirs, so that the address a captured step has recorded for a matrix's rows stays good as long as the
+    matrix lives, and a captured step holds no restored rows of its own."""
+    __slots__ = ("tiled", "_buf")
 
     shape = property(lambda self: self.tiled.shape)
     dtype = property(lambda self: self.tiled.dtype)
@@ -221,19 +223,19 @@ class TiledOnly:
 
     def __init__(self, tiled: torch.Tensor):
         self.tiled = tiled
-        self._scratch()            # made now, while the weights are bound, so that the memory left for the cache counts it
-
-    def _scratch(self) -> torch.Tensor:
-        t = self.tiled
-        buf = _untile_scratch.get(t.device)
-        if buf is None or buf.numel() < t.numel():
-            buf = _untile_scratch[t.device] = torch.empty((t.numel(),), dtype=torch.bfloat16, device=t.device)
-        return buf[:t.numel()].view(t.shape)
+        # The device's scratch tensor is made large enough now, while the weights are bound, so that the memory left for
+        # the cache counts it; the matrix takes hold of it at its first use, when all matrices of its model exist and
+        # the tensor has the size of the largest.
+        buf = _untile_scratch.get(tiled.device)
+        if buf is None or buf.numel() < tiled.numel():
+            _untile_scratch[tiled.device] = torch.empty((tiled.numel(),), dtype=torch.bfloat16, device=tiled.device)
+        self._buf = None
 
     def rows(self) -> torch.Tensor:
-        if torch.cuda.is_current_stream_capturing():
-            return untile_weight(self.tiled)
-        return untile_weight(self.tiled, self._scratch())
+        t = self.tiled
+        if self._buf is None:
+            self._buf = _untile_scratch[t.device]
+        return untile_weight(t, self._buf[:t.numel()].view(t.shape))
 
 
 def weight_forms(w: torch.Tensor, keep_rows: bool = False):

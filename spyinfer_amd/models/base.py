@@ -32,7 +32,8 @@ class DecoderModel:
         self.embed, self.position, self.layers = embed, position, list(layers)
         self.final_norm, self.lm_head = final_norm, lm_head
         self.schedule = list(schedule) if schedule is not None else [LayerCall(i, i) for i in range(len(self.layers))]
-        n = dict(embed="model.embed_tokens", layers="model.layers.%d", final_norm="model.norm", lm_head="lm_head")
+        n = dict(embed="model.embed_tokens", position="model.position", layers="model.layers.%d", final_norm="model.norm",
+                 lm_head="lm_head")
         n.update(names or {})
         self.names = n
         self.max_positions = max_positions
@@ -46,7 +47,7 @@ class DecoderModel:
     def weight_specs(self) -> List[WeightSpec]:
         specs = list(self.embed.weight_specs(self.names["embed"]))
         if self.position is not None:
-            specs += self.position.weight_specs("model.position")
+            specs += self.position.weight_specs(self.names["position"])
         for i, layer in enumerate(self.layers):
             specs += layer.weight_specs(self.names["layers"] % i)
         specs += self.final_norm.weight_specs(self.names["final_norm"])
@@ -56,7 +57,7 @@ class DecoderModel:
     def bind(self, weights: Dict[str, torch.Tensor], device) -> None:
         self.embed.bind(self.names["embed"], weights)
         if self.position is not None:
-            self.position.bind("model.position", weights)
+            self.position.bind(self.names["position"], weights)
             self.position.prepare(device, self.max_positions)
         for i, layer in enumerate(self.layers):
             layer.bind(self.names["layers"] % i, weights)
@@ -88,6 +89,13 @@ class DecoderModel:
     def plan(self, batch) -> None:
         for call in self.schedule:
             self.layers[call.layer].mixer.plan(batch)
+
+    def capturable(self, batch) -> bool:
+        """Whether this step may be recorded in a HIP graph: every part that runs in it says so (``Part.capturable``)."""
+        parts = [self.embed, self.final_norm, self.lm_head] + [self.layers[i] for i in sorted({c.layer for c in self.schedule})]
+        if self.position is not None:
+            parts.append(self.position)
+        return all(p.capturable(batch) for p in parts)
 
     def forward(self, batch, storage, logits_out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Runs the batch's tokens through all calls of the run order; float32 logits [R, vocab]

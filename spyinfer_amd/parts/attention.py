@@ -138,6 +138,11 @@ class PagedAttention(Mixer):
         return batch.shared[note]
 
     # ---- step ------------------------------------------------------------
+    def capturable(self, batch):
+        # everything a step changes is read from the batch's device arrays; the one launch shape that follows the
+        # requests' lengths, the number of key parts, is in the graph's key (plan_attention_tiles)
+        return self.position is None or self.position.capturable(batch)
+
     def can_fold(self, batch):
         # (beyond 64 rows the products take their inputs in operand order only, which the attention hands over when every
         # entry is a single token)

@@ -29,6 +29,17 @@ class Part:
         """Take the tensors named by ``weight_specs(prefix)`` (already on the device).  A part that copies tensors into
         a form of its own (fused, reordered) may take them out of ``weights`` (``pop``), so that the originals are freed."""
 
+    def capturable(self, batch) -> bool:
+        """May this part's work on ``batch`` (a step of single tokens) be recorded once in a HIP graph and replayed for
+        later steps of the same shape?  A replay runs the recorded kernels with the recorded addresses and sizes; only
+        the CONTENTS of the batch's device arrays (token ids, positions, ``slot_ids``, block tables, what ``plan``
+        added) are those of the new step.  So True needs: everything that differs from step to step is read on the
+        device from those arrays (never from ``batch.entries``, ``batch.lens`` or other host values, which a replay
+        does not see), no copy to the host and no wait for the device, and launch shapes that depend only on the arrays'
+        lengths and on what ``plan`` put into the graph's key (``batch.add_graph_key``).  The default is False: a part
+        that does not say otherwise is always run kernel by kernel, and so is every step of a model that has one."""
+        return False
+
 
 class Norm(Part):
     """y = norm(x) over the hidden dimension."""

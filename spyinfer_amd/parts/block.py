@@ -25,6 +25,9 @@ class PreNormBlock(Block):
     def entry_norm(self):
         return self.norm1
 
+    def capturable(self, batch):
+        return all(part.capturable(batch) for part in (self.norm1, self.mixer, self.norm2, self.ffn))
+
     def forward(self, resid, pending, batch, cache, store=True, next_norm=None):
         act = batch.act_dtype
         ready = isinstance(pending, ops.ScaledInput)

@@ -21,6 +21,9 @@ class TokenEmbedding(Part):
     def bind(self, prefix, weights):
         self.weight = weights[prefix + ".weight"]
 
+    def capturable(self, batch):
+        return True
+
     def forward(self, ids):
         return ops.embedding(ids, self.weight)
 
@@ -53,6 +56,9 @@ class LMHead(Part):
             self.weight, self.weight_tiled = ops.weight_forms(self.tied_to.weight, keep_rows=True)   # the table's rows are looked up
         else:
             self.weight, self.weight_tiled = ops.weight_forms(weights.pop(prefix + ".weight"))
+
+    def capturable(self, batch):
+        return True
 
     def can_fold(self, batch):
         # without the matrix's rows the library's product would have them restored first (more bytes than the product

@@ -37,6 +37,9 @@ class GatedMLP(FeedForward):
             self.w_gate_up, self.w_gate_up_tiled = ops.weight_forms(self.w_gate_up)
         self.w_down, self.w_down_tiled = ops.weight_forms(weights.pop(prefix + ".down_proj.weight"))
 
+    def capturable(self, batch):
+        return True
+
     def can_fold(self, batch):
         return ops.fused_decode_ok(batch.T, batch.act_dtype, self.w_gate_up_tiled, self.w_down_tiled, max_rows=self.fold_rows)
 

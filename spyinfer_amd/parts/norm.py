@@ -22,6 +22,9 @@ class RMSNorm(Norm):
     def bind(self, prefix, weights):
         self.weight = weights[prefix + ".weight"]
 
+    def capturable(self, batch):
+        return True
+
     def add_norm(self, resid, delta, out_dtype, rows=None):
         return ops.add_rms_norm(resid, delta, self.weight, self.eps, out_dtype, rows)
 

@@ -33,5 +33,8 @@ class RotaryEmbedding(PositionEncoding):
         self.cos = torch.cos(ang).contiguous().to(device)
         self.sin = torch.sin(ang).contiguous().to(device)
 
+    def capturable(self, batch):
+        return True
+
     def rotary(self):
         return self.cos, self.sin, self.rotary_dim

@@ -25,7 +25,8 @@ from .safetensors_io import open_folder
 class WeightSpec:
     name: str
     shape: Tuple[int, ...]
-    #: "matrix" (projection / embedding), "norm" (scale vector centred on 1), "table" (integer table)
+    #: "matrix" (projection / embedding), "norm" (scale vector centred on 1), "bias" (vector centred on 0),
+    #: "table" (integer table); the role decides how the random-weights mode draws the tensor
     role: str = "matrix"
     #: names whose presence is tolerated but not read (a tied head stored again)
     optional: bool = False

@@ -3,8 +3,8 @@ from a configuration and a seed.
 
 Every tensor is drawn from its own stream keyed by (seed, tensor name), so the
 values do not depend on the order of tensors or on other tensors' shapes:
-matrices ~ N(0, matrix_std), norm scales ~ norm_mean + N(0, norm_std), integer
-tables uniform.  The folder is then read back by name like any other model.
+matrices ~ N(0, matrix_std), norm scales ~ norm_mean + N(0, norm_std), biases and
+other vectors centred on zero ~ N(0, bias_std), integer tables uniform.  The folder is then read back by name like any other model.
 The reference has no such mode.
 """
 from __future__ import annotations
@@ -20,6 +20,9 @@ from .loader import WeightSpec
 from .safetensors_io import write_file
 
 
+ROLES = ("matrix", "norm", "bias", "table")
+
+
 def _stream(seed: int, name: str) -> torch.Generator:
     digest = hashlib.sha256(("%d:%s" % (seed, name)).encode()).digest()
     g = torch.Generator(device="cpu")
@@ -29,16 +32,20 @@ def _stream(seed: int, name: str) -> torch.Generator:
 
 def random_tensors(specs: Iterable[WeightSpec], seed: int, dtype: torch.dtype = torch.bfloat16,
                    matrix_std: float = 0.02, norm_mean: float = 1.0, norm_std: float = 0.01,
-                   table_range: int = 2) -> Dict[str, torch.Tensor]:
+                   table_range: int = 2, bias_std: float = 0.02) -> Dict[str, torch.Tensor]:
     out = {}
     for s in specs:
         if s.optional:
             continue
+        if s.role not in ROLES:
+            raise ValueError("tensor %s has the role %r; known roles: %s" % (s.name, s.role, ", ".join(ROLES)))
         g = _stream(seed, s.name)
         if s.role == "table":
             out[s.name] = torch.randint(0, table_range, s.shape, generator=g, dtype=torch.int32)
         elif s.role == "norm":
             out[s.name] = (norm_mean + norm_std * torch.randn(s.shape, generator=g, dtype=torch.float32)).to(dtype)
+        elif s.role == "bias":
+            out[s.name] = (bias_std * torch.randn(s.shape, generator=g, dtype=torch.float32)).to(dtype)
         else:
             # big matrices are filled in row blocks to bound the float32 staging memory
             t = torch.empty(s.shape, dtype=dtype)
@@ -53,7 +60,8 @@ def random_tensors(specs: Iterable[WeightSpec], seed: int, dtype: torch.dtype = 
 
 
 def random_tensors_on_device(specs: Iterable[WeightSpec], seed: int, dtype: torch.dtype, device,
-                             matrix_std: float = 0.02, norm_mean: float = 1.0, norm_std: float = 0.0) -> Dict[str, torch.Tensor]:
+                             matrix_std: float = 0.02, norm_mean: float = 1.0, norm_std: float = 0.0,
+                             bias_std: float = 0.02) -> Dict[str, torch.Tensor]:
     """Random weights made on the device itself, for measurements at sizes whose files would take
     minutes to write and read.  Same distributions as ``random_tensors``, other values."""
     g = torch.Generator(device=device)
@@ -66,6 +74,8 @@ def random_tensors_on_device(specs: Iterable[WeightSpec], seed: int, dtype: torc
             out[s.name] = torch.randint(0, 2, s.shape, generator=g, dtype=torch.int32, device=device)
         elif s.role == "norm":
             out[s.name] = (norm_mean + norm_std * torch.randn(s.shape, generator=g, dtype=torch.float32, device=device)).to(dtype)
+        elif s.role == "bias":
+            out[s.name] = (bias_std * torch.randn(s.shape, generator=g, dtype=torch.float32, device=device)).to(dtype)
         else:
             t = torch.empty(s.shape, dtype=dtype, device=device)
             t.normal_(0.0, matrix_std, generator=g)

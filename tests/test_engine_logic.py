@@ -106,3 +106,62 @@ def test_a_step_metadata_fits_the_bound_used_for_captured_steps(folders, emu_ops
         model.plan(batch)
         _layout, total = batch.layout()
         assert 4 * total <= ModelRunner.graph_metadata_bytes(live, 1, runner.fixed_max_blocks)
+
+
+class _CacheNeeds:
+    """Stands for a model where only its cache needs and vocabulary are asked."""
+
+    def __init__(self, specs, vocab_size=100):
+        self._specs, self.vocab_size = list(specs), vocab_size
+
+    def cache_specs(self):
+        return self._specs
+
+
+def test_cache_pool_leaves_room_for_the_state_slots():
+    """Per-request state of fixed size is allocated for max_num_seqs requests in every layer cache that has any, whatever
+    the pool's size: it comes off the memory before the pages are counted, so that pages and slots together stay inside
+    what was handed in.  State that does not fit by itself is an error with the way out in it; a model that keeps state
+    only gets its one page after the same look at the memory."""
+    from spyinfer_amd.cache import FixedState, PagedKV
+    from spyinfer_amd.config.engine_config import EngineConfig
+    from spyinfer_amd.engine.llm_engine import pages_for_memory
+    kv, state = PagedKV(2, 64), FixedState((1 << 21,), "float32")              # 8 MB of state per request and layer
+    model = _CacheNeeds([kv, state, kv, state])
+    cfg = EngineConfig(max_num_seqs=16, max_model_len=1 << 20, kvcache_block_size=16, gpu_memory_utilization=1.0, enforce_eager=True)
+    free = 1 << 30
+    pages = pages_for_memory(free, cfg, model)
+    per_page = 2 * (2 * 2 * 64 * 16 * 2)
+    slots = 16 * 2 * (8 << 20)
+    assert pages == (int(free * 0.9) - slots) // per_page
+    assert pages * per_page + slots <= free
+    cfg.max_num_seqs = 512                                                    # the default: 8 GB of state
+    with pytest.raises(ValueError, match="lower max_num_seqs"):
+        pages_for_memory(free, cfg, model)
+    only_state = _CacheNeeds([state, None])
+    cfg.max_num_seqs = 16
+    assert pages_for_memory(free, cfg, only_state) == 1
+    cfg.max_num_seqs = 512
+    with pytest.raises(ValueError, match="lower max_num_seqs"):
+        pages_for_memory(free, cfg, only_state)
+
+
+def test_groups_with_a_window_take_what_their_windows_need_and_leave_the_rest():
+    from spyinfer_amd.cache import CacheManager, PagedKV
+    from spyinfer_amd.cache.manager import window_pages
+    from spyinfer_amd.config.engine_config import EngineConfig
+    from spyinfer_amd.engine.llm_engine import pages_for_memory
+    full, win = PagedKV(1, 64), PagedKV(1, 64, window=100)
+    cfg = EngineConfig(max_num_seqs=4, max_model_len=1 << 16, kvcache_block_size=16, gpu_memory_utilization=1.0, enforce_eager=True,
+                       max_num_batched_tokens=64)
+    per_page = 2 * 64 * 16 * 2
+    most = 4 * window_pages(100, 16, 64)                      # (99 + 64) / 16 rounded up, one more for a start inside a page
+    assert window_pages(100, 16, 64) == 12 and window_pages(100, 16) == 8
+    free = 64 << 20
+    budget = int(free * 0.9)
+    assert pages_for_memory(free, cfg, _CacheNeeds([full, win])) == (budget - most * per_page) // per_page
+    assert CacheManager.pages_of_group(win, 16, 10 ** 6, 4, 64) == most
+    assert pages_for_memory(free, cfg, _CacheNeeds([win, win])) >= most          # every group is full: what is offered is not taken
+    m = CacheManager([full, win], 16, 1000, 4, max_step_tokens=64)
+    assert [g.pool.num_pages for g in m.page_groups] == [1000, most]
+    assert [g.pool.num_pages for g in CacheManager([full, win], 16, 1000, 4).page_groups] == [1000, 1000]

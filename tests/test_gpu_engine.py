@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from tests import replay_cases as rc
-from tests.configs import INIT, TINY_A, TINY_B, TINY_C, TINY_D
+from tests.configs import INIT, TINY_A, TINY_B, TINY_C, TINY_D, TINY_E
 from tests.gpu_util import require_gpu
 from tests.plain.qwen3_plain import PlainQwen3
 
@@ -648,3 +648,202 @@ def test_toy_architecture_with_state(dtype, tmp_path):
         assert not np.allclose(outs["whole"][(first, 40)], outs["whole"][(first, 5)], atol=1e-3)
     finally:
         unregister_architecture("ToyRunningMeanLM")
+
+
+def _running_mean_on_device(base):
+    """The toy mixer again, written on the batch's device arrays alone (``slot_ids``, ``token_entry``, ``cu_q``): no
+    value of the step is read on the host, so its decode steps may be recorded in a graph, and it says so."""
+
+    class RunningMeanOnDevice(base):
+        def capturable(self, batch):
+            return True
+
+        def plan(self, batch):
+            pass
+
+        def forward(self, x, batch, cache, store=True):
+            H, T = self.hidden, x.shape[0]
+            xs = x.float()
+            entry = batch.token_entry.long()
+            start = batch.cu_q.long()[entry]                       # first token of every token's entry
+            slots = batch.slot_ids.long()
+            csum = torch.cumsum(xs, 0)
+            before = torch.where((start > 0)[:, None], csum[(start - 1).clamp(min=0)], torch.zeros_like(csum))
+            state = cache.state[slots[entry]]                      # [T, H + 1]: the sums and the count before this step
+            sums = csum - before + state[:, :H]
+            cnt = state[:, H] + (torch.arange(T, device=x.device) - start + 1).float()
+            if store:
+                last = batch.cu_q.long()[1:] - 1
+                cache.state.index_copy_(0, slots, torch.cat([sums[last], cnt[last][:, None]], 1))
+            return (sums / cnt[:, None] * self.gain.float()).to(x.dtype)
+
+    return RunningMeanOnDevice
+
+
+@pytest.mark.parametrize("kind", ["host", "device"])
+def test_toy_with_state_through_the_entry_point_with_graphs(kind, tmp_path):
+    """The toy architecture with a running state behind ``LLMEngine`` with graphs allowed (the default): seven requests
+    of different lengths, three at a time, so that slots and pages are handed out again.  The mixer that walks
+    ``batch.entries`` on the host does not call itself capturable, so no step of its model is recorded; the same
+    mixer written on the device arrays does, and its decode steps are replayed.  Greedy tokens equal the plain pass's
+    either way: a replay with the slots of the recorded step would mix the requests' states."""
+    from spyinfer_amd.config import register_architecture, unregister_architecture
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    from spyinfer_amd.weights import write_random_model
+    import spyinfer_amd.parts.base as parts_base
+    require_gpu()
+    ToyConfig, build = _toy_parts()
+    if kind == "device":
+        host_build = build
+
+        def build(cfg):
+            model = host_build(cfg)
+            for layer in model.layers:
+                if type(layer.mixer).__name__ == "RunningMean":
+                    layer.mixer.__class__ = _running_mean_on_device(type(layer.mixer))
+            return model
+    register_architecture("ToyRunningMeanLM", ToyConfig, build)
+    try:
+        cfg = dict(architectures=["ToyRunningMeanLM"], hidden_size=64, num_hidden_layers=3, vocab_size=97, intermediate_size=80)
+        folder = write_random_model(str(tmp_path / "toy"), cfg, 72, torch.bfloat16, **INIT)
+        lengths, news = [70, 9, 41, 3, 33, 18, 55], [12, 20, 9, 25, 14, 17, 11]
+        ps = prompts(97, lengths, 13)
+        eng = LLMEngine(folder, dtype="float32", max_model_len=128, num_kvcache_blocks=14, max_num_seqs=3, max_num_batched_tokens=48)
+        assert not eng.config.enforce_eager and eng.runner.use_graphs
+        slots_seen = []
+        admit = eng.runner.manager.admit
+        eng.runner.manager.admit = lambda rid: (lambda rc: (slots_seen.append(rc.slot), rc)[1])(admit(rid))
+        ids = [eng.add_request(p, SamplingParams(max_new_tokens=n, ignore_eos=True)) for p, n in zip(ps, news)]
+        while eng.has_unfinished_requests():
+            eng.step()
+        got = [eng.get_generated_tokens(i) for i in ids]
+        assert len(slots_seen) >= 7 and max(slots_seen.count(s) for s in set(slots_seen)) >= 2      # slots were used again
+        if kind == "host":
+            assert eng.runner.graph_replays == 0 and not eng.runner._graphs
+        else:
+            assert eng.runner.graph_replays >= 20 and eng.model.capturable(None)
+        for p, n, g in zip(ps, news, got):
+            toks = list(p)
+            for t in g:
+                logits = _plain_running_mean_lm(folder, toks)[-1]
+                best = int(torch.argmax(logits))
+                assert t == best or float(logits[best] - logits[t]) < 1e-3, "request of %d tokens leaves the plain pass" % len(p)
+                toks.append(t)
+            assert len(g) == n
+        eng.runner.manager.check()
+        assert eng.runner.manager.slots.num_free == 3
+        # a part that says nothing is taken to read the step on the host
+        assert parts_base.Part().capturable(None) is False
+    finally:
+        unregister_architecture("ToyRunningMeanLM")
+
+
+def test_matrices_in_tiles_only_in_a_captured_step_of_130_tokens():
+    """``weight_copies="tiled"`` with more single tokens in a step than the products take from the tiles (130 > 128): every
+    matrix's rows are restored ahead of its product into the device's one scratch tensor, inside a graph capture as
+    outside.  Logits equal those of the runner that keeps both forms, step by step, and the captured step holds no
+    restored rows of its own (one copy of every matrix would be 132 MB here)."""
+    from spyinfer_amd.config.registry import architecture_of
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.runner import ModelRunner, bind_weights
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.weights.random_init import random_tensors_on_device
+    dev = require_gpu()
+    V, R = 8192, 130
+    raw = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_act="silu", num_hidden_layers=4, hidden_size=1024,
+               num_attention_heads=8, num_key_value_heads=2, head_dim=128, intermediate_size=4096, vocab_size=V,
+               rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=256)
+    arch = architecture_of(raw)
+    runners = {}
+    for copies in ("both", "tiled"):
+        model = arch.build(arch.config_cls.from_dict(raw))
+        bind_weights(model, random_tensors_on_device(model.weight_specs(), 5, torch.bfloat16, dev, matrix_std=0.04), dev, copies)
+        runners[copies] = ModelRunner(model, "bfloat16", dev, 16, 2 * R, R, enforce_eager=copies == "both", max_model_len=32)
+    tiled = runners["tiled"]
+    assert isinstance(tiled.model.layers[0].ffn.w_gate_up, ops.TiledOnly) and isinstance(tiled.model.lm_head.weight, ops.TiledOnly)
+    one_copy_each = sum(m.tiled.numel() * 2 for layer in tiled.model.layers
+                        for m in (layer.mixer.w_qkv, layer.mixer.w_o, layer.ffn.w_gate_up, layer.ffn.w_down)) + tiled.model.lm_head.weight.tiled.numel() * 2
+    assert one_copy_each > (120 << 20)
+    g = torch.Generator().manual_seed(2)
+    caches = {k: [r.manager.admit(i) for i in range(R)] for k, r in runners.items()}
+    base = None
+    for step in range(6):
+        toks = torch.randint(0, V, (R,), generator=g).tolist()
+        out = {}
+        for k, r in runners.items():
+            for c in caches[k]:
+                r.manager.reserve(c, 1)
+            out[k] = r.step([StepEntry(c, [t], [0]) for c, t in zip(caches[k], toks)]).clone()
+        assert torch.allclose(out["tiled"], out["both"], atol=8e-2, rtol=2e-2), "step %d: %g" % (step, (out["tiled"] - out["both"]).abs().max())
+        if step == 0:
+            torch.cuda.synchronize()
+            base = torch.cuda.memory_reserved(dev)           # after the eager step: the scratch tensor and the activations exist
+    torch.cuda.synchronize()
+    assert tiled.graph_replays >= 4 and len(tiled._graphs) == 1
+    grown = torch.cuda.memory_reserved(dev) - base
+    # what does grow: the library's workspace of 76 MB, which a first product inside a capture takes from the graph's pool,
+    # the logits tensor and a segment for the activations (94 MB were measured)
+    assert grown <= (112 << 20), "the captured step holds %d MB more (one restored copy of every matrix: %d MB)" % (
+        grown >> 20, one_copy_each >> 20)
+
+
+LONG_N, SHORT_N, LONG_STEPS = 4200, 37, 40
+
+
+@pytest.fixture(scope="module")
+def long_model(tmp_path_factory):
+    """Config E with 4608 positions and doubled q and k norm weights (single far keys carry most of a softmax's weight),
+    a sequence of 4240 tokens and one of 77, and the plain pass's logits of both."""
+    from safetensors.torch import load_file
+    from spyinfer_amd.weights import write_file, write_random_model
+    raw = dict(TINY_E, max_position_embeddings=4608)
+    folder = write_random_model(str(tmp_path_factory.mktemp("long")), raw, 91, torch.bfloat16, **INIT)
+    path = os.path.join(folder, "model.safetensors")
+    w = {k: v.clone() for k, v in load_file(path).items()}
+    for k in w:
+        if k.endswith("q_norm.weight") or k.endswith("k_norm.weight"):
+            w[k] = (w[k].float() * 2.0).to(torch.bfloat16)
+    write_file(path, w)
+    g = torch.Generator().manual_seed(8)
+    seqs = [torch.randint(0, raw["vocab_size"], (n + LONG_STEPS,), generator=g).tolist() for n in (LONG_N, SHORT_N)]
+    plain = PlainQwen3(folder)
+    ref = [plain.forward(s) for s in seqs]
+    # the construction does what it says: without the keys 1280..1535 (one of the 16 parts) the plain logits move visibly
+    cut = plain.forward(seqs[0][:1280] + seqs[0][1536:])
+    assert (cut[-LONG_STEPS:] - ref[0][-LONG_STEPS:]).abs().max() > 0.5
+    return folder, seqs, ref
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_request_of_4200_tokens_decodes_under_graphs(dtype, long_model):
+    """One long request beside a short one, decode steps recorded and replayed: block tables of the fixed width that
+    4608 positions need (288 pages), the long request's keys in 16 parts.  A part of the keys that is lost, read through
+    a wrong page or merged wrongly moves the logits far beyond the tolerance (the fixture asserts it on the plain pass).
+    Logits of every decode step against the plain pass of the whole sequences."""
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.runner import ModelRunner, load_model
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    folder, seqs, ref = long_model
+    long_n, short_n, steps = LONG_N, SHORT_N, LONG_STEPS
+    runner = ModelRunner(load_model(folder, dtype, dev), dtype, dev, 16, 300, 2, enforce_eager=False, max_model_len=4608)
+    assert runner.fixed_max_blocks == 288
+    caches = [runner.manager.admit(i) for i in range(2)]
+    for lo in range(0, long_n, 2048):                               # the long prompt in portions
+        n = min(2048, long_n - lo)
+        runner.manager.reserve(caches[0], n)
+        runner.step([StepEntry(caches[0], seqs[0][lo:lo + n], [])])
+    runner.manager.reserve(caches[1], short_n)
+    runner.step([StepEntry(caches[1], seqs[1][:short_n], [])])
+    tol = dict(atol=1e-4, rtol=1e-4) if dtype == "float32" else dict(atol=0.28, rtol=0.02)
+    parts = set()
+    for i in range(steps):
+        for c in caches:
+            runner.manager.reserve(c, 1)
+        got = runner.step([StepEntry(caches[0], [seqs[0][long_n + i]], [0]), StepEntry(caches[1], [seqs[1][short_n + i]], [0])]).cpu()
+        parts.add(ops.key_parts_for(long_n + i + 1))
+        want = torch.stack([ref[0][long_n + i], ref[1][short_n + i]])
+        assert torch.allclose(got, want, **tol), "decode step %d (%s): off by %g / %g" % (
+            i, "replayed" if i >= 2 else "eager or captured", (got[0] - want[0]).abs().max(), (got[1] - want[1]).abs().max())
+    assert parts == {16} and runner.graph_replays >= steps - 2

@@ -200,3 +200,39 @@ def test_a_parked_cache_gives_its_slot_to_a_new_request():
     b = seq(1, 3)
     s.add_sequence(b)
     assert [(x.seq.id) for x in run_step(m, s)] == [1] and a.cache is None
+
+
+def test_a_model_with_windows_only_runs_requests_longer_than_its_pool():
+    """Every paged layer reads the last 10 keys only, and the window gives back the pages it has passed: a pool of 6
+    pages of 4 tokens (24 tokens) runs a prompt of 60 tokens to 90, in portions as large as the free pages allow, and a
+    second request beside it."""
+    m = CacheManager([PagedKV(1, 8, window=10), PagedKV(1, 8, window=10)], page_size=4, num_pages=6, max_num_seqs=2)
+    assert m.max_tokens_per_request() > 1 << 40
+    s = Scheduler(m, 64, 2, 128)
+    a = seq(0, 60, max_new_tokens=30, ignore_eos=True)
+    s.add_sequence(a)                                        # not refused, though 60 > 24
+    portions = []
+    while a.num_generated < 30:
+        out = run_step(m, s)
+        assert out, "the request is stuck"
+        portions.append(out[0].num_tokens)
+        assert len(a.cache.pages_held(0)) <= 6
+    assert len(a) == 90 and max(portions) <= 24 and portions.count(1) >= 29
+    s.finish(a, "max_new_tokens")
+    assert m.num_free_pages() == [6]
+    # two at once: the second waits for pages, then runs; nothing is preempted for good
+    b, c = seq(1, 30, max_new_tokens=8, ignore_eos=True), seq(2, 17, max_new_tokens=8, ignore_eos=True)
+    s.add_sequence(b); s.add_sequence(c)
+    for _ in range(200):
+        if not s.has_unfinished():
+            break
+        for sc in run_step(m, s):
+            if sc.seq.num_generated >= 8:
+                s.finish(sc.seq, "max_new_tokens")
+    assert not s.has_unfinished() and len(b) == 38 and len(c) == 25
+    m.check()
+    # a window that the pool cannot hold is a limit like any other
+    small = CacheManager([PagedKV(1, 8, window=40)], page_size=4, num_pages=6, max_num_seqs=2)
+    assert small.max_tokens_per_request() == 24
+    with pytest.raises(ValueError, match="cache pool"):
+        Scheduler(small, 64, 2, 128).add_sequence(seq(3, 60))

@@ -124,3 +124,43 @@ def test_broken_files(tmp_path):
     p.write_bytes(struct.pack("<Q", len(hdr)) + hdr + b"\0" * 8)
     with pytest.raises(SafetensorsError, match="needs 16"):
         SafetensorsFile(str(p))
+
+
+def test_roles_of_the_random_weights_mode():
+    """A vector centred on zero (a bias) has a role of its own: drawn as a norm's scale it would sit around one."""
+    from spyinfer_amd.weights import WeightSpec
+    specs = [WeightSpec("m", (64, 32)), WeightSpec("n", (4096,), "norm"), WeightSpec("b", (4096,), "bias"), WeightSpec("t", (9,), "table")]
+    w = random_tensors(specs, 3, torch.float32, bias_std=0.05)
+    assert abs(float(w["n"].mean()) - 1.0) < 0.01 and abs(float(w["b"].mean())) < 0.01 and 0.04 < float(w["b"].std()) < 0.06
+    assert w["t"].dtype == torch.int32 and w["m"].shape == (64, 32)
+    with pytest.raises(ValueError, match="known roles"):
+        random_tensors([WeightSpec("x", (3,), "offset")], 3)
+
+
+def test_every_part_of_a_model_is_named_through_its_names():
+    """The position encoding's tensors lie under the prefix that the model's ``names`` give, like the other parts'."""
+    from spyinfer_amd.models import DecoderModel
+    from spyinfer_amd.parts import GatedMLP, LMHead, PagedAttention, PreNormBlock, RMSNorm, TokenEmbedding
+    from spyinfer_amd.parts.base import PositionEncoding
+    from spyinfer_amd.weights import WeightSpec
+
+    class Table(PositionEncoding):
+        def weight_specs(self, prefix):
+            return [WeightSpec(prefix + ".table", (32, 64)), WeightSpec(prefix + ".offset", (64,), "bias")]
+
+        def bind(self, prefix, weights):
+            self.table, self.offset = weights[prefix + ".table"], weights[prefix + ".offset"]
+
+    emb = TokenEmbedding(50, 64)
+    block = PreNormBlock(RMSNorm(64, 1e-6), PagedAttention(64, 2, 1, 32, None), RMSNorm(64, 1e-6), GatedMLP(64, 96))
+    kw = dict(config=None, embed=emb, layers=[block], final_norm=RMSNorm(64, 1e-6), lm_head=LMHead(50, 64, tied_to=emb))
+    default = DecoderModel(position=Table(), **kw)
+    assert {s.name for s in default.weight_specs() if "table" in s.name or "offset" in s.name} == {"model.position.table", "model.position.offset"}
+    pos = Table()
+    named = DecoderModel(position=pos, names=dict(position="wpe", layers="h.%d", embed="wte"), **kw)
+    names = {s.name for s in named.weight_specs()}
+    assert {"wpe.table", "wpe.offset", "wte.weight", "h.0.mlp.down_proj.weight", "model.norm.weight"} <= names
+    assert not any(n.startswith("model.position") for n in names)
+    w = random_tensors([s for s in named.weight_specs() if s.name.startswith("wpe")], 1, torch.float32)
+    pos.bind("wpe", w)
+    assert pos.table.shape == (32, 64) and abs(float(pos.offset.mean())) < 0.02
