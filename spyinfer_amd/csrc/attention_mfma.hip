@@ -24,8 +24,8 @@
 // per-head RMS norm costs two lane exchanges and the rotation none.  The entry's new key is prepared the same way
 // by every lane for its own 8-value pieces, put in the place of the cache's row in the one block and round that reach
 // its position, and stored to the cache from there; so is the new value.  No other block reads that position.
-// (Letting the block that finishes last merge, found with a counter and device-scope fences, was
-// measured slower: 26 us against 17 us at 8 requests, because each fence writes back and invalidates L2.)
+// (The merge by the last block uses no fence: with device-scope fences on both sides, each of which writes back and
+// invalidates the whole L2, it took 26 us against 17 us at 8 requests.  What orders it instead is said at the site.)
 #include "common.h"
 #include "attention_merge.h"
 #include <math.h>
@@ -132,14 +132,6 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     constexpr int KK = DMAX / 32;   // 32-wide chunks of the head dim for Q.K
     constexpr int DT = DMAX / 16;   // 16-row tiles of the head dim for P.V
     extern __shared__ float lds[];   // the waves' O, m, l: AW (head sizes up to 128) or AW - 1 times (DT * 4 + 2) * 64 floats
-#ifdef AM_TIMING
-    long long tstamp[8];
-    int nstamp = 0;
-#define AM_STAMP(dep) { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); tstamp[nstamp++] = clock64() + ((dep) & 0); }
-    AM_STAMP(0)
-#else
-#define AM_STAMP(dep)
-#endif
     const int tile = blockIdx.x, hk = blockIdx.y, sp = blockIdx.z;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: loops over it stay scalar
     // a key's page and its place inside: a shift and a mask for pages that are a power of two (log2p >= 0), instead of
@@ -185,7 +177,6 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     const int per = (nblk + splits - 1) / splits;
     const int b_begin = sp * per, b_end = min(nblk, b_begin + per);
 
-    AM_STAMP(nblk)      // 1: the entry's description and the query row are there
     f32x4_t acc[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -279,7 +270,6 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         }
         __builtin_amdgcn_sched_barrier(0);
     }
-    AM_STAMP(kpage)     // 3: pages looked up
     if (b_begin + wave < b_end) AM_LOAD_K(b_begin + wave, kpage)
     if constexpr (FUSED) {
         __builtin_amdgcn_sched_barrier(0);
@@ -292,7 +282,6 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
             if (new_page < 0 || new_page >= num_pages) has_new = false;   // no page: nothing to store or to use
         }
     }
-    AM_STAMP(kpage)     // 4: first keys there
     // One block of 32 keys.  LAST: the wave's last block, which alone can hold keys beyond the request's and the step's
     // new key, and after which no keys are asked for; the blocks before it have no condition around their loads.
     auto block = [&](const int b, auto last_block) {
@@ -403,7 +392,6 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     }
 #undef AM_LOOKUP
 #undef AM_LOAD_K
-    AM_STAMP(0)         // 5: key blocks done
     // the four lanes of a row hold partial sums of l
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
@@ -478,12 +466,6 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         for (int i = 0; i < MINE; ++i) mo[i] = acc[i];
     }
 
-    AM_STAMP(0)         // 6: waves merged
-#ifdef AM_TIMING
-    if (tile == 0 && hk == 0 && sp == 0 && threadIdx.x == 0 && ws) {
-        for (int i = 0; i < nstamp; ++i) reinterpret_cast<long long*>(ws)[i] = tstamp[i];
-    }
-#endif
     if (splits == 1) {
         if (!row_ok) return;
         const float inv = l > 0.f ? 1.0f / l : 0.f;
@@ -507,6 +489,17 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         // The parts of a (tile, kv head) are merged here, by the block that finishes last (a counter per tile and head,
         // left at zero), instead of by a second kernel.  The dies' L2s are not coherent inside a kernel: the parts go
         // through the caches (stores of system scope, waited for before the block counts itself) and are read past them.
+        // ORDER.  No release/acquire pair states that the parts are visible before the count: the HIP memory model would
+        // ask for a release on the counter's increment and an acquire behind it, which this compiler turns into a
+        // write-back and an invalidation of the whole L2 (the 9 us above).  What stands in for them is how gfx950 executes
+        // these instructions: (1) an atomic store of system scope is a write-through store (sc0 sc1) that has reached
+        // memory, past every L2, when the wave's vmcnt has counted it, and s_waitcnt(0) waits for that; (2) the barrier
+        // behind it puts every wave's wait before thread 0's increment, and the increment is an atomic of device scope,
+        // which all dies execute at one place beyond their L2s (it could not count across dies otherwise), so no block
+        // sees the count before the stores it follows have arrived; (3) the last block's loads of
+        // system scope miss L1 and L2 (sc0 sc1) and so read what memory holds, and they are issued after the barrier
+        // that follows the increment's return.  Do not weaken any of the three (ordinary stores, no wait, ordinary
+        // loads), and do not "strengthen" the atomics to release/acquire without measuring: it is correct and slow.
         // A part lies lane for lane: O[(dt 4 + i)][64 lanes], then m[16], l[16].
         __shared__ unsigned am_last;
 #pragma unroll

@@ -27,12 +27,7 @@
 
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 
-#ifndef GD_HALVES
-#define GD_HALVES 1       // 0: blocks of three halves of column tiles are never taken (for measurements)
-#endif
-#ifndef GD_WAVES_GATED
-#define GD_WAVES_GATED 4
-#endif
+constexpr int GD_WAVES_GATED = 4;     // waves of a block of the gated product with a pair of column tiles per block
 
 // H3: a block has three halves of column tiles (24 columns) instead of one tile: tile t whole and the lower half of
 // tile t + 1, or the upper half of tile t and tile t + 1 whole, in turn.  For a matrix of one and a half column tiles per
@@ -348,7 +343,7 @@ static bool gd_launch2(const GdArgs& a) {
     bool halves_rows = false;
     if constexpr (EPI == EPI_STORE && SCALED && XT && !OT && sizeof(TC) == 2) {
         const int cus_ = gd_compute_units();
-        halves_rows = GD_HALVES && a.N % 48 == 0 && (a.N / 24) % cus_ == 0 && (a.N / 16) % cus_ != 0;
+        halves_rows = a.N % 48 == 0 && (a.N / 24) % cus_ == 0 && (a.N / 16) % cus_ != 0;
     }
     // beyond four row tiles: blocks of eight waves (a wave per row tile runs the epilogue), one column tile; built for
     // what a decode step has: inputs in operand order, the residual product of a plain input with its output in operand
@@ -359,7 +354,7 @@ static bool gd_launch2(const GdArgs& a) {
         bool halves = false;
         if constexpr (EPI == EPI_STORE && SCALED && XT && !OT && sizeof(TC) == 2) {
             const int cus = gd_compute_units();
-            const bool uneven = GD_HALVES && (a.N / 16) % cus != 0;
+            const bool uneven = (a.N / 16) % cus != 0;
             if (uneven && a.N % 48 == 0 && (a.N / 24) % cus == 0) {
                 gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT, 3><<<a.N / 24, W * 64, 0, a.st>>>(GD_ARGS);
                 halves = true;

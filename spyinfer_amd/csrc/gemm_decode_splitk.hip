@@ -181,6 +181,11 @@ __global__ __launch_bounds__(GW * 64, 1) void gemm_decode_splitk_kernel(
 #pragma unroll
             for (int i = 0; i < 4; ++i) __hip_atomic_store(mine + (p * 4 + i) * 64, v[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         }
+        // ORDER (as at the attention's merge of key parts): no release/acquire pair, which this compiler turns into a
+        // write-back and invalidation of the whole L2 (30 us a call).  Instead: the stores of system scope write through
+        // every cache and have reached memory when vmcnt has counted them, which this wait is for; the barrier puts all
+        // waves' waits before thread 0's increment, an atomic of device scope that all dies execute at one place; the last block's loads of system scope
+        // read past the caches, after the barrier behind the increment.  Ordinary stores or loads here would be wrong.
         __builtin_amdgcn_s_waitcnt(0);                     // the stores have arrived before the block counts itself done
     }
     __syncthreads();

@@ -23,8 +23,7 @@ CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
 LIB_NAME = "libspyinfer_hip.so"
 ARCH = "gfx950"
 # -packed-fp32-ops off: hipcc forms packed fp32 instructions on its own from float code otherwise
-# SPYINFER_HIPCC_EXTRA: further flags for tuning builds (e.g. -D switches); part of the library's digest
-HIPCC_FLAGS = os.environ.get("SPYINFER_HIPCC_EXTRA", "").split() + ["-O3", "-std=c++17", "-fPIC", "--offload-arch=" + ARCH, "-Xclang", "-target-feature", "-Xclang",
+HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", "--offload-arch=" + ARCH, "-Xclang", "-target-feature", "-Xclang",
                "-packed-fp32-ops", "-Wno-unused-result", "-ffp-contract=fast"]
 
 _lock = threading.Lock()

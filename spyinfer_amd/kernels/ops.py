@@ -76,7 +76,14 @@ class _Hip:
     def call(self, name, *args):
         rc = getattr(self.lib, name)(*args)
         if rc != 0:
-            raise KernelError("%s: %s" % (name, self.lib.spy_last_error().decode()))
+            message = self.lib.spy_last_error().decode()
+            # a call that failed may have left counters of the device's workspace away from zero (a launch that went out
+            # in part); with such a counter no block of a later call would ever count itself last, and that call would
+            # write nothing and report nothing.  So the workspaces start from zero again.
+            if not torch.cuda.is_current_stream_capturing():
+                for ws in _decode_workspaces.values():
+                    ws.zero_()
+            raise KernelError("%s: %s" % (name, message))
 
     @staticmethod
     def stream():
@@ -153,10 +160,6 @@ SKINNY_MAX_ROWS_F32_OUT = 64
 _LIBRARY_F32_OUT = True      # torch.mm(..., out_dtype=float32) exists in this torch (float32 sums kept in the result)
 
 
-#: Keep a second copy of every bfloat16 weight matrix in MFMA tile order for the decode kernel (its loads are
-#: then whole cache lines).  Costs the weights' size again in device memory; the row-major copy stays for the
-#: library product of prefill.
-TILED_WEIGHTS = True
 #: Most rows that the decode products (``decode_linear`` and its kin) take.
 FUSED_DECODE_MAX_ROWS = 128
 
@@ -172,9 +175,9 @@ def default_fold_rows(weight_elements: int) -> int:
 
 def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
     """``w [N, K]`` in the order the decode kernel reads it: [K/128 chunks][N/16 tiles][4 steps][g = 4][r = 16][8], the
-    values of lane 16 g + r being w[16 tile + r][128 chunk + 32 step + 8 g ..].  None if the copy is switched off or
-    the shape or dtype does not allow it (then the kernel for row-major matrices stands)."""
-    if not TILED_WEIGHTS or not w.is_cuda or w.dtype != torch.bfloat16 or w.dim() != 2:
+    values of lane 16 g + r being w[16 tile + r][128 chunk + 32 step + 8 g ..].  None if the shape or dtype
+    does not allow it (then the kernel for row-major matrices stands)."""
+    if not w.is_cuda or w.dtype != torch.bfloat16 or w.dim() != 2:
         return None
     N, K = w.shape
     if N % 16 or K % 128 or N * 256 + 8192 >= (1 << 32):
@@ -367,6 +370,8 @@ class ScaledInput:
         self.xw, self.ss_parts, self.eps, self.norm = xw, ss_parts, float(eps), norm
 
 
+# Two switches that the tests flip, to hold the folded decode steps against the same steps with norm kernels of their own,
+# and the hand-over in operand order against the row-major one; nothing in the engine sets them.
 #: False switches the folded decode products off (every norm then runs as a kernel of its own).
 FUSED_DECODE = True
 #: False: the decode products hand their outputs to each other row-major
@@ -389,9 +394,15 @@ def fused_decode_ok(rows: int, act_dtype, *tiled_weights, max_rows: Optional[int
                for t in tiled_weights)
 
 
+def folded_products_take(prepared, rows: int) -> bool:
+    """Whether the folded decode products can start from what a block has at hand for ``rows`` rows: ``prepared`` is the
+    ``ScaledInput`` that the part before made for the block's first norm, or None (a norm kernel then makes ordinary
+    [M, K] rows).  Up to 64 rows they take either; beyond, only the operand order that they write for each other."""
+    return rows <= 64 or (isinstance(prepared, ScaledInput) and isinstance(prepared.xw, OperandRows))
+
+
 _decode_workspaces = {}
 ATTENTION_COUNTERS = 4096          # counters at the start of the device's workspace (16 KB)
-MERGE_IN_KERNEL = True             # False: the attention's key parts are merged by a second kernel (for measurements)
 
 
 def decode_workspace(device) -> Optional[torch.Tensor]:
@@ -407,6 +418,13 @@ def decode_workspace(device) -> Optional[torch.Tensor]:
         ws = torch.zeros((hip().lib.spy_gemm_decode_workspace(),), dtype=torch.uint8, device=torch.device("cuda", index))
         _decode_workspaces[index] = ws
     return ws
+
+
+def workspace_counters_clean(device) -> bool:
+    """True if every counter of the device's workspace is at zero, as each call leaves them (a check for tests and for
+    debugging; it waits for the device)."""
+    ws = decode_workspace(device)
+    return ws is None or not bool(ws[:4 * ATTENTION_COUNTERS].any())
 
 
 def _gemm_decode(x, tiled: torch.Tensor, epi: int, n_out: int, out, resid, xw_out, w_next, ss_out) -> None:
@@ -581,7 +599,7 @@ class AttentionMeta:
         self.fixed_shape = fixed_shape
 
 
-MFMA_ATTENTION = True      # False forces the plain kernel for bfloat16 too (used by tests)
+MFMA_ATTENTION = True      # False forces the plain kernel for bfloat16 too (the kernel tests flip it; nothing else does)
 DECODE_MAX_SPLITS = 16      # most key parts of a tile (the merge kernel's time grows with them)
 DECODE_KEYS_PER_SPLIT = 256  # a part wants this many keys at least (measured at 1100 keys, 1 to 4 requests: 4-8 parts best)
 
@@ -633,13 +651,11 @@ class RawQKV:
         self.qkv, self.q_norm_w, self.k_norm_w, self.eps, self.cos, self.sin, self.store = qkv, q_norm_w, k_norm_w, eps, cos, sin, store
 
 
-FUSED_ATTENTION = True     # False: the norm, rotation and store always run as a kernel of their own
-
 
 def fused_attention_ok(dtype, meta: AttentionMeta, n_q: int, n_kv: int, d: int, page_size: int, rotary_dim: int, q_norm_w, k_norm_w) -> bool:
     """True if this step's attention may take the raw product (``RawQKV``): every entry a single token, bfloat16,
     head_dim 64, 128 or 256 rotated whole or not at all, 16-row tiles built for this group size."""
-    if not FUSED_ATTENTION or not mfma_attention_ok(dtype, d, page_size):
+    if not mfma_attention_ok(dtype, d, page_size):
         return False
     if meta.T != meta.S or meta.max_q_len != 1 or meta.tiles is None or meta.tiles_group != n_q // n_kv or n_q // n_kv > 16:
         return False
@@ -729,7 +745,7 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
                                                                ctypes.c_int(splits))
             ws = torch.empty((max(1, ws_floats),), dtype=torch.float32, device=q.device)
             # with counters the last block of a (tile, kv head) merges its parts; without, a second kernel does
-            counters = decode_workspace(q.device) if splits > 1 and MERGE_IN_KERNEL else None
+            counters = decode_workspace(q.device) if splits > 1 else None
             if raw is not None:
                 wcode = _code(raw.q_norm_w, "head norm weight") if raw.q_norm_w is not None else F32
                 fused = (_ptr(raw.qkv), _ptr(raw.q_norm_w), _ptr(raw.k_norm_w), ctypes.c_int(wcode), ctypes.c_float(raw.eps),

@@ -31,9 +31,16 @@ class PreNormBlock(Block):
     def forward(self, resid, pending, batch, cache, store=True, next_norm=None):
         act = batch.act_dtype
         ready = isinstance(pending, ops.ScaledInput)
-        if self.norm2.foldable(act) is not None and self.mixer.can_fold(batch) and self.ffn.can_fold(batch):
+        mine = ready and pending.norm is self.norm1
+        fold = self.norm2.foldable(act) is not None and self.mixer.can_fold(batch) and self.ffn.can_fold(batch)
+        if fold and not ops.folded_products_take(pending if mine else None, batch.T):
+            # beyond 64 rows the folded products take an input in operand order only, which only the part before this
+            # block can have prepared (another kind of block, a position encoding on the embeddings, parts that fold up
+            # to fewer rows may not have): the plain path then
+            fold = False
+        if fold:
             # few rows: the sums go into the stream inside the products, the norms' scales into the products after them
-            if ready and pending.norm is self.norm1:
+            if mine:
                 n1 = pending
             else:
                 n1 = self.norm1.add_norm(resid, None if ready else pending, act)

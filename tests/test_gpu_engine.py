@@ -467,6 +467,39 @@ def test_folded_decode_steps_of_many_requests(tmp_path_factory, requests):
     assert torch.allclose(runs[0][-1], ref, **TOL["bfloat16"]), (runs[0][-1] - ref).abs().max()
 
 
+def test_layers_that_fold_up_to_different_rows(tmp_path_factory):
+    """A run order in which a block that folds follows one that does not (parts built to fold up to fewer rows): at
+    100 single tokens the second block gets an ordinary addend, not the prepared input in operand order that the
+    folded products need beyond 64 rows, and takes the plain path instead of asking a product for what it refuses."""
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.runner import ModelRunner, load_model
+    from spyinfer_amd.weights import write_random_model
+    dev = require_gpu()
+    folder = write_random_model(str(tmp_path_factory.mktemp("eng_mixfold")), TINY_D, 65, torch.bfloat16, **INIT)
+    plain = PlainQwen3(folder)
+    model = load_model(folder, "bfloat16", dev)
+    model.layers[0].mixer.fold_rows = model.layers[0].ffn.fold_rows = 48
+    model.layers[2].ffn.fold_rows = 48                   # and a block whose mixer folds and whose feed-forward does not
+    requests = 100
+    ps = prompts(400, [3 + (5 * i) % 19 for i in range(requests)], 6)
+    runner = ModelRunner(model, "bfloat16", dev, 16, 4 * requests, requests, enforce_eager=True, max_model_len=64)
+    caches = [runner.manager.admit(i) for i in range(requests)]
+    for c, p in zip(caches, ps):
+        runner.manager.reserve(c, len(p))
+    runner.step([StepEntry(c, p, []) for c, p in zip(caches, ps)])
+    g = torch.Generator().manual_seed(7)
+    seqs = [list(p) for p in ps]
+    for i in range(3):
+        toks = torch.randint(0, 400, (requests,), generator=g).tolist()
+        for c in caches:
+            runner.manager.reserve(c, 1)
+        for q, t in zip(seqs, toks):
+            q.append(t)
+        got = runner.step([StepEntry(c, [t], [0]) for c, t in zip(caches, toks)]).cpu()
+    ref = torch.stack([plain.forward(q)[-1] for q in seqs])
+    assert torch.allclose(got, ref, **TOL["bfloat16"]), (got - ref).abs().max()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_and_first_tokens(folder_c, dtype, tmp_path):
     require_gpu()

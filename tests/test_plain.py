@@ -108,9 +108,11 @@ def test_model_is_causal_and_shift_invariant(model_b):
     assert torch.allclose(m64.forward(toks).float(), full, atol=2e-4)
 
 
-def test_norm_placement(model_b):
-    """q/k norm comes before the rotation and v is not normed: scaling q_norm's weight scales the
-    scores, which changes logits; scaling v through a 'v norm' does not exist."""
+def test_a_zero_q_norm_weight_gives_uniform_attention(model_b):
+    """The q norm's weight multiplies the queries: with a zero weight in layer 0 every score there is zero, the
+    attention is the plain mean over the causal prefix (finite, different, and unchanged where there is one key).  Where
+    the norms stand in the layer (before the rotation, before or after the residual sum, the final norm) is held by the
+    mutations of the second transcription below, not here."""
     toks = [1, 2, 3, 4, 5]
     base = model_b.forward(toks)
     w = dict(model_b.w)

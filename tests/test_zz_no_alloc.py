@@ -6,6 +6,7 @@ import pytest
 import torch
 
 from tests.gpu_util import require_gpu
+from tests.plain.sampler_plain import choose
 
 pytestmark = pytest.mark.gpu
 
@@ -42,6 +43,18 @@ def test_sample_static_equals_sample():
         assert out.tolist() == want.tolist(), "R=%d V=%d" % (R, V)
         greedy = [r for r in range(R) if r % 3 == 0]
         assert out[greedy].tolist() == logits[greedy].argmax(dim=1).tolist()
+        # the sampled rows against the plain sampler (float64 cumulative distribution over ascending ids): the two entry
+        # points share their kernels, so agreeing with each other does not show that either is right
+        lg, tp, uu, got = logits.cpu().double().numpy(), temperature.cpu().tolist(), u.cpu().tolist(), out.cpu().tolist()
+        checked = 0
+        for r in range(R):
+            if tp[r] == 0.0:
+                continue
+            tok, margin = choose(lg[r], tp[r], uu[r])
+            if margin > 1e-5:                                              # a draw at an interval's edge may fall either way in float32
+                assert got[r] == tok, "row %d: %d, the plain sampler picks %d" % (r, got[r], tok)
+                checked += 1
+        assert checked >= (R - len(greedy)) * 3 // 4
 
 
 def test_sample_static_refuses_more_rows_than_its_array_holds():
