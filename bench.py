@@ -5,9 +5,14 @@ Default: the Qwen3-8B shape (36 layers, hidden 4096, 32 query and
 8 key/value heads of 128, intermediate 12288, vocabulary 151936, untied head) with random
 bfloat16 weights; 8 requests with 1024-token random prompts decode through the engine's own step
 (scheduler, step function, cache, kernels, device sampling).  A "step" is one decode step.
+The timed steps are centred on the workload's mean context: with 1024-token prompts and 256 generated tokens
+(``--gen-len``) that is 1152 tokens, so untimed steps run up to context 1152 - steps / 2 first, whatever ``--steps`` is.
 Prints ONE JSON line: decoded tokens per second, plus the prefill of 2048 tokens, the decode
 step's HBM roofline, and decode at batch 1, 32 and 64 (tokens per second under "points"; their time per step,
-mean context and share of the HBM roofline under "points_detail").
+mean context and share of the HBM roofline under "points_detail").  Beside the fractions of the published peaks
+(8 TB/s, 2.5 PFLOP/s) the line gives fractions of rates measured at start-up on this GPU: a plain read of 2 GB
+("measured_read_gbs", "frac_of_measured") and the library's product of 2048 rows with the model's gate/up matrix
+("library_tflops", "frac_of_library").
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--dtype bfloat16|float32]
 
@@ -51,6 +56,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (both numbers are reported)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=1024)
+    ap.add_argument("--gen-len", type=int, default=256,
+                    help="tokens that the workload generates per request: the timed steps are centred on its mean context")
     ap.add_argument("--context", type=int, default=4096, help="max_model_len")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
@@ -115,12 +122,14 @@ def main() -> int:
     kv_bytes_per_token = sum(s.page_bytes(1, run_dtype) for s in model.cache_specs() if s is not None and s.paged)
 
     def decode_run(batch, steps, warmup):
-        """tokens/s, ms/step, mean context over the timed steps."""
-        ids = [eng.add_request(p, SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + 64, ignore_eos=True))
+        """tokens/s, ms/step, mean context over the timed steps.  Untimed steps first, ``warmup`` at least, until the
+        timed window is centred on the workload's mean context (prompt + gen_len / 2)."""
+        untimed = max(warmup, min((args.gen_len - steps) // 2, args.context - args.prompt_len - steps - 2))
+        ids = [eng.add_request(p, SamplingParams(temperature=0.0, max_new_tokens=untimed + steps + 64, ignore_eos=True))
                for p in prompts(batch, args.prompt_len)]
         while any(s.is_prefill or s.num_generated == 0 for s in (eng._sequences[i] for i in ids)):
             eng.step()                                                       # prompts, in portions under the budget
-        for _ in range(warmup):
+        for _ in range(untimed):
             eng.step()
         ctx0 = sum(len(eng._sequences[i]) for i in ids) / batch
         torch.cuda.synchronize()
@@ -183,6 +192,23 @@ def main() -> int:
                        "mean_rows_per_step": round(mean_rows, 2), "preemptions": pre, "page_size": page, "parallelism": "single GPU"}}))
         return 0
 
+    # what this GPU gives a kernel that only reads, and the library a product of the prefill's shape: the rates that the
+    # decode step and the prefill are held against beside the published peaks
+    read_gbs = ops.measure_read_rate(dev) / 1e9
+    lib_flops = None
+    if args.dtype == "bfloat16":
+        a = torch.randn((args.prefill_tokens, H), dtype=torch.bfloat16, device=dev)
+        b = torch.randn((2 * I, H), dtype=torch.bfloat16, device=dev)
+        best = None
+        for _ in range(6):
+            t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0.record()
+            torch.matmul(a, b.t())
+            t1.record()
+            t1.synchronize()
+            best = t0.elapsed_time(t1) if best is None else min(best, t0.elapsed_time(t1))
+        lib_flops = 2.0 * args.prefill_tokens * 2 * I * H / (best * 1e-3)
+        del a, b
     value, ms, ctx = decode_run(args.batch, args.steps, args.warmup)
     step_bytes = weight_bytes + args.batch * ctx * kv_bytes_per_token
     achieved = step_bytes / (ms * 1e-3) / 1e9
@@ -197,7 +223,7 @@ def main() -> int:
         extra["decode_b%d" % b] = round(v, 1)
         b_gbs = (weight_bytes + b * b_ctx * kv_bytes_per_token) / (b_ms * 1e-3) / 1e9
         detail["decode_b%d" % b] = {"ms_per_step": round(b_ms, 4), "mean_context": round(b_ctx, 1), "hbm_gbs": round(b_gbs, 1),
-                                    "hbm_frac": round(b_gbs / PEAK_HBM_GBS, 4)}
+                                    "hbm_frac": round(b_gbs / PEAK_HBM_GBS, 4), "frac_of_measured": round(b_gbs / read_gbs, 4)}
     line = {
         "metric": "decode tok/s at batch %d (%s, %d-token prompts)" % (args.batch, shape_name, args.prompt_len),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -208,9 +234,12 @@ def main() -> int:
                    "seq_len": args.context, "prompt_len": args.prompt_len, "mean_context": round(ctx, 1), "page_size": page,
                    "graphs": not args.enforce_eager, "run_ahead": bool(eng.run_ahead), "parallelism": "single GPU"},
         "prefill": {"value": round(T / pf, 1), "tokens": T, "ms": round(pf * 1e3, 3),
-                    "frac": round(pf_flops / pf / PEAK_FLOPS[args.dtype], 4)},
+                    "frac": round(pf_flops / pf / PEAK_FLOPS[args.dtype], 4),
+                    "library_tflops": None if lib_flops is None else round(lib_flops / 1e12, 1),
+                    "frac_of_library": None if lib_flops is None else round(pf_flops / pf / lib_flops, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+                     "frac": round(achieved / PEAK_HBM_GBS, 4), "measured_read_gbs": round(read_gbs, 1),
+                     "frac_of_measured": round(achieved / read_gbs, 4)},
         "points": extra,
         "points_detail": detail,
     }

@@ -67,7 +67,7 @@ class _Hip:
                      "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_prefill",
                      "spy_attention_prefill_workspace", "spy_swiglu", "spy_untile_weight",
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
-                     "spy_gemm_decode", "spy_gemm_decode_workspace", "spy_embedding_sumsq", "spy_sample_static"):
+                     "spy_gemm_decode", "spy_gemm_decode_workspace", "spy_embedding_sumsq", "spy_sample_static", "spy_measure_read"):
             if not hasattr(self.lib, name):
                 raise KernelError("the kernel library %s lacks %s: it is older than its sources; build it again "
                                   "(spyinfer_amd.kernels.build.build())" % (self.lib._name, name))
@@ -794,3 +794,26 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor) -> 
         hip().call("spy_sample", _ptr(logits), _ptr(temperature), _ptr(u), _ptr(out), ctypes.c_int(R), ctypes.c_int(V),
                    _ptr(ws), _Hip.stream())
     return out
+
+
+# --------------------------------------------------------------------------
+def measure_read_rate(device, num_bytes: int = 2 << 30, repeats: int = 5) -> float:
+    """Bytes per second that a kernel which only reads gets from this device's memory: ``num_bytes`` (far more than the
+    caches hold) read once per launch, the best of ``repeats`` launches.  For measurements (bench.py quotes the decode
+    step against it); the engine does not call it."""
+    device = torch.device(device)
+    num_bytes = max(1 << 20, num_bytes // 16 * 16)
+    buf = torch.empty((num_bytes,), dtype=torch.uint8, device=device)
+    buf.random_(0, 256)
+    blocks = 8 * torch.cuda.get_device_properties(device).multi_processor_count
+    sink = torch.zeros((blocks * 256,), dtype=torch.int32, device=device)
+    best = None
+    for _ in range(repeats + 1):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        hip().call("spy_measure_read", _ptr(buf), ctypes.c_int64(num_bytes), ctypes.c_int(blocks), _ptr(sink), _Hip.stream())
+        end.record()
+        end.synchronize()
+        ms = start.elapsed_time(end)
+        best = ms if best is None else min(best, ms)
+    return num_bytes / (best * 1e-3)
