@@ -189,7 +189,7 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_kernel(
 // CT: column tiles of 16 per block.  Every block reads all of X, from L2, and with MT row tiles that is MT times the
 // bytes of its W tile: with two column tiles the X fragments in registers serve both, and X's traffic halves.
 // H3 (with CT = 2, the stored product): three halves of column tiles per block, as in gemm_decode_kernel.
-template <int EPI, bool SCALED, typename TC, int MT, int CT, int GD_WAVES, bool XT, bool OT, bool H3 = false>
+template <int EPI, bool SCALED, typename TC, int MT, int CT, int GD_WAVES, bool XT, bool OT, bool H3 = false, int NCH = 0>
 __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, TC* __restrict__ C, float* __restrict__ resid_out,
     bf16_t* __restrict__ xw_out, const bf16_t* __restrict__ w_next, float* __restrict__ ss_out, const float* __restrict__ ss_in,
@@ -258,10 +258,56 @@ __global__ __launch_bounds__(GD_WAVES * 64) void gemm_decode_rows_kernel(
                 acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[nt][j], B[mt][j], acc[nt][mt], 0, 0, 0);
     // (two chunks per round, and the next chunk's operands asked for before this chunk's products, were measured at two
     // to four row tiles: no gain either)
-    for (int c = wave; c < nfull; c += GD_WAVES) {
-        bf16x8_t a[NT][4], b[MT][4];
-        GDR_LOAD(a, b, c)
-        GDR_MFMA(a, b)
+    if constexpr (NCH > 0) {
+        // NCH chunks per wave exactly (the host has checked K = 128 NCH waves), all in straight-line code.  A ring of RW
+        // chunks of W is under way while one is multiplied (all of the wave's W if it has no more), so that a compute unit
+        // keeps enough of the matrix in flight to cover the memory's latency: a loop that loads a chunk and then multiplies
+        // has a round trip to memory per chunk and streams at a third of the memory's rate.  X, which comes from L2, is
+        // asked for two chunks ahead, and ahead of the W asked for in the same turn: loads come back in the order they
+        // were issued, so an X piece behind a W piece waits for memory with it.  Every load is unconditional (rows of X
+        // beyond M: the last row's address, or the operand order's padding; their sums are not stored), and scheduling
+        // barriers keep the compiler from sinking the loads below the products.
+        constexpr int RW = NCH * NT <= 4 ? NCH : (NT == 1 ? 4 : 2);
+        bf16x8_t a[RW][NT][4], b[2][MT][4];
+#define GDR_LOAD_W(A, I)                                                                                             \
+    {                                                                                                                \
+        const char* wb = wbase + (size_t)(wave + (I) * GD_WAVES) * chunk_stride;                                     \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                                \
+            _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) {                                                      \
+                if (!H3) A[nt][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wb + woff[nt] + 1024 * j));            \
+                else A[nt][j] = w_on[nt & 1] ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wb + woff[nt] + 1024 * j))  \
+                                             : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};                                                         \
+            }                                                                                                        \
+    }
+#define GDR_LOAD_X(B, I)                                                                                             \
+    {                                                                                                                \
+        const char* xb = xbase + (size_t)(wave + (I) * GD_WAVES) * (XT ? 4 * MT * 1024 : GD_CHUNK * 2);              \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                                \
+            _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                        \
+                B[mt][j] = *reinterpret_cast<const bf16x8_t*>(xb + xoff[mt] + (XT ? MT * 1024 : 64) * j);            \
+    }
+#pragma unroll
+        for (int i = 0; i < RW; ++i) {
+            GDR_LOAD_W(a[i], i)
+            if (i < 2) GDR_LOAD_X(b[i], i)
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            GDR_MFMA(a[i % RW], b[i & 1])
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + 2 < NCH) GDR_LOAD_X(b[i & 1], i + 2)
+            if (i + RW < NCH) GDR_LOAD_W(a[i % RW], i + RW)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#undef GDR_LOAD_X
+#undef GDR_LOAD_W
+    } else {
+        for (int c = wave; c < nfull; c += GD_WAVES) {
+            bf16x8_t a[NT][4], b[MT][4];
+            GDR_LOAD(a, b, c)
+            GDR_MFMA(a, b)
+        }
     }
 #undef GDR_LOAD
 #undef GDR_MFMA
@@ -349,6 +395,11 @@ static bool gd_launch2(const GdArgs& a) {
     // what a decode step has: inputs in operand order, the residual product of a plain input with its output in operand
     // order, the stored product of a normed input
     constexpr bool TALL = XT && ((EPI == EPI_RESID && !SCALED && OT) || (EPI == EPI_STORE && SCALED));
+    // With up to eight chunks of K per wave, and three row tiles or more, the chunks run in straight-line code behind a ring of
+    // loads (measured, 4096 x 4096 and 6144 x 4096: 10.9 / 12.1 us against 11.7 / 13.5 and 14.8 / 16.3 against 15.5 / 17.8 at 48
+    // / 64 rows; at 24 and 32 rows the loop is as fast or faster: 8.9 / 9.8 and 12.2 / 13.2 against 9.4 / 9.4 and 13.6 / 13.6).
+    // What bounds these products from three row tiles on is the L2's throughput: every block pulls all of X through it.
+    const int nch = (EPI != EPI_GATED && a.K % (GD_CHUNK * W) == 0 && a.K / (GD_CHUNK * W) <= 8) ? a.K / (GD_CHUNK * W) : 0;
     if (a.M <= 16) {
         // one and a half column tiles per compute unit: three halves of tiles per block
         bool halves = false;
@@ -365,12 +416,23 @@ static bool gd_launch2(const GdArgs& a) {
         }
         if (!halves) gemm_decode_kernel<EPI, SCALED, TC, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);
     }
+#define GD_ROWS_N(MT, CT, H3, BLOCKS, NCH) gemm_decode_rows_kernel<EPI, SCALED, TC, MT, CT, W, XT, OT, H3, NCH><<<BLOCKS, W * 64, 0, a.st>>>(GD_ARGS)
+#define GD_ROWS_PICK(MT, CT, H3, BLOCKS)                                                                             \
+    if constexpr (EPI != EPI_GATED && MT >= 3) {                                                                     \
+        switch (nch) {                                                                                               \
+        case 4: GD_ROWS_N(MT, CT, H3, BLOCKS, 4); break;                                                             \
+        case 5: GD_ROWS_N(MT, CT, H3, BLOCKS, 5); break;                                                             \
+        case 8: GD_ROWS_N(MT, CT, H3, BLOCKS, 8); break;                                                             \
+        default: GD_ROWS_N(MT, CT, H3, BLOCKS, 0);                                                                   \
+        }                                                                                                            \
+    } else GD_ROWS_N(MT, CT, H3, BLOCKS, 0)
+#define GD_ROWS_ONE(MT) GD_ROWS_PICK(MT, 1, false, a.N / 16)
 #define GD_ROWS(MT)                                                                                                  \
     if constexpr (EPI == EPI_STORE) {                                                                                \
-        if (halves_rows) gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 2, W, XT, OT, true><<<a.N / 24, W * 64, 0, a.st>>>(GD_ARGS); \
-        else if (two) gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 2, W, XT, OT><<<a.N / 32, W * 64, 0, a.st>>>(GD_ARGS);   \
-        else gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 1, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS);      \
-    } else gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 1, W, XT, OT><<<a.N / 16, W * 64, 0, a.st>>>(GD_ARGS)
+        if (halves_rows) { GD_ROWS_PICK(MT, 2, true, a.N / 24); }                                                    \
+        else if (two) { GD_ROWS_PICK(MT, 2, false, a.N / 32); }                                                      \
+        else GD_ROWS_ONE(MT);                                                                                        \
+    } else GD_ROWS_ONE(MT)
 #define GD_ROWS_TALL(MT)                                                                                             \
     if constexpr (TALL) gemm_decode_rows_kernel<EPI, SCALED, TC, MT, 1, 8, XT, OT><<<a.N / 16, 512, 0, a.st>>>(GD_ARGS); \
     else return false;
@@ -381,6 +443,9 @@ static bool gd_launch2(const GdArgs& a) {
     else { GD_ROWS_TALL(8) }
 #undef GD_ROWS_TALL
 #undef GD_ROWS
+#undef GD_ROWS_ONE
+#undef GD_ROWS_PICK
+#undef GD_ROWS_N
 #undef GD_ARGS
     return true;
 }

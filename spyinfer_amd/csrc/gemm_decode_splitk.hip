@@ -70,11 +70,9 @@ __global__ __launch_bounds__(GW * 64, 1) void gemm_decode_splitk_kernel(
     if (SCALED) gd_ss_share<MT, GW * 4>(ss_in, n_parts, wave * 4 + g, r, ss_part);
 
     const size_t chunk_stride = (size_t)tiles * 4096;
-    unsigned xoff[MT];
-    bool x_ok[MT];
+    unsigned xoff[MT];                // (rows beyond M: the last row's address, or the operand order's padding)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        x_ok[mt] = 16 * mt + r < M;
         xoff[mt] = XT ? (unsigned)mt * 1024u + 16u * lane : (unsigned)min(16 * mt + r, M - 1) * (unsigned)K * 2u + 16u * g;
     }
     const char* xbase = reinterpret_cast<const char*>(X);
@@ -89,8 +87,14 @@ __global__ __launch_bounds__(GW * 64, 1) void gemm_decode_splitk_kernel(
         for (int mt = 0; mt < MT; ++mt) acc[ct][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     const char* wbase = reinterpret_cast<const char*>(Wt) + (size_t)t0 * 4096 + 16u * lane;
     {
-        // one step at a time, the next step's operands asked for before this step's products
-        bf16x8_t a0[CT], b0[MT], a1[CT], b1[MT];
+        // A ring of four steps' operands: three steps are under way while one is multiplied, so that a compute unit keeps
+        // enough of the matrix in flight to cover the memory's latency (with one step under way the product of 64 rows
+        // streamed at half the memory's rate).  What keeps the ring full in the compiled code: every load is
+        // unconditional (rows of X beyond M are read from the last row, or from the padding of the operand order; their
+        // sums are never stored), and the last four steps, which ask for nothing more, are peeled from the loop.  A load
+        // under a condition makes the compiler count the loads in flight as the fewest there may be, and a load that the
+        // loop's last turn skips makes it wait for all of them in every turn.
+        bf16x8_t a0[CT], b0[MT], a1[CT], b1[MT], a2[CT], b2[MT], a3[CT], b3[MT];
 #define SK_LOAD(A, B, STEP)                                                                                          \
         {                                                                                                            \
             const int c_ = c_begin + wave + GW * ((STEP) >> 2), h_ = (STEP) & 3;                                     \
@@ -102,35 +106,34 @@ __global__ __launch_bounds__(GW * 64, 1) void gemm_decode_splitk_kernel(
                 A[ct] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wb + (size_t)t * 4096 + 1024 * h_)); \
             }                                                                                                        \
             _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                        \
-                B[mt] = x_ok[mt] ? *reinterpret_cast<const bf16x8_t*>(xb + xoff[mt] + (XT ? MT * 1024 : 64) * h_)    \
-                                 : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};                                                 \
+                B[mt] = *reinterpret_cast<const bf16x8_t*>(xb + xoff[mt] + (XT ? MT * 1024 : 64) * h_);              \
         }
 #define SK_MFMA(A, B)                                                                                                \
         _Pragma("unroll") for (int ct = 0; ct < CT; ++ct)                                                            \
             _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                        \
                 acc[ct][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[ct], B[mt], acc[ct][mt], 0, 0, 0);
-        if constexpr (GW == 4) {
-            // (a wave that has a SIMD's registers to itself keeps three steps' operands under way instead of one)
-            bf16x8_t a2[CT], b2[MT], a3[CT], b3[MT];
-            if (my_steps > 0) { SK_LOAD(a0, b0, 0) SK_LOAD(a1, b1, 1) SK_LOAD(a2, b2, 2) }
-            for (int st = 0; st < my_steps; st += 4) {     // (a multiple of 4)
-                SK_LOAD(a3, b3, st + 3)
-                SK_MFMA(a0, b0)
-                if (st + 4 < my_steps) SK_LOAD(a0, b0, st + 4)
-                SK_MFMA(a1, b1)
-                if (st + 4 < my_steps) SK_LOAD(a1, b1, st + 5)
-                SK_MFMA(a2, b2)
-                if (st + 4 < my_steps) SK_LOAD(a2, b2, st + 6)
-                SK_MFMA(a3, b3)
+        if (my_steps > 0) {                                 // (a multiple of 4)
+            SK_LOAD(a0, b0, 0) SK_LOAD(a1, b1, 1) SK_LOAD(a2, b2, 2)
+            int st = 0;
+            // (the scheduling barriers keep the compiler from sinking the loads below the products, which would let the
+            // queue of loads run empty once per turn)
+#define SK_FENCE __builtin_amdgcn_sched_barrier(0);
+            for (; st + 4 < my_steps; st += 4) {
+                SK_LOAD(a3, b3, st + 3) SK_FENCE
+                SK_MFMA(a0, b0) SK_FENCE
+                SK_LOAD(a0, b0, st + 4) SK_FENCE
+                SK_MFMA(a1, b1) SK_FENCE
+                SK_LOAD(a1, b1, st + 5) SK_FENCE
+                SK_MFMA(a2, b2) SK_FENCE
+                SK_LOAD(a2, b2, st + 6) SK_FENCE
+                SK_MFMA(a3, b3) SK_FENCE
             }
-        } else {
-            if (my_steps > 0) SK_LOAD(a0, b0, 0)
-            for (int st = 0; st < my_steps; st += 2) {     // (a multiple of 4)
-                SK_LOAD(a1, b1, st + 1)
-                SK_MFMA(a0, b0)
-                if (st + 2 < my_steps) SK_LOAD(a0, b0, st + 2)
-                SK_MFMA(a1, b1)
-            }
+            SK_LOAD(a3, b3, st + 3) SK_FENCE
+            SK_MFMA(a0, b0) SK_FENCE
+            SK_MFMA(a1, b1) SK_FENCE
+            SK_MFMA(a2, b2) SK_FENCE
+            SK_MFMA(a3, b3)
+#undef SK_FENCE
         }
 #undef SK_LOAD
 #undef SK_MFMA
@@ -242,22 +245,11 @@ long long gd_splitk_workspace_bytes() {
     return SK_COUNTER_BYTES + (long long)gd_compute_units() * SK_MAX_TILES_PER_BLOCK * 1024;
 }
 
-#ifndef SK_MIN_CHUNKS
-#define SK_MIN_CHUNKS 12    // chunks of K that a part has at least (three for every two waves of eight)
-#endif
-#ifndef SK_MIN_FILL
-#define SK_MIN_FILL 85      // per cent of the compute units that must get a block (qkv of 7168 x 5120, 448 tiles, in 224
-                            // blocks: 32.7 against 41.4 us at 96 rows)
-#endif
-#ifndef SK_EVEN_FILL
-#define SK_EVEN_FILL 85     // per cent of the blocks' turns that a tile per block must fill to stand up to 32 rows
-#endif
-#ifndef SK_STORE_FROM
-#define SK_STORE_FROM 64    // rows beyond which the stored product splits K
-#endif
-#ifndef GD_SPLITK
-#define GD_SPLITK 1       // 0: never taken (for measurements)
-#endif
+constexpr int SK_MIN_CHUNKS = 12;    // chunks of K that a part has at least (three for every two waves of eight)
+constexpr int SK_MIN_FILL = 85;      // per cent of the compute units that must get a block (qkv of 7168 x 5120, 448 tiles, in 224
+                                     // blocks: 32.7 against 41.4 us at 96 rows)
+constexpr int SK_EVEN_FILL = 85;     // per cent of the blocks' turns that a tile per block must fill to stand up to 32 rows
+constexpr int SK_STORE_FROM = 64;    // rows beyond which the stored product splits K
 
 // Column tiles per block and parts of K: the pair that gives the most compute units a block, a part with at least 12
 // chunks of K for its 8 waves (with one chunk per wave the way of the parts through memory costs more than X's traffic:
@@ -320,7 +312,7 @@ static bool sk_rows(const GdArgs& a) {
 // Built for the combinations that a decode step has: the residual product of a plain input (row-major or in operand
 // order) with its output in operand order, and the stored bfloat16 product of a normed input in operand order.
 bool gd_splitk_try(const GdArgs& a, int epi, bool scaled, bool f32_out) {
-    if (!GD_SPLITK || a.ws == nullptr || a.M > 128 || a.N % 16 != 0 || a.K % GD_CHUNK != 0) return false;
+    if (a.ws == nullptr || a.M > 128 || a.N % 16 != 0 || a.K % GD_CHUNK != 0) return false;
     const int cus = gd_compute_units(), tiles = a.N / 16;
     if (tiles >= 2 * cus) return false;                             // many columns: the kernels that walk column tiles
     // Up to 32 rows the kernels with a column tile per block are as fast where their blocks fill the compute units evenly

@@ -47,10 +47,8 @@ __global__ __launch_bounds__(GW * 64, 1) void gemm_decode_wide_kernel(
     const int t_begin = (int)((long long)tiles * blockIdx.x / gridDim.x), t_end = (int)((long long)tiles * (blockIdx.x + 1) / gridDim.x);
     const size_t chunk_stride = (size_t)(GATES * tiles) * 4096;
     unsigned xoff[MT];
-    bool x_ok[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        x_ok[mt] = 16 * mt + r < M;
         xoff[mt] = XT ? (unsigned)mt * 1024u + 16u * lane : (unsigned)min(16 * mt + r, M - 1) * (unsigned)K * 2u + 16u * g;
     }
     const char* xbase = reinterpret_cast<const char*>(X);
@@ -81,38 +79,58 @@ __global__ __launch_bounds__(GW * 64, 1) void gemm_decode_wide_kernel(
                         wb + (size_t)((nt / CT) * tiles + ct) * 4096 + 1024 * h_));                                  \
                 }                                                                                                    \
                 _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                    \
-                    B[mt] = x_ok[mt] ? *reinterpret_cast<const bf16x8_t*>(xb + xoff[mt] + (XT ? MT * 1024 : 64) * h_) \
-                                     : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};                                             \
+                    B[mt] = *reinterpret_cast<const bf16x8_t*>(xb + xoff[mt] + (XT ? MT * 1024 : 64) * h_);          \
             }
 #define GDW_MFMA(A, B)                                                                                               \
             _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                                        \
                 _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                                    \
                     acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A[nt], B[mt], acc[nt][mt], 0, 0, 0);
+            // Every load is unconditional (rows of X beyond M: the last row's address, or the operand order's padding; their
+            // sums are not stored) and the last steps, which ask for nothing more, are peeled from the loops: a load under a
+            // condition makes the compiler count the loads in flight as the fewest there may be, and one that the last turn
+            // skips makes it wait for all of them in every turn.  The scheduling barriers keep it from sinking the loads
+            // below the products.
+#define GDW_FENCE __builtin_amdgcn_sched_barrier(0);
             if constexpr (GW == 4 && NT + MT <= 12) {
                 // a wave that has a SIMD's registers to itself keeps three steps' operands under way instead of one (four
                 // waves with one step each would have too few bytes in flight to keep the memory busy), where four steps'
                 // operands fit the 256 registers that loads can write
                 bf16x8_t a2[NT], b2[MT], a3[NT], b3[MT];
-                if (my_steps > 0) { GDW_LOAD(a0, b0, 0) GDW_LOAD(a1, b1, 1) GDW_LOAD(a2, b2, 2) }
-                for (int st = 0; st < my_steps; st += 4) {     // (a multiple of 4)
-                    GDW_LOAD(a3, b3, st + 3)
-                    GDW_MFMA(a0, b0)
-                    if (st + 4 < my_steps) GDW_LOAD(a0, b0, st + 4)
-                    GDW_MFMA(a1, b1)
-                    if (st + 4 < my_steps) GDW_LOAD(a1, b1, st + 5)
-                    GDW_MFMA(a2, b2)
-                    if (st + 4 < my_steps) GDW_LOAD(a2, b2, st + 6)
+                if (my_steps > 0) {                             // (a multiple of 4)
+                    GDW_LOAD(a0, b0, 0) GDW_LOAD(a1, b1, 1) GDW_LOAD(a2, b2, 2)
+                    int st = 0;
+                    for (; st + 4 < my_steps; st += 4) {
+                        GDW_LOAD(a3, b3, st + 3) GDW_FENCE
+                        GDW_MFMA(a0, b0) GDW_FENCE
+                        GDW_LOAD(a0, b0, st + 4) GDW_FENCE
+                        GDW_MFMA(a1, b1) GDW_FENCE
+                        GDW_LOAD(a1, b1, st + 5) GDW_FENCE
+                        GDW_MFMA(a2, b2) GDW_FENCE
+                        GDW_LOAD(a2, b2, st + 6) GDW_FENCE
+                        GDW_MFMA(a3, b3) GDW_FENCE
+                    }
+                    GDW_LOAD(a3, b3, st + 3) GDW_FENCE
+                    GDW_MFMA(a0, b0) GDW_FENCE
+                    GDW_MFMA(a1, b1) GDW_FENCE
+                    GDW_MFMA(a2, b2) GDW_FENCE
                     GDW_MFMA(a3, b3)
                 }
             } else {
-                if (my_steps > 0) GDW_LOAD(a0, b0, 0)
-                for (int st = 0; st < my_steps; st += 2) {     // (a multiple of 4)
-                    GDW_LOAD(a1, b1, st + 1)
-                    GDW_MFMA(a0, b0)
-                    if (st + 2 < my_steps) GDW_LOAD(a0, b0, st + 2)
+                if (my_steps > 0) {                             // (a multiple of 4)
+                    GDW_LOAD(a0, b0, 0)
+                    int st = 0;
+                    for (; st + 2 < my_steps; st += 2) {
+                        GDW_LOAD(a1, b1, st + 1) GDW_FENCE
+                        GDW_MFMA(a0, b0) GDW_FENCE
+                        GDW_LOAD(a0, b0, st + 2) GDW_FENCE
+                        GDW_MFMA(a1, b1) GDW_FENCE
+                    }
+                    GDW_LOAD(a1, b1, st + 1) GDW_FENCE
+                    GDW_MFMA(a0, b0) GDW_FENCE
                     GDW_MFMA(a1, b1)
                 }
             }
+#undef GDW_FENCE
 #undef GDW_LOAD
 #undef GDW_MFMA
         }
@@ -185,12 +203,7 @@ __global__ __launch_bounds__(GW * 64, 1) void gemm_decode_wide_kernel(
     }
 }
 
-#ifndef GD_WIDE
-#define GD_WIDE 1     // 0: the wide kernel is never taken (for measurements)
-#endif
-#ifndef GD_WIDE_MIN_ROWS
-#define GD_WIDE_MIN_ROWS 9
-#endif
+constexpr int GD_WIDE_MIN_ROWS = 9;     // rows from which the kernel that walks column tiles is taken
 
 // Column tiles per group of the wide kernel for blocks that walk `per` tiles each with MT row tiles: the CT that moves the
 // fewest bytes through L2, X once per group (MT units per step) and W once per tile (GATES units).
@@ -204,12 +217,9 @@ static int wide_ct(int per, int MT, int gates, int max_ct) {
     return best;
 }
 
-#ifndef GD_GW4_FROM
-#define GD_GW4_FROM 5        // (four waves from three row tiles on, measured at 40 to 64 rows: gate/up 41-43 us against 35-37)
-#endif
-#ifndef GD_GW4_STORE_FROM
-#define GD_GW4_STORE_FROM 3  // (the stored product, whose four-wave blocks take up to twelve column tiles at a time: the output head of
-#endif                       // 151936 x 4096 at 48 / 64 / 96 rows 253 / 267 / 288 us against 266 / 283 / 307 with eight waves and six tiles)
+constexpr int GD_GW4_FROM = 5;        // (four waves from three row tiles on, measured at 40 to 64 rows: gate/up 41-43 us against 35-37)
+constexpr int GD_GW4_STORE_FROM = 3;  // (the stored product, whose four-wave blocks take up to twelve column tiles at a time: the output head of
+                                      // 151936 x 4096 at 48 / 64 / 96 rows 253 / 267 / 288 us against 266 / 283 / 307 with eight waves and six tiles)
 
 // The most column tiles of a group: its accumulators (GATES * CT * MT tiles of four registers) leave room for its
 // operands up to 24 tiles, 48 for a wave that has a SIMD to itself.
@@ -248,7 +258,7 @@ static bool gd_launch_wide(const GdArgs& a) {
         // fewer than two tiles per CU: one tile per block, two blocks per CU (beyond four row tiles the gated product has
         // no other kernel: it walks here whatever the width, two column tiles at a time at least)
         const bool only = MT > 4 && EPI == EPI_GATED;
-        if (!GD_WIDE || (tiles < 2 * cus && !only)) return false;
+        if (tiles < 2 * cus && !only) return false;
         const int per = (tiles + cus - 1) / cus;
         const int blocks = tiles < cus ? tiles : cus;
         if constexpr (FOUR) {
