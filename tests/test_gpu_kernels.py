@@ -852,3 +852,13 @@ def test_sample_frequencies():
     freq = torch.bincount(out, minlength=4).double() / R
     p = torch.softmax(logits[0].double() / 0.7, 0)
     assert (freq - p).abs().max() < 0.03
+
+
+def test_zz_the_workspace_counters_are_left_at_zero():
+    """Runs after the kernel tests of this file: the counters that the products with K split over blocks and the attention
+    with its parts merged by the last block share are at zero, as every call must leave them (a counter left away from
+    zero would make no block of a later call count itself last)."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    torch.cuda.synchronize()
+    assert ops.workspace_counters_clean(dev)
