@@ -82,7 +82,10 @@ class _Hip:
             # write nothing and report nothing.  So the workspaces start from zero again.
             if not torch.cuda.is_current_stream_capturing():
                 for ws in _decode_workspaces.values():
-                    ws.zero_()
+                    try:
+                        ws.zero_()
+                    except RuntimeError:
+                        pass                      # the device itself is in trouble: the first error is the one to report
             raise KernelError("%s: %s" % (name, message))
 
     @staticmethod
