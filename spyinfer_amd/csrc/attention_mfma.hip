@@ -128,11 +128,25 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
     int n_q, int n_kv, int d, float scale, int window, int splits, float* __restrict__ ws, FusedQKV fz, int out_tiles,
-    unsigned* counters, int log2p) {
+    unsigned* counters, int log2p, const int* __restrict__ pieces) {
     constexpr int KK = DMAX / 32;   // 32-wide chunks of the head dim for Q.K
     constexpr int DT = DMAX / 16;   // 16-row tiles of the head dim for P.V
     extern __shared__ float lds[];   // the waves' O, m, l: AW (head sizes up to 128) or AW - 1 times (DT * 4 + 2) * 64 floats
-    const int tile = blockIdx.x, hk = blockIdx.y, sp = blockIdx.z;
+    // Which (tile, kv head, part of the keys) this block has: its place in the grid, or (FUSED, `pieces` given) a record
+    // of 8 ints that the host made for this block: { entry, kv head, first and end block of 32 keys, number of this
+    // part, parts of the (entry, kv head), first workspace slot of its parts, the entry's keys }.  The host cuts every
+    // entry's keys by what the whole step has to read, so that blocks have even shares whatever the entries' lengths
+    // are; a record with entry -1 is a block without work.
+    int tile = blockIdx.x, hk = blockIdx.y, sp = blockIdx.z;
+    int pc_begin = 0, pc_end = 0, pc_slot = 0, pc_kvl = 0;
+    const bool cut_by_host = FUSED && pieces != nullptr;
+    if (cut_by_host) {
+        const int4 r0 = *reinterpret_cast<const int4*>(pieces + (size_t)blockIdx.x * 8);
+        const int4 r1 = *reinterpret_cast<const int4*>(pieces + (size_t)blockIdx.x * 8 + 4);
+        if (r0.x < 0) return;
+        tile = r0.x, hk = r0.y, pc_begin = r0.z, pc_end = r0.w;
+        sp = r1.x, splits = r1.y, pc_slot = r1.z, pc_kvl = r1.w;
+    }
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: loops over it stay scalar
     // a key's page and its place inside: a shift and a mask for pages that are a power of two (log2p >= 0), instead of
     // a division of two dozen instructions per lane, four of them per block of keys
@@ -147,8 +161,9 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     const int q0 = FUSED ? s : cu_q[s];
     const int n = FUSED ? 1 : cu_q[s + 1] - q0;
     const int nrows = n * G;
-    const int p0 = pos0[s];
-    const int kvl = kv_len[s];
+    // (the host's record brings the entry's length along: one round trip less before the pages can be asked for)
+    const int p0 = cut_by_host ? pc_kvl - 1 : pos0[s];
+    const int kvl = cut_by_host ? pc_kvl : kv_len[s];
     const int* bt = block_table + (size_t)s * max_blocks;
 
     // this lane's query row (as column of S^T and O^T)
@@ -175,7 +190,7 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
     lo &= ~31;
     const int nblk = hi >= lo ? (hi - lo) / 32 + 1 : 0;
     const int per = (nblk + splits - 1) / splits;
-    const int b_begin = sp * per, b_end = min(nblk, b_begin + per);
+    const int b_begin = cut_by_host ? pc_begin : sp * per, b_end = min(nblk, cut_by_host ? pc_end : b_begin + per);
 
     f32x4_t acc[DT];
 #pragma unroll
@@ -484,7 +499,9 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         }
         return;
     }
-    float* w = ws + (((size_t)tile * n_kv + hk) * splits + sp) * (16 * (DMAX + 2));
+    // the first of this (tile, kv head)'s parts in the workspace: where the grid puts it, or where the host's record says
+    const size_t slot0 = cut_by_host ? (size_t)pc_slot : ((size_t)tile * n_kv + hk) * splits;
+    float* w = ws + (slot0 + sp) * (16 * (DMAX + 2));
     if (SPREAD && counters) {
         // The parts of a (tile, kv head) are merged here, by the block that finishes last (a counter per tile and head,
         // left at zero), instead of by a second kernel.  The dies' L2s are not coherent inside a kernel: the parts go
@@ -524,7 +541,7 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         // trip for up to eight parts (a loop that adds as it loads has one per part).
         constexpr int MAXS = 16, BATCH = 8;                // (the caller keeps to 16 parts)
         constexpr int PART = 16 * (DMAX + 2);
-        const float* base = ws + ((size_t)tile * n_kv + hk) * splits * PART;
+        const float* base = ws + slot0 * PART;
         float pm[MAXS], pl[MAXS];
 #pragma unroll
         for (int i = 0; i < MAXS; ++i) {
@@ -595,6 +612,9 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
 
 static int dmax_of(int d) { return d <= 64 ? 64 : (d <= 128 ? 128 : 256); }
 
+// Floats of one part's sums in the workspace (keys cut by the host: one part per record).
+extern "C" int64_t spy_attention_mfma_part_workspace(int d) { return 16 * (dmax_of(d) + 2); }
+
 extern "C" int64_t spy_attention_mfma_workspace(int num_tiles, int n_kv, int d, int splits) {
     if (splits <= 1) return 0;
     return (int64_t)num_tiles * n_kv * splits * 16 * (dmax_of(d) + 2);
@@ -610,7 +630,7 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
                                   const int* tile_row0, int num_tiles, int S, int T, int n_q, int n_kv, int d, float scale,
                                   int window, int splits, float* ws, const void* qkv, const void* qw, const void* kw, int w_dtype,
                                   float eps, const float* cos_t, const float* sin_t, int max_pos, int store, int out_tiles,
-                                  unsigned* counters, int n_counters, hipStream_t st) {
+                                  unsigned* counters, int n_counters, const int* pieces, int num_pieces, hipStream_t st) {
     SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
                 "spy_attention_mfma: empty operand");
     SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 256, "spy_attention_mfma: head_dim %d is not a multiple of 16 in 16..256", d);
@@ -632,18 +652,25 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
     } else {
         SPY_REQUIRE(q, "spy_attention_mfma: no queries");
     }
+    if (pieces) {
+        // the keys cut by the host (see the kernel's top): one block per record, parts merged by their last block only
+        SPY_REQUIRE(qkv && num_pieces > 0, "spy_attention_mfma: keys cut by the host are for the fused variant");
+        SPY_REQUIRE(d <= 128 && counters && ws && (long long)num_tiles * n_kv <= n_counters && ((uintptr_t)pieces % 16) == 0,
+                    "spy_attention_mfma: keys cut by the host need head_dim <= 128, a workspace and a counter per (entry, kv head) (%d x %d, %d counters)",
+                    num_tiles, n_kv, n_counters);
+    }
     int log2p = -1;                                        // pages of a power of two: shifts instead of divisions
     if ((P & (P - 1)) == 0) { log2p = 0; while ((1 << log2p) < P) ++log2p; }
-    const dim3 grid(num_tiles, n_kv, splits);
+    const dim3 grid = pieces ? dim3(num_pieces, 1, 1) : dim3(num_tiles, n_kv, splits);
     const dim3 mgrid(num_tiles, n_kv);
     // The parts merged by each (tile, kv head)'s last block instead of a second kernel: with counters (zeroed once by the
     // caller, one per tile and head, left at zero by every call; calls that overlap on one device race on them), up to
     // 16 parts and head sizes up to 128.
-    unsigned* const cnt = (counters && splits > 1 && splits <= 16 && d <= 128 && (long long)num_tiles * n_kv <= n_counters) ? counters : nullptr;
+    unsigned* const cnt = (pieces || (counters && splits > 1 && splits <= 16 && d <= 128 && (long long)num_tiles * n_kv <= n_counters)) ? counters : nullptr;
 #define ATT_LAUNCH(DM, FZ, FL)                                                                                                \
     attention_mfma_kernel<DM, FZ, FL><<<grid, AW * 64, (DM <= 128 ? AW : AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>(  \
         (bf16_t*)out, (const bf16_t*)q, (bf16_t*)kc, (bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,  \
-        tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz, out_tiles, cnt, log2p)
+        tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz, out_tiles, cnt, log2p, pieces)
 #define ATT_CASE(DM)                                                                                                          \
     if (qkv) ATT_LAUNCH(DM, true, true); else if (d == DM) ATT_LAUNCH(DM, false, true); else ATT_LAUNCH(DM, false, false);       \
     if (cnt) {}                                                                                                               \

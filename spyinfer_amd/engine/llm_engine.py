@@ -58,7 +58,8 @@ def pages_for_memory(free_bytes: int, config: EngineConfig, model) -> int:
     if not config.enforce_eager:
         groups = len({s for s in specs if s.paged})
         graphs = ModelRunner.graph_logits_bytes(config.max_num_seqs, model.vocab_size) \
-            + ModelRunner.MAX_GRAPHS * ModelRunner.graph_metadata_bytes(config.max_num_seqs, groups, blocks)
+            + ModelRunner.MAX_GRAPHS * ModelRunner.graph_metadata_bytes(config.max_num_seqs, groups, blocks,
+                                                                        model.plan_ints(config.max_num_seqs))
     budget = int(max(0, free_bytes - graphs) * config.gpu_memory_utilization * 0.9)
     state = config.max_num_seqs * sum(s.page_bytes(page, dtype) for s in specs if not s.paged)
     if state > budget:

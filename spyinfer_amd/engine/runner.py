@@ -109,17 +109,19 @@ class ModelRunner:
         return 4 * max_num_seqs * vocab_size
 
     @staticmethod
-    def graph_metadata_bytes(entries: int, page_groups: int, fixed_max_blocks: int) -> int:
+    def graph_metadata_bytes(entries: int, page_groups: int, fixed_max_blocks: int, plan_ints: int = 0) -> int:
         """Upper bound of a captured step's own metadata buffer: per entry a row of ``fixed_max_blocks`` page numbers
-        in every page group and 64 further integers (token, position, lengths, slots, tiles; each array padded to 16 B)."""
-        return 4 * (entries * (page_groups * fixed_max_blocks + 64) + 256)
+        in every page group and 64 further integers (token, position, lengths, slots; each array padded to 16 B), and
+        what the model's parts plan for a step of that size (``DecoderModel.plan_ints``)."""
+        return 4 * (entries * (page_groups * fixed_max_blocks + 64) + 256 + plan_ints)
 
     def graph_memory_bound(self, max_graphs: Optional[int] = None) -> int:
         """Most device bytes that captured steps hold beside the activations of the largest of them (which any step,
         captured or not, needs while it runs): the shared logits tensor and ``max_graphs`` metadata buffers."""
         n = self.max_graphs if max_graphs is None else max_graphs
         return self.graph_logits_bytes(self.max_num_seqs, self.model.vocab_size) \
-            + n * self.graph_metadata_bytes(self.max_num_seqs, len(self.manager.page_groups), self.fixed_max_blocks)
+            + n * self.graph_metadata_bytes(self.max_num_seqs, len(self.manager.page_groups), self.fixed_max_blocks,
+                                            self.model.plan_ints(self.max_num_seqs))
 
     def prepare(self, entries: Sequence[StepEntry]) -> "PreparedStep":
         """The host work of a step that does not need the device: the batch's arrays, the checks, the parts' plans."""

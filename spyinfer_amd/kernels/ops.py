@@ -15,6 +15,7 @@ from __future__ import annotations
 import ctypes
 from typing import Optional
 
+import numpy as np
 import torch
 
 from . import build as _build
@@ -64,7 +65,7 @@ class _Hip:
         self.lib = _build.load()
         self.lib.spy_last_error.restype = ctypes.c_char_p
         for name in ("spy_embedding", "spy_add_rmsnorm", "spy_rmsnorm", "spy_gemm", "spy_qknorm_rope_store",
-                     "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_prefill",
+                     "spy_attention_generic", "spy_attention_mfma", "spy_attention_mfma_workspace", "spy_attention_mfma_part_workspace", "spy_attention_prefill",
                      "spy_attention_prefill_workspace", "spy_swiglu", "spy_untile_weight",
                      "spy_sample", "spy_sample_workspace", "spy_gemm_skinny", "spy_gemm_skinny_swiglu",
                      "spy_gemm_decode", "spy_gemm_decode_workspace", "spy_embedding_sumsq", "spy_sample_static", "spy_measure_read"):
@@ -589,10 +590,11 @@ class AttentionMeta:
     head-in-group) rows for entries with few rows and 128-row tiles for entries with many, built
     for one group size ``tiles_group``; None if not built.
     ``big_rows``: rows of a "big" tile (128 or 256, see ``prefill_tile_rows``).
-    Host-side: S, T, max_blocks, max_kv_len, max_q_len."""
+    Host-side: S, T, max_blocks, max_kv_len, max_q_len.
+    What the arrays say must be true: the kernels read entries, pages and pieces as they are given."""
 
     def __init__(self, cu_q, pos0, kv_len, block_table, token_entry, positions, S, T, max_blocks, max_kv_len, max_q_len,
-                 tiles=None, tiles_group=0, fixed_shape=False, big_rows=128):
+                 tiles=None, tiles_group=0, fixed_shape=False, big_rows=128, pieces=None):
         self.cu_q, self.pos0, self.kv_len, self.block_table = cu_q, pos0, kv_len, block_table
         self.token_entry, self.positions = token_entry, positions
         self.S, self.T, self.max_blocks, self.max_kv_len, self.max_q_len = S, T, max_blocks, max_kv_len, max_q_len
@@ -600,6 +602,9 @@ class AttentionMeta:
         #: True: the step is captured in a graph (block tables have a fixed width; what a launch's shape takes from the
         #: requests' lengths, the number of key parts, is part of the graph's key)
         self.fixed_shape = fixed_shape
+        #: {(n_kv, window, head_dim): int32 [records, 8] on the device}: the keys of a step of single tokens cut into pieces by
+        #: ``decode_pieces``, for the attention that takes the raw product; empty if not built
+        self.pieces = pieces or {}
 
 
 MFMA_ATTENTION = True      # False forces the plain kernel for bfloat16 too (the kernel tests flip it; nothing else does)
@@ -612,6 +617,152 @@ def key_parts_for(max_kv_len: int) -> int:
     A step captured in a graph keeps the number it was captured with, so this number belongs to the graph's key."""
     return max(1, min(DECODE_MAX_SPLITS, -(-int(max_kv_len) // DECODE_KEYS_PER_SPLIT)))
 DECODE_SPLIT_TARGET = 256   # blocks (of 4 waves) wanted in flight when all entries are single tokens (measured: B=8 best at 4 parts)
+
+
+# ---- the keys of a step of single tokens, cut into even shares on the host -------------------------------------------
+PIECE_UNITS = 256           # compute units that the pieces are dealt to; each runs two blocks at a time
+PIECE_MIN_BLOCKS = 8        # a part wants this many blocks of 32 keys at least (DECODE_KEYS_PER_SPLIT)
+PIECE_RECORD = 8            # ints per record
+# What the estimate of a cut's time is made of, in microseconds (measured with 8 kv heads of 128, 8 to 96 requests of
+# even and uneven lengths; the estimates are within 8 % rms of the kernel's times, and the cut they choose was the
+# fastest of those measured, to within the timings' noise, in every case):
+PIECE_START_US = 7.0        # from the kernel's start to a block's first keys, and its end
+PIECE_MERGE_US = 3.0        # the way of the parts through memory, once per step that cuts any entry
+PIECE_ROUND_US = 4.0        # each further round of blocks on the units beyond the two that are there from the start
+PIECE_BLOCK_US = 0.45       # a unit's time for a block of 32 keys (16 KB) while it reads alone
+PIECE_SHARED_US = 0.56      # what all units reading at once add to it (the two add as squares)
+
+
+DECODE_PIECES = True        # False: every entry's keys in one number of parts (the kernel tests flip it; nothing else does)
+
+
+def decode_pieces_ok(entries: int, tokens: int, act_dtype, n_kv: int, d: int) -> bool:
+    """Whether a step's keys are cut on the host: single tokens only, bfloat16, a head size whose parts the attention
+    kernel merges by itself, a counter for every (entry, kv head)."""
+    return (DECODE_PIECES and MFMA_ATTENTION and entries == tokens and entries > 0 and act_dtype == torch.bfloat16
+            and d in (64, 128) and entries * n_kv <= ATTENTION_COUNTERS)
+
+
+def decode_pieces_capacity(entries: int, n_kv: int) -> int:
+    """Records in the array that ``decode_pieces`` fills for a step of ``entries`` single tokens: a fixed number (a
+    launch shape), whatever the requests' lengths are."""
+    return 2 * PIECE_UNITS + entries * n_kv
+
+
+def _piece_sizes(nblk, width, even):
+    """How entries of ``nblk`` blocks of 32 keys are cut into parts of at most ``width`` blocks: [entries, 16] sizes (0:
+    no such part) and the numbers of parts.  Parts of one size and the rest (the last part, which also prepares and
+    stores the new key, is the shortest); a rest shorter than half of what a part may be joins the part before it.  ``even``: the
+    size is the least that gives the entry no more parts than ``width`` does (37 blocks at width 12: 10, 10, 10, 7
+    instead of 12, 12, 13)."""
+    n = nblk.astype(np.int64)
+    idx = np.arange(DECODE_MAX_SPLITS, dtype=np.int64)[None, :]
+    w = np.full_like(n, width)
+    if even:
+        w = np.maximum(1, -(-n // np.maximum(1, -(-n // width))))
+    full = n // w
+    rest = n - full * w
+    joined = (rest > 0) & (2 * rest < np.minimum(PIECE_MIN_BLOCKS, w)) & (full > 0)
+    parts = np.maximum(1, full + ((rest > 0) & ~joined))
+    sizes = np.where(idx < full[:, None], w[:, None], 0)
+    last = (parts - 1)[:, None]
+    sizes = np.where((idx == last) & (rest > 0)[:, None], np.where(joined, w + rest, rest)[:, None], sizes)
+    return sizes, parts
+
+
+def _estimated_time(sizes_per_entry, n_kv, d=128) -> float:
+    """Microseconds of the attention kernel for a cut.  The blocks go out largest first, unit c taking blocks c and
+    c + 256 and later blocks going where least is left; the units share the memory evenly (a unit with one block gets as
+    much as one with two), so a step ends with its fullest unit, which reads alone at the end at what a unit can take."""
+    s = np.repeat(sizes_per_entry[sizes_per_entry > 0], n_kv).astype(np.float64)
+    s = -np.sort(-s)
+    U = PIECE_UNITS
+    load = np.zeros(U)
+    for r0 in (0, U):
+        chunk = s[r0:r0 + U]
+        load[:chunk.shape[0]] += chunk
+    for r0 in range(2 * U, s.shape[0], U):
+        chunk = s[r0:r0 + U]
+        load = np.sort(load)
+        load[:chunk.shape[0]] += chunk
+    load = np.sort(load)
+    steps = np.diff(load, prepend=0.0)
+    reading = U - np.arange(U)                              # units still reading while the i-th fullest finishes
+    t = float((steps * np.sqrt(PIECE_BLOCK_US ** 2 + (reading * (PIECE_SHARED_US / U)) ** 2)).sum()) * (d / 128.0)
+    return t + PIECE_START_US + PIECE_ROUND_US * max(0, -(-int(s.shape[0]) // (2 * U)) - 1)
+
+
+_piece_plans = {}
+
+
+def _piece_plan(nblk, n_kv, d=128):
+    """(sizes [S, 16], parts [S]) for entries of ``nblk`` blocks: not cut, or cut at W blocks, W being the whole step's
+    blocks over the compute units or over twice as many, of one size per entry or W and a rest: whichever of the five
+    has the shortest estimated time.  A function of the lengths alone (the same step is always cut the same way); the
+    last few results are kept, since a request's number of blocks changes once in 32 steps."""
+    key = (nblk.tobytes(), n_kv, d, PIECE_UNITS, PIECE_MIN_BLOCKS, PIECE_START_US, PIECE_MERGE_US, PIECE_ROUND_US)
+    hit = _piece_plans.get(key)
+    if hit is not None:
+        return hit
+    S = int(nblk.shape[0])
+    total = int(nblk.sum()) * n_kv
+    floor = max(1, -(-int(nblk.max(initial=1)) // DECODE_MAX_SPLITS))
+    whole = nblk[:, None] * (np.arange(DECODE_MAX_SPLITS)[None, :] == 0)
+    best = (_estimated_time(whole, n_kv, d), whole, np.ones(S, dtype=np.int64))
+    for k in (1, 2):
+        width = max(PIECE_MIN_BLOCKS, floor, -(-total // (PIECE_UNITS * k)))
+        for even in (True, False):
+            sizes, parts = _piece_sizes(nblk, width, even)
+            if int(parts.max(initial=1)) > 1:
+                t = _estimated_time(sizes, n_kv, d) + PIECE_MERGE_US
+                if t < best[0]:
+                    best = (t, sizes, parts)
+    if len(_piece_plans) >= 32:
+        _piece_plans.pop(next(iter(_piece_plans)))
+    _piece_plans[key] = best[1:]
+    return best[1:]
+
+
+def decode_pieces(kv_len, n_kv: int, window: int = 0, capacity: Optional[int] = None, head_dim: int = 128):
+    """Cuts the keys of a step of single tokens into pieces for the fused attention kernel, one block each, so that the
+    compute units have even shares whatever the requests' lengths are (with one number of parts for all entries, a step
+    takes as long as its longest request's part).  ``kv_len`` [S]: keys of every entry after this step.  Returns int32
+    [capacity, 8] records { entry, kv head, first and end block of 32 keys (counted from the first block the entry's
+    window sees), number of the part, parts of the (entry, kv head), workspace slot of its first part, kv_len }, largest
+    pieces first, entry -1 in the unused ones.
+
+    Entries are cut into parts of at most W blocks, W being the whole step's blocks over the 256 compute units or over
+    twice as many, the parts of an entry even or W and a rest, or they are not cut at all: whichever of the five gives
+    the shortest estimated time."""
+    kv_len = np.asarray(kv_len, dtype=np.int64)
+    S = int(kv_len.shape[0])
+    capacity = decode_pieces_capacity(S, n_kv) if capacity is None else capacity
+    p0 = kv_len - 1
+    lo = (np.maximum(0, p0 - window + 1) if window > 0 else np.zeros_like(p0)) & ~31
+    nblk = np.maximum(0, (p0 - lo) // 32 + 1)
+    sizes, parts = _piece_plan(nblk, n_kv, head_dim)
+    begin = np.cumsum(sizes, axis=1) - sizes
+    ent, part = np.nonzero(sizes > 0)
+    count = int(ent.shape[0])
+    if count * n_kv > capacity:
+        raise KernelError("decode_pieces: %d pieces for %d records" % (count * n_kv, capacity))
+    order = np.argsort(-sizes[ent, part], kind="stable")
+    ent, part = ent[order], part[order]
+    # workspace slots: the parts of an (entry, kv head) lie together, entries and heads in order
+    first_slot = (np.cumsum(parts) - parts) * n_kv
+    rec = np.full((capacity, PIECE_RECORD), -1, dtype=np.int32)
+    hk = np.tile(np.arange(n_kv, dtype=np.int64), count)
+    ent, part = np.repeat(ent, n_kv), np.repeat(part, n_kv)
+    n = count * n_kv
+    rec[:n, 0] = ent
+    rec[:n, 1] = hk
+    rec[:n, 2] = begin[ent, part]
+    rec[:n, 3] = begin[ent, part] + sizes[ent, part]
+    rec[:n, 4] = part
+    rec[:n, 5] = parts[ent]
+    rec[:n, 6] = first_slot[ent] + hk * parts[ent]
+    rec[:n, 7] = kv_len[ent]
+    return rec
 
 
 PREFILL_ATTENTION_MAX_HEAD_DIM = 128
@@ -744,11 +895,22 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
             # split into parts, each part a block of 4 waves that wants 128 keys at least, and a second kernel merges.
             want = max(1, DECODE_SPLIT_TARGET // max(1, n_small * n_kv))
             splits = max(1, min(want, key_parts_for(meta.max_kv_len)))
-            ws_floats = hip().lib.spy_attention_mfma_workspace(ctypes.c_int(n_small), ctypes.c_int(n_kv), ctypes.c_int(d),
-                                                               ctypes.c_int(splits))
+            # a step of single tokens whose keys the host has cut into pieces (decode_pieces): one block per record
+            pieces = meta.pieces.get((n_kv, win, d)) if raw is not None and d <= 128 and n_small * n_kv <= ATTENTION_COUNTERS else None
+            counters = decode_workspace(q.device) if splits > 1 or pieces is not None else None
+            if counters is None:
+                pieces = None
+            if pieces is not None:
+                _dev(pieces)
+                _check(pieces.dtype == torch.int32 and pieces.dim() == 2 and pieces.shape[1] == PIECE_RECORD and pieces.shape[0] > 0
+                       and pieces.data_ptr() % 16 == 0, "paged_attention: pieces must be int32 [records, 8], 16-byte aligned")
+                ws_floats = pieces.shape[0] * hip().lib.spy_attention_mfma_part_workspace(ctypes.c_int(d))
+                splits = 1
+            else:
+                ws_floats = hip().lib.spy_attention_mfma_workspace(ctypes.c_int(n_small), ctypes.c_int(n_kv), ctypes.c_int(d),
+                                                                   ctypes.c_int(splits))
             ws = torch.empty((max(1, ws_floats),), dtype=torch.float32, device=q.device)
             # with counters the last block of a (tile, kv head) merges its parts; without, a second kernel does
-            counters = decode_workspace(q.device) if splits > 1 else None
             if raw is not None:
                 wcode = _code(raw.q_norm_w, "head norm weight") if raw.q_norm_w is not None else F32
                 fused = (_ptr(raw.qkv), _ptr(raw.q_norm_w), _ptr(raw.k_norm_w), ctypes.c_int(wcode), ctypes.c_float(raw.eps),
@@ -760,7 +922,8 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
             hip().call("spy_attention_mfma", _ptr(out), _ptr(None if raw is not None else q), _ptr(k_cache), _ptr(v_cache), *common,
                        _ptr(small_entry), _ptr(small_row0), ctypes.c_int(n_small), *sizes, ctypes.c_int(splits), _ptr(ws), *fused,
                        ctypes.c_int(operand.tiles if operand is not None else 0), _ptr(counters),
-                       ctypes.c_int(0 if counters is None else ATTENTION_COUNTERS), _Hip.stream())
+                       ctypes.c_int(0 if counters is None else ATTENTION_COUNTERS), _ptr(pieces),
+                       ctypes.c_int(0 if pieces is None else pieces.shape[0]), _Hip.stream())
         return operand if operand is not None else out
     hip().call("spy_attention_generic", _ptr(out), _ptr(q), _code(q, "q"), _ptr(k_cache), _ptr(v_cache),
                ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(meta.kv_len), _ptr(meta.block_table),

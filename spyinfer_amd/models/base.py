@@ -90,6 +90,13 @@ class DecoderModel:
         for call in self.schedule:
             self.layers[call.layer].mixer.plan(batch)
 
+    def plan_ints(self, entries: int) -> int:
+        """Most int32 values that the mixers' plans add to a step of ``entries`` single tokens (``Mixer.plan_arrays``)."""
+        arrays = {}
+        for call in self.schedule:
+            arrays.update(self.layers[call.layer].mixer.plan_arrays(entries))
+        return sum(arrays.values()) + 4 * len(arrays)
+
     def capturable(self, batch) -> bool:
         """Whether this step may be recorded in a HIP graph: every part that runs in it says so (``Part.capturable``)."""
         parts = [self.embed, self.final_norm, self.lm_head] + [self.layers[i] for i in sorted({c.layer for c in self.schedule})]

@@ -27,11 +27,15 @@ ROWS_PER_TILE = 16        # rows of (token, head-in-group) pairs in a small atte
 BIG_MIN_ROWS = 64         # entries with at least this many rows go to the prefill kernel
 
 
-def plan_attention_tiles(batch, group_size: int, big_rows: int = 0) -> None:
+def plan_attention_tiles(batch, group_size: int, big_rows: int = 0, key_parts: bool = True) -> None:
     """Adds to the step's arrays the tiles over each entry's rows (token-major, head-in-group minor) for a query-head
     group of ``group_size``: entries with at least BIG_MIN_ROWS rows are cut into tiles of ``big_rows`` rows (the
     LDS-sharing prefill kernel; 0: never), the others into 16-row tiles (one block of waves each).  Once per step,
-    group size and tile size."""
+    group size and tile size.  ``key_parts``: the caller's launches take the number of key parts from the longest
+    request (False: its keys are cut another way, ``plan_decode_pieces``)."""
+    if key_parts:
+        # the 16-row tiles' keys are split into a number of parts that follows the longest request: a launch shape
+        batch.add_graph_key("attention_key_parts", ops.key_parts_for(batch.max_kv_len))
     note = ("attention_tiles", group_size, big_rows)
     if note in batch.shared:
         return
@@ -55,8 +59,16 @@ def plan_attention_tiles(batch, group_size: int, big_rows: int = 0) -> None:
         batch.add_array("tile_entry_%s_%d_%d" % (kind, group_size, big_rows), tile_entry)
         batch.add_array("tile_row0_%s_%d_%d" % (kind, group_size, big_rows), tile_row0)
     batch.shared[note] = counts
-    # the 16-row tiles' keys are split into a number of parts that follows the longest request: a launch shape
-    batch.add_graph_key("attention_key_parts", ops.key_parts_for(batch.max_kv_len))
+
+
+def plan_decode_pieces(batch, n_kv: int, window: int, head_dim: int) -> None:
+    """Adds to the arrays of a step of single tokens its keys cut into pieces of even size (``ops.decode_pieces``), for
+    layers of ``n_kv`` kv heads of ``head_dim`` and this window.  The array's length follows the numbers of entries and
+    heads alone."""
+    note = ("decode_pieces", n_kv, window, head_dim)
+    if note not in batch.shared:
+        batch.add_array("decode_pieces_%d_%d_%d" % note[1:], ops.decode_pieces(batch.host_array("kv_len"), n_kv, window, head_dim=head_dim))
+        batch.shared[note] = True
 
 
 def attention_meta(batch, group: int, group_size: int, big_rows: int = 0) -> ops.AttentionMeta:
@@ -70,10 +82,12 @@ def attention_meta(batch, group: int, group_size: int, big_rows: int = 0) -> ops
         if counts is not None:
             tiles = {kind: (batch.array("tile_entry_%s_%d_%d" % (kind, group_size, big_rows)),
                             batch.array("tile_row0_%s_%d_%d" % (kind, group_size, big_rows)), n) for kind, n in counts.items()}
+        pieces = {key[1:]: batch.array("decode_pieces_%d_%d_%d" % key[1:]).view(-1, ops.PIECE_RECORD)
+                  for key in batch.shared if isinstance(key, tuple) and key[0] == "decode_pieces"}
         meta = ops.AttentionMeta(batch.array("cu_q"), batch.array("pos0"), batch.array("kv_len"), batch.block_table(group),
                                  batch.array("token_entry"), batch.array("positions"), batch.S, batch.T, batch.max_blocks[group],
                                  batch.max_kv_len, batch.max_q_len, tiles, group_size, fixed_shape=batch.fixed_shape,
-                                 big_rows=big_rows or 128)
+                                 big_rows=big_rows or 128, pieces=pieces)
         batch.shared[note] = meta
     return meta
 
@@ -124,7 +138,24 @@ class PagedAttention(Mixer):
         return PagedKV(self.num_kv_heads, self.head_dim, self.window)
 
     def plan(self, batch) -> None:
-        plan_attention_tiles(batch, self.num_heads // self.num_kv_heads, self._big_rows(batch, batch.page_size))
+        # a step of single tokens that the fused kernel will take has its keys cut into even pieces on the host
+        pieces = ops.decode_pieces_ok(batch.S, batch.T, batch.act_dtype, self.num_kv_heads, self.head_dim) and self._rotated_whole()
+        plan_attention_tiles(batch, self.num_heads // self.num_kv_heads, self._big_rows(batch, batch.page_size), key_parts=not pieces)
+        if pieces:
+            plan_decode_pieces(batch, self.num_kv_heads, int(self.window or 0), self.head_dim)
+
+    def plan_arrays(self, entries):
+        G = self.num_heads // self.num_kv_heads
+        out = {"tile_entry_small_%d" % G: entries, "tile_row0_small_%d" % G: entries}
+        if ops.decode_pieces_ok(entries, entries, torch.bfloat16, self.num_kv_heads, self.head_dim):
+            out["decode_pieces_%d_%d_%d" % (self.num_kv_heads, int(self.window or 0), self.head_dim)] = \
+                ops.decode_pieces_capacity(entries, self.num_kv_heads) * ops.PIECE_RECORD
+        return out
+
+    def _rotated_whole(self) -> bool:
+        """The head is rotated whole or not at all, and the group is one tile: what the fused kernel takes."""
+        rot = self.position.rotary() if self.position is not None else None
+        return (rot is None or rot[2] in (0, self.head_dim)) and self.num_heads // self.num_kv_heads <= 16
 
     def _big_rows(self, batch, page_size: int) -> int:
         """Rows of the tiles for this step's entries with many rows; 0 if the prefill kernel does not take this head

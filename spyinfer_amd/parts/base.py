@@ -85,6 +85,12 @@ class Mixer(Part):
         """Called once per step and per distinct mixer before the batch goes to the device:
         may add integer arrays to it with ``batch.add_array``."""
 
+    def plan_arrays(self, entries: int) -> dict:
+        """{array name: most int32 values} of what ``plan`` adds to a step of ``entries`` single tokens: the runner's
+        account of the device memory that a captured step of that size holds.  Arrays that several layers share have
+        one name."""
+        return {}
+
     def forward(self, x: torch.Tensor, batch, cache, store: bool = True) -> torch.Tensor:
         """x [T, H] (normed) -> [T, H].  ``cache`` is this call's layer cache
         (``PagedKVLayer``/``StateLayer``/None).  ``store=False``: read the cache of

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from tests import replay_cases as rc
-from tests.configs import INIT, TINY_A, TINY_B, TINY_C
+from tests.configs import INIT, TINY_A, TINY_B, TINY_C, TINY_D
 from tests.plain.qwen3_plain import PlainQwen3
 
 
@@ -13,7 +13,7 @@ from tests.plain.qwen3_plain import PlainQwen3
 def folders(tmp_path_factory):
     from spyinfer_amd.weights import write_random_model
     out = {}
-    for name, cfg, seed in (("A", TINY_A, 11), ("B", TINY_B, 12), ("C", TINY_C, 13)):
+    for name, cfg, seed in (("A", TINY_A, 11), ("B", TINY_B, 12), ("C", TINY_C, 13), ("D", TINY_D, 14)):
         out[name] = write_random_model(str(tmp_path_factory.mktemp("model_" + name)), cfg, seed, torch.bfloat16, **INIT)
     return out
 
@@ -80,21 +80,27 @@ def test_cache_pool_is_sized_after_the_memory_of_captured_steps():
     assert pages_for_memory(free, cfg, model) == int(free * 0.5 * 0.9) // per_page
     cfg.enforce_eager = False
     logits = 4 * 64 * 384
-    meta = ModelRunner.MAX_GRAPHS * 4 * (64 * (1 * 64 + 64) + 256)        # one page group, 512 / 8 = 64 pages per request
+    # one page group, 512 / 8 = 64 pages per request; the attention's plan for 64 single tokens: a tile each (two arrays
+    # of 64) and, the model's 2 kv heads of 32 not being a head size whose keys are cut on the host, nothing else
+    planned = 2 * 64 + 2 * 4
+    assert model.plan_ints(64) == planned
+    meta = ModelRunner.MAX_GRAPHS * 4 * (64 * (1 * 64 + 64) + 256 + planned)
     assert ModelRunner.graph_logits_bytes(64, 384) == logits
-    assert ModelRunner.MAX_GRAPHS * ModelRunner.graph_metadata_bytes(64, 1, 64) == meta
+    assert ModelRunner.MAX_GRAPHS * ModelRunner.graph_metadata_bytes(64, 1, 64, planned) == meta
     assert pages_for_memory(free, cfg, model) == int((free - logits - meta) * 0.5 * 0.9) // per_page
     assert pages_for_memory(1 << 20, cfg, model) == 1                       # less free memory than the graphs take: one page, no negative count
     cfg.gpu_memory_utilization = 1.0
     assert pages_for_memory(1 << 40, cfg, model) == 64 * 64                 # the cap
 
 
-def test_a_step_metadata_fits_the_bound_used_for_captured_steps(folders, emu_ops):
-    """The per-entry bound of a captured step's metadata (a row of page numbers per page group and 64 further integers)
-    holds for real decode batches with fixed-width block tables."""
+@pytest.mark.parametrize("name,act", [("B", torch.float32), ("B", torch.bfloat16), ("D", torch.bfloat16)])
+def test_a_step_metadata_fits_the_bound_used_for_captured_steps(name, act, folders, emu_ops):
+    """The per-entry bound of a captured step's metadata (a row of page numbers per page group, 64 further integers and
+    what the parts plan) holds for real decode batches with fixed-width block tables, also where the attention's keys
+    are cut on the host (bfloat16, a head size of 64)."""
     from spyinfer_amd.engine.batch import StepBatch, StepEntry
     from spyinfer_amd.engine.runner import ModelRunner, load_model
-    model = load_model(folders["B"], "float32", "cpu")
+    model = load_model(folders[name], "float32", "cpu")
     runner = ModelRunner(model, "float32", "cpu", 8, 64, 6, max_model_len=128)
     caches = [runner.manager.admit(i) for i in range(6)]
     for n, c in enumerate(caches):
@@ -102,10 +108,11 @@ def test_a_step_metadata_fits_the_bound_used_for_captured_steps(folders, emu_ops
         runner.manager.commit(c, 3 + 7 * n)
         runner.manager.reserve(c, 1)
     for live in (1, 3, 6):
-        batch = StepBatch([StepEntry(c, [5], [0]) for c in caches[:live]], runner.manager, torch.float32, "cpu", 384, runner.fixed_max_blocks)
+        batch = StepBatch([StepEntry(c, [5], [0]) for c in caches[:live]], runner.manager, act, "cpu", model.vocab_size, runner.fixed_max_blocks)
         model.plan(batch)
         _layout, total = batch.layout()
-        assert 4 * total <= ModelRunner.graph_metadata_bytes(live, 1, runner.fixed_max_blocks)
+        assert 4 * total <= ModelRunner.graph_metadata_bytes(live, len(runner.manager.page_groups), runner.fixed_max_blocks, model.plan_ints(live))
+        assert batch.has_array("decode_pieces_1_0_64") == (name == "D")
 
 
 class _CacheNeeds:

@@ -726,14 +726,24 @@ FUSED_CASES = [
 ]
 
 
+def _with_pieces(meta, kv_len, n_kv, window, d, dev):
+    """The step's keys cut on the host, as the attention part plans them."""
+    from spyinfer_amd.kernels import ops
+    rec = ops.decode_pieces(kv_len, n_kv, int(window or 0), head_dim=d)
+    meta.pieces = {(n_kv, int(window or 0), d): torch.from_numpy(rec).to(dev)}
+    return rec
+
+
 @pytest.mark.parametrize("case", range(len(FUSED_CASES)))
 @pytest.mark.parametrize("wdtype", DTYPES)
 @pytest.mark.parametrize("keys_per_part", [256, 32])
-def test_attention_taking_the_raw_product(case, wdtype, keys_per_part, monkeypatch):
+@pytest.mark.parametrize("cut", ["evenly", "by_the_host"])
+def test_attention_taking_the_raw_product(case, wdtype, keys_per_part, cut, monkeypatch):
     """Single tokens: the attention kernel norms and rotates q and the new key itself, uses the new key and value and
     stores them.  The slots of the new tokens hold NaN before the call, so a kernel that read them before writing, or
     did not write, fails; the rest of the cache must stay as it was.  Positions at the edges of pages and of 32-key
-    blocks; few and many parts of the keys."""
+    blocks; few and many parts of the keys, all entries in the same number of parts or cut by the host into pieces of
+    even size."""
     from spyinfer_amd.kernels import ops
     from spyinfer_amd.parts.rotary import RotaryEmbedding
     dev = require_gpu()
@@ -742,6 +752,15 @@ def test_attention_taking_the_raw_product(case, wdtype, keys_per_part, monkeypat
     entries = [(a, 1) for a in cached]
     _q, kc, vc, bt, te, ps, meta = make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed=50 + case, window=window)
     monkeypatch.setattr(ops, "DECODE_KEYS_PER_SPLIT", keys_per_part)
+    if cut == "by_the_host":
+        if d > 128:
+            pytest.skip("head sizes beyond 128 are not cut by the host")
+        monkeypatch.setattr(ops, "PIECE_MIN_BLOCKS", keys_per_part // 32)
+        if keys_per_part < 256:                  # as many parts as there can be
+            for name, value in (("PIECE_UNITS", 64 * len(cached)), ("PIECE_START_US", 0.0), ("PIECE_MERGE_US", 0.0), ("PIECE_ROUND_US", 0.0)):
+                monkeypatch.setattr(ops, name, value)
+        rec = _with_pieces(meta, [a + 1 for a in cached], n_kv, window, d, dev)
+        assert keys_per_part == 256 or max(cached) < 128 or rec[:, 5].max() > 1
     T = len(entries)
     qkv = rnd((T, (n_q + 2 * n_kv) * d), dtype, "cpu", 60 + case)
     qw = (1 + 0.2 * rnd((d,), torch.float32, "cpu", 61)).to(wdtype) if norm else None
@@ -784,6 +803,59 @@ def test_attention_taking_the_raw_product(case, wdtype, keys_per_part, monkeypat
     out2 = ops.paged_attention(None, kc2, vc2, P, meta, n_q, n_kv, d, scale, window, raw)
     close(out2, ref, dtype, scale=3.0, what="fused attention without store, case %d" % case)
     assert same(kc2, kc_ref) and same(vc2, vc_ref)
+
+
+@pytest.mark.parametrize("case", [(16, 4, 128, 16, 40, 2600, None), (8, 8, 64, 32, 70, 900, None), (32, 8, 128, 16, 9, 6000, 1500),
+                                  (16, 2, 128, 16, 130, 400, None)])
+def test_attention_of_requests_of_uneven_lengths_cut_by_the_host(case):
+    """Dozens of single tokens whose requests have a few to thousands of keys: the host cuts the long ones into pieces,
+    leaves the short ones whole, and the kernel's blocks take one piece each.  Every entry's far keys carry weight.
+    Reference: float64 softmax over the entry's keys, the new key normed and rotated, in its place."""
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.parts.rotary import RotaryEmbedding
+    dev = require_gpu()
+    n_q, n_kv, d, P, S, top, window = case
+    dtype, theta, eps = torch.bfloat16, 1e6, 1e-6
+    gen = torch.Generator().manual_seed(S)
+    cached = torch.randint(4, top, (S,), generator=gen).tolist()
+    cached[0], cached[1] = 3 * top, 5
+    entries = [(a, 1) for a in cached]
+    _q, kc, vc, kept, cu, meta = _long_case(dtype, dev, n_q, n_kv, d, P, entries, seed=S)
+    rec = _with_pieces(meta, [a + 1 for a in cached], n_kv, window, d, dev)
+    assert rec[:, 5].max() > 1 and (rec[rec[:, 0] >= 0][:, 5] == 1).any(), "some entries cut, some whole"
+    qkv = rnd((S, (n_q + 2 * n_kv) * d), dtype, "cpu", 7)
+    qw, kw = ((1 + 0.2 * rnd((d,), torch.float32, "cpu", 8 + i)).to(dtype) for i in range(2))
+    rope = RotaryEmbedding(d, theta, d)
+    rope.prepare(dev, 3 * top + 1)
+    rq, rk, rv = plain_qk(qkv, n_q, n_kv, d, qw, kw, eps, theta, d, torch.tensor(cached))
+    # the far keys that _long_case planted follow its own queries; plant them again for the queries of this step
+    kc = kc.clone()
+    kv_of = torch.arange(n_q) * n_kv // n_q
+    for s, a in enumerate(cached):
+        K, V = kept[s]
+        lo = max(0, a - window + 1) if window else 0
+        for c in {min(a, lo + 3), (lo + a) // 2 // P * P}:
+            if lo <= c < a:
+                for h in range(n_q):
+                    K[c, kv_of[h]] = (rq[s, h] * 1.2).to(dtype)
+                kc[meta.block_table[s, c // P].item(), :, c % P, :] = K[c]
+    raw = ops.RawQKV(qkv.to(dev), qw.to(dev), kw.to(dev), eps, rope.cos, rope.sin, True)
+    scale = 1.0 / math.sqrt(d)
+    kc_dev, vc_dev = kc.to(dev), vc.to(dev)
+    out = ops.paged_attention(None, kc_dev, vc_dev, P, meta, n_q, n_kv, d, scale, window, raw).cpu().double()
+    for s, a in enumerate(cached):
+        K, V = (x.double().clone() for x in kept[s])
+        K[a], V[a] = rk[s].to(dtype).double(), rv[s].to(dtype).double()
+        lo = max(0, a - window + 1) if window else 0
+        scores = torch.einsum("hd,chd->hc", rq[s].to(dtype).double(), K[lo:a + 1, kv_of]) * scale
+        pr = torch.softmax(scores, dim=-1)
+        ref = torch.einsum("hc,chd->hd", pr, V[lo:a + 1, kv_of]).reshape(1, n_q * d)
+        close(out[s:s + 1], ref, dtype, scale=3.0, what="entry %d with %d keys" % (s, a + 1))
+        # the new key and value are in the cache
+        page = meta.block_table[s, a // P].item()
+        close(kc_dev[page, :, a % P, :], rk[s], dtype, scale=8.0, what="stored key of entry %d" % s)
+        assert torch.equal(vc_dev[page, :, :, a % P].cpu().double(), rv[s].to(dtype).double())
+    assert ops.workspace_counters_clean(dev)
 
 
 @pytest.mark.parametrize("case", [1, 3, 8, 9])
