@@ -8,7 +8,8 @@ bfloat16 weights; 8 requests with 1024-token random prompts decode through the e
 The timed steps are centred on the workload's mean context: with 1024-token prompts and 256 generated tokens
 (``--gen-len``) that is 1152 tokens, so untimed steps run up to context 1152 - steps / 2 first, whatever ``--steps`` is.
 Prints ONE JSON line: decoded tokens per second, plus the prefill of 2048 tokens, the decode
-step's HBM roofline, and decode at batch 1, 32 and 64 (tokens per second under "points"; their time per step,
+step's HBM roofline, and decode at batch 1, 32 and 64 and at batch 32 with prompts of uneven lengths (128 to 2048
+tokens, ``--uneven``) (tokens per second under "points"; their time per step,
 mean context and share of the HBM roofline under "points_detail").  Beside the fractions of the published peaks
 (8 TB/s, 2.5 PFLOP/s) the line gives fractions of rates measured at start-up on this GPU: a plain read of 2 GB
 ("measured_read_gbs", "frac_of_measured") and the library's product of 2048 rows with the model's gate/up matrix
@@ -62,6 +63,8 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,32,64", help="further decode batch sizes to report (empty: none)")
+    ap.add_argument("--uneven", default="32", help="decode batch sizes to report with prompts of uneven lengths, uniform in "
+                                                   "128 .. 2 x prompt-len (empty: none)")
     ap.add_argument("--enforce-eager", action="store_true")
     ap.add_argument("--weight-copies", default="both", choices=["both", "tiled"], help="EngineConfig.weight_copies")
     ap.add_argument("--seed", type=int, default=0)
@@ -101,7 +104,8 @@ def main() -> int:
     torch.cuda.empty_cache()
 
     points = [int(x) for x in args.points.split(",") if x.strip()]
-    max_batch = max([args.batch, args.serve] + points)
+    uneven = [int(x) for x in args.uneven.split(",") if x.strip()]
+    max_batch = max([args.batch, args.serve] + points + uneven)
     page = 16
     pages_per_req = -(-args.context // page)
     eng = LLMEngine.__new__(LLMEngine)
@@ -121,12 +125,14 @@ def main() -> int:
     weight_bytes = (L * layer_params + H + V * H) * act_bytes              # every weight a decode step uses, once
     kv_bytes_per_token = sum(s.page_bytes(1, run_dtype) for s in model.cache_specs() if s is not None and s.paged)
 
-    def decode_run(batch, steps, warmup):
+    def decode_run(batch, steps, warmup, lengths=None):
         """tokens/s, ms/step, mean context over the timed steps.  Untimed steps first, ``warmup`` at least, until the
-        timed window is centred on the workload's mean context (prompt + gen_len / 2)."""
-        untimed = max(warmup, min((args.gen_len - steps) // 2, args.context - args.prompt_len - steps - 2))
-        ids = [eng.add_request(p, SamplingParams(temperature=0.0, max_new_tokens=untimed + steps + 64, ignore_eos=True))
-               for p in prompts(batch, args.prompt_len)]
+        timed window is centred on the workload's mean context (prompt + gen_len / 2).  ``lengths``: the prompts'
+        lengths, if not all ``--prompt-len``."""
+        lengths = [args.prompt_len] * batch if lengths is None else lengths
+        untimed = max(warmup, min((args.gen_len - steps) // 2, args.context - max(lengths) - steps - 2))
+        ids = [eng.add_request(prompts(1, n)[0], SamplingParams(temperature=0.0, max_new_tokens=untimed + steps + 64, ignore_eos=True))
+               for n in lengths]
         while any(s.is_prefill or s.num_generated == 0 for s in (eng._sequences[i] for i in ids)):
             eng.step()                                                       # prompts, in portions under the budget
         for _ in range(untimed):
@@ -224,6 +230,14 @@ def main() -> int:
         b_gbs = (weight_bytes + b * b_ctx * kv_bytes_per_token) / (b_ms * 1e-3) / 1e9
         detail["decode_b%d" % b] = {"ms_per_step": round(b_ms, 4), "mean_context": round(b_ctx, 1), "hbm_gbs": round(b_gbs, 1),
                                     "hbm_frac": round(b_gbs / PEAK_HBM_GBS, 4), "frac_of_measured": round(b_gbs / read_gbs, 4)}
+    for b in uneven:
+        lengths = torch.randint(128, min(2 * args.prompt_len, args.context - args.gen_len) + 1, (b,), generator=g).tolist()
+        v, b_ms, b_ctx = decode_run(b, max(20, args.steps // 2), max(4, args.warmup // 2), lengths)
+        extra["decode_b%d_uneven" % b] = round(v, 1)
+        b_gbs = (weight_bytes + b * b_ctx * kv_bytes_per_token) / (b_ms * 1e-3) / 1e9
+        detail["decode_b%d_uneven" % b] = {"ms_per_step": round(b_ms, 4), "mean_context": round(b_ctx, 1), "longest_prompt": max(lengths),
+                                           "shortest_prompt": min(lengths), "hbm_gbs": round(b_gbs, 1),
+                                           "hbm_frac": round(b_gbs / PEAK_HBM_GBS, 4), "frac_of_measured": round(b_gbs / read_gbs, 4)}
     line = {
         "metric": "decode tok/s at batch %d (%s, %d-token prompts)" % (args.batch, shape_name, args.prompt_len),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
