@@ -65,6 +65,9 @@ def main() -> int:
     ap.add_argument("--points", default="1,32,64", help="further decode batch sizes to report (empty: none)")
     ap.add_argument("--uneven", default="32", help="decode batch sizes to report with prompts of uneven lengths, uniform in "
                                                    "128 .. 2 x prompt-len (empty: none)")
+    ap.add_argument("--spread", action="store_true", help="the headline batch's prompts too have uneven lengths (128 .. 2 x prompt-len)")
+    ap.add_argument("--even-key-parts", action="store_true",
+                    help="every request's keys in one number of parts instead of the host's cut by the step's lengths (for comparison)")
     ap.add_argument("--enforce-eager", action="store_true")
     ap.add_argument("--weight-copies", default="both", choices=["both", "tiled"], help="EngineConfig.weight_copies")
     ap.add_argument("--seed", type=int, default=0)
@@ -88,6 +91,8 @@ def main() -> int:
     from spyinfer_amd.weights.random_init import random_tensors_on_device
 
     ops.hip()
+    if args.even_key_parts:
+        ops.DECODE_PIECES = False
     dev = torch.device("cuda:0")
     shape_name, shape = SHAPES[args.shape]
     raw = dict(shape)
@@ -215,7 +220,8 @@ def main() -> int:
             best = t0.elapsed_time(t1) if best is None else min(best, t0.elapsed_time(t1))
         lib_flops = 2.0 * args.prefill_tokens * 2 * I * H / (best * 1e-3)
         del a, b
-    value, ms, ctx = decode_run(args.batch, args.steps, args.warmup)
+    spread = lambda b: torch.randint(128, min(2 * args.prompt_len, args.context - args.gen_len) + 1, (b,), generator=g).tolist()
+    value, ms, ctx = decode_run(args.batch, args.steps, args.warmup, spread(args.batch) if args.spread else None)
     step_bytes = weight_bytes + args.batch * ctx * kv_bytes_per_token
     achieved = step_bytes / (ms * 1e-3) / 1e9
     pf = prefill_run(args.prefill_tokens)
@@ -231,7 +237,7 @@ def main() -> int:
         detail["decode_b%d" % b] = {"ms_per_step": round(b_ms, 4), "mean_context": round(b_ctx, 1), "hbm_gbs": round(b_gbs, 1),
                                     "hbm_frac": round(b_gbs / PEAK_HBM_GBS, 4), "frac_of_measured": round(b_gbs / read_gbs, 4)}
     for b in uneven:
-        lengths = torch.randint(128, min(2 * args.prompt_len, args.context - args.gen_len) + 1, (b,), generator=g).tolist()
+        lengths = spread(b)
         v, b_ms, b_ctx = decode_run(b, max(20, args.steps // 2), max(4, args.warmup // 2), lengths)
         extra["decode_b%d_uneven" % b] = round(v, 1)
         b_gbs = (weight_bytes + b * b_ctx * kv_bytes_per_token) / (b_ms * 1e-3) / 1e9
@@ -246,7 +252,8 @@ def main() -> int:
         "config": {"model": shape_name, "layers": L, "layers_of_model": model_layers, "hidden": H, "q_heads": nq,
                    "kv_heads": nkv, "head_dim": d, "intermediate": I, "vocab": V, "global_batch": args.batch,
                    "seq_len": args.context, "prompt_len": args.prompt_len, "mean_context": round(ctx, 1), "page_size": page,
-                   "graphs": not args.enforce_eager, "run_ahead": bool(eng.run_ahead), "parallelism": "single GPU"},
+                   "graphs": not args.enforce_eager, "run_ahead": bool(eng.run_ahead), "parallelism": "single GPU",
+                   "uneven_prompts": bool(args.spread), "keys_cut_by_host": bool(ops.DECODE_PIECES)},
         "prefill": {"value": round(T / pf, 1), "tokens": T, "ms": round(pf * 1e3, 3),
                     "frac": round(pf_flops / pf / PEAK_FLOPS[args.dtype], 4),
                     "library_tflops": None if lib_flops is None else round(lib_flops / 1e12, 1),

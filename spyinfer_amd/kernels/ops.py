@@ -692,35 +692,44 @@ def _estimated_time(sizes_per_entry, n_kv, d=128) -> float:
     return t + PIECE_START_US + PIECE_ROUND_US * max(0, -(-int(s.shape[0]) // (2 * U)) - 1)
 
 
-_piece_plans = {}
+_piece_choices = {}
 
 
-def _piece_plan(nblk, n_kv, d=128):
-    """(sizes [S, 16], parts [S]) for entries of ``nblk`` blocks: not cut, or cut at W blocks, W being the whole step's
-    blocks over the compute units or over twice as many, of one size per entry or W and a rest: whichever of the five
-    has the shortest estimated time.  A function of the lengths alone (the same step is always cut the same way); the
-    last few results are kept, since a request's number of blocks changes once in 32 steps."""
-    key = (nblk.tobytes(), n_kv, d, PIECE_UNITS, PIECE_MIN_BLOCKS, PIECE_START_US, PIECE_MERGE_US, PIECE_ROUND_US)
-    hit = _piece_plans.get(key)
-    if hit is not None:
-        return hit
-    S = int(nblk.shape[0])
-    total = int(nblk.sum()) * n_kv
-    floor = max(1, -(-int(nblk.max(initial=1)) // DECODE_MAX_SPLITS))
-    whole = nblk[:, None] * (np.arange(DECODE_MAX_SPLITS)[None, :] == 0)
-    best = (_estimated_time(whole, n_kv, d), whole, np.ones(S, dtype=np.int64))
+def _piece_choice(nblk, n_kv, d=128):
+    """How a step whose entries have ``nblk`` blocks of keys is cut: None (not at all) or (W, even): parts of at most W
+    blocks, W being the whole step's blocks over the compute units or over twice as many, an entry's parts of one size
+    or W and a rest: whichever of the five has the shortest estimated time.  Decided from the lengths rounded up to 8
+    blocks, so that a step is always cut the same way and the choice is looked up in most steps (a request's rounded
+    length changes once in 256 steps); the last choices are kept."""
+    coarse = nblk >> 3
+    key = (coarse.tobytes(), n_kv, d, PIECE_UNITS, PIECE_MIN_BLOCKS, PIECE_START_US, PIECE_MERGE_US, PIECE_ROUND_US)
+    if key in _piece_choices:
+        return _piece_choices[key]
+    rounded = (coarse << 3) + 7
+    total = int(rounded.sum()) * n_kv
+    floor = max(1, -(-int(rounded.max(initial=1)) // DECODE_MAX_SPLITS))
+    whole = rounded[:, None] * (np.arange(DECODE_MAX_SPLITS)[None, :] == 0)
+    best = (_estimated_time(whole, n_kv, d), None)
     for k in (1, 2):
         width = max(PIECE_MIN_BLOCKS, floor, -(-total // (PIECE_UNITS * k)))
         for even in (True, False):
-            sizes, parts = _piece_sizes(nblk, width, even)
+            sizes, parts = _piece_sizes(rounded, width, even)
             if int(parts.max(initial=1)) > 1:
                 t = _estimated_time(sizes, n_kv, d) + PIECE_MERGE_US
                 if t < best[0]:
-                    best = (t, sizes, parts)
-    if len(_piece_plans) >= 32:
-        _piece_plans.pop(next(iter(_piece_plans)))
-    _piece_plans[key] = best[1:]
-    return best[1:]
+                    best = (t, (width, even))
+    if len(_piece_choices) >= 64:
+        _piece_choices.pop(next(iter(_piece_choices)))
+    _piece_choices[key] = best[1]
+    return best[1]
+
+
+def _piece_plan(nblk, n_kv, d=128):
+    """(sizes [S, 16], parts [S]) for entries of ``nblk`` blocks (``_piece_choice``, ``_piece_sizes``)."""
+    choice = _piece_choice(nblk, n_kv, d)
+    if choice is None:
+        return nblk[:, None] * (np.arange(DECODE_MAX_SPLITS)[None, :] == 0), np.ones(nblk.shape[0], dtype=np.int64)
+    return _piece_sizes(nblk, choice[0], choice[1])
 
 
 def decode_pieces(kv_len, n_kv: int, window: int = 0, capacity: Optional[int] = None, head_dim: int = 128):
