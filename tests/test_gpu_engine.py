@@ -825,6 +825,43 @@ def test_matrices_in_tiles_only_in_a_captured_step_of_130_tokens():
 LONG_N, SHORT_N, LONG_STEPS = 4200, 37, 40
 
 
+def test_requests_of_uneven_lengths_decode_under_graphs(tmp_path):
+    """Twenty requests of 1 to 1500 tokens decode 40 steps, recorded once and replayed: the host cuts every step's keys
+    anew (long requests into parts, short ones whole; the cut changes as requests pass 32-key blocks), the recorded
+    launch stays the same.  Logits of every step and request against the plain pass of the whole sequences."""
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.runner import ModelRunner, load_model
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.weights import write_random_model
+    dev = require_gpu()
+    raw = dict(TINY_E, max_position_embeddings=2048)
+    folder = write_random_model(str(tmp_path), raw, 17, torch.bfloat16, **INIT)
+    lengths = [1, 5, 31, 32, 33, 63, 64, 100, 129, 200, 255, 300, 450, 511, 700, 900, 1100, 1279, 1400, 1500]
+    steps = 40
+    g = torch.Generator().manual_seed(3)
+    seqs = [torch.randint(0, raw["vocab_size"], (n + steps,), generator=g).tolist() for n in lengths]
+    plain = PlainQwen3(folder)
+    ref = [plain.forward(q) for q in seqs]
+    R = len(lengths)
+    runner = ModelRunner(load_model(folder, "bfloat16", dev), "bfloat16", dev, 16, sum(-(-(n + steps) // 16) for n in lengths) + 4, R,
+                         enforce_eager=False, max_model_len=2048)
+    caches = [runner.manager.admit(i) for i in range(R)]
+    for c, q, n in zip(caches, seqs, lengths):
+        runner.manager.reserve(c, n)
+        runner.step([StepEntry(c, q[:n], [])])
+    cuts = set()
+    for i in range(steps):
+        for c in caches:
+            runner.manager.reserve(c, 1)
+        got = runner.step([StepEntry(c, [q[n + i]], [0]) for c, q, n in zip(caches, seqs, lengths)]).cpu()
+        want = torch.stack([r[n + i] for r, n in zip(ref, lengths)])
+        assert torch.allclose(got, want, **TOL["bfloat16"]), "step %d: off by %s" % (i, (got - want).abs().max(1).values.tolist())
+        rec = ops.decode_pieces([n + i + 1 for n in lengths], raw["num_key_value_heads"], 0, head_dim=raw["head_dim"])
+        cuts.add(tuple(rec[rec[:, 4] == 0][:, 5].tolist()))
+    assert runner.graph_replays >= steps - 2 and len(runner._graphs) == 1
+    assert len(cuts) > 1 and max(max(c) for c in cuts) > 1 and min(min(c) for c in cuts) == 1
+
+
 @pytest.fixture(scope="module")
 def long_model(tmp_path_factory):
     """Config E with 4608 positions and doubled q and k norm weights (single far keys carry most of a softmax's weight),
@@ -852,7 +889,8 @@ def long_model(tmp_path_factory):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_request_of_4200_tokens_decodes_under_graphs(dtype, long_model):
     """One long request beside a short one, decode steps recorded and replayed: block tables of the fixed width that
-    4608 positions need (288 pages), the long request's keys in 16 parts.  A part of the keys that is lost, read through
+    4608 positions need (288 pages), the long request's keys in 16 parts (float32: the plain kernel reads them in one) or
+    in the dozen and more pieces that the host cuts them into beside the short request, which stays whole.  A part of the keys that is lost, read through
     a wrong page or merged wrongly moves the logits far beyond the tolerance (the fixture asserts it on the plain pass).
     Logits of every decode step against the plain pass of the whole sequences."""
     from spyinfer_amd.engine.batch import StepEntry
@@ -877,6 +915,10 @@ def test_a_request_of_4200_tokens_decodes_under_graphs(dtype, long_model):
             runner.manager.reserve(c, 1)
         got = runner.step([StepEntry(caches[0], [seqs[0][long_n + i]], [0]), StepEntry(caches[1], [seqs[1][short_n + i]], [0])]).cpu()
         parts.add(ops.key_parts_for(long_n + i + 1))
+        if dtype == "bfloat16":
+            # how the host cuts this step's keys: the long request in a dozen parts and more, the short one whole
+            rec = ops.decode_pieces([long_n + i + 1, short_n + i + 1], TINY_E["num_key_value_heads"], 0, head_dim=TINY_E["head_dim"])
+            assert rec[rec[:, 0] == 0][0, 5] >= 12 and rec[rec[:, 0] == 1][0, 5] == 1
         want = torch.stack([ref[0][long_n + i], ref[1][short_n + i]])
         assert torch.allclose(got, want, **tol), "decode step %d (%s): off by %g / %g" % (
             i, "replayed" if i >= 2 else "eager or captured", (got[0] - want[0]).abs().max(), (got[1] - want[1]).abs().max())
