@@ -36,20 +36,26 @@ def _code(t: torch.Tensor, what: str) -> int:
     return _CODES[t.dtype]
 
 
-def _check(cond: bool, msg: str) -> None:
+def _check(cond: bool, msg: str, *args) -> None:
+    """``msg % args`` is made only when the check fails."""
     if not cond:
-        raise KernelError(msg)
+        raise KernelError(msg % args if args else msg)
 
 
 def _dev(*tensors) -> None:
+    # (messages are made only when a check fails: a step has thousands of these)
     dev = None
     for t in tensors:
         if t is None:
             continue
-        _check(t.is_cuda, "a kernel operand lies on %s; the kernels run on the GPU only" % t.device)
-        _check(t.is_contiguous(), "a kernel operand is not contiguous")
-        dev = dev or t.device
-        _check(t.device == dev, "kernel operands lie on different devices")
+        if not t.is_cuda:
+            raise KernelError("a kernel operand lies on %s; the kernels run on the GPU only" % t.device)
+        if not t.is_contiguous():
+            raise KernelError("a kernel operand is not contiguous")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise KernelError("kernel operands lie on different devices")
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -91,7 +97,9 @@ class _Hip:
 
     @staticmethod
     def stream():
-        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        # torch's current HIP stream of the current device, by the two calls that do no more than read it (the Stream
+        # object of torch.cuda.current_stream() costs 3 us to build, and a step has hundreds of launches)
+        return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice()))
 
 
 def hip() -> _Hip:
@@ -260,7 +268,7 @@ def _result(out: Optional[torch.Tensor], M: int, N: int, dtype: torch.dtype, dev
     if out is None:
         return torch.empty((M, N), dtype=dtype, device=device)
     _check(tuple(out.shape) == (M, N) and out.dtype == dtype and out.device == device and out.is_contiguous(),
-           "the result tensor brought by the caller must be contiguous %s [%d, %d] on %s" % (dtype, M, N, device))
+           "the result tensor brought by the caller must be contiguous %s [%d, %d] on %s", dtype, M, N, device)
     return out
 
 
@@ -353,7 +361,7 @@ class OperandRows:
     @staticmethod
     def empty(rows: int, width: int, device) -> "OperandRows":
         _check(0 < rows <= FUSED_DECODE_MAX_ROWS and width % 32 == 0,
-               "operand order takes 1..%d rows of a width that is a multiple of 32" % FUSED_DECODE_MAX_ROWS)
+               "operand order takes 1..%d rows of a width that is a multiple of 32", FUSED_DECODE_MAX_ROWS)
         return OperandRows(torch.empty((width // 32, row_tiles(rows), 64, 8), dtype=torch.bfloat16, device=device), rows, width)
 
     def to_rows(self) -> torch.Tensor:
@@ -443,15 +451,15 @@ def _gemm_decode(x, tiled: torch.Tensor, epi: int, n_out: int, out, resid, xw_ou
     x_tiled = isinstance(xs, OperandRows)
     if x_tiled:
         _check(xs.width == K and tuple(xs.data.shape) == (K // 32, xs.tiles, 64, 8) and xs.data.dtype == torch.bfloat16,
-               "decode product: x in operand order must be bfloat16 [%d / 32, row tiles, 64, 8]" % K)
+               "decode product: x in operand order must be bfloat16 [%d / 32, row tiles, 64, 8]", K)
         M, xs = xs.rows, xs.data
     else:
-        _check(xs.dtype == torch.bfloat16 and xs.dim() == 2 and xs.shape[1] == K, "decode product: x must be bfloat16 [M, %d]" % K)
+        _check(xs.dtype == torch.bfloat16 and xs.dim() == 2 and xs.shape[1] == K, "decode product: x must be bfloat16 [M, %d]", K)
         M = xs.shape[0]
     out_tiled = isinstance(out, OperandRows) or isinstance(xw_out, OperandRows)
     mp = 16 * row_tiles(M)
-    _check(ss is None or ss.shape[1] == mp, "decode product: the parts of the sums of squares must have %d columns" % mp)
-    _check(ss_out is None or tuple(ss_out.shape) == (n_out // 16, mp), "decode product: the new parts must be [N / 16, %d]" % mp)
+    _check(ss is None or ss.shape[1] == mp, "decode product: the parts of the sums of squares must have %d columns", mp)
+    _check(ss_out is None or tuple(ss_out.shape) == (n_out // 16, mp), "decode product: the new parts must be [N / 16, %d]", mp)
     for o in (out, xw_out):
         if isinstance(o, OperandRows):
             _check(o.rows == M and o.width == n_out and tuple(o.data.shape) == (n_out // 32, o.tiles, 64, 8),
@@ -459,7 +467,7 @@ def _gemm_decode(x, tiled: torch.Tensor, epi: int, n_out: int, out, resid, xw_ou
     out_t = out.data if isinstance(out, OperandRows) else out
     xw_t = xw_out.data if isinstance(xw_out, OperandRows) else xw_out
     _dev(xs, ss, tiled, out_t, resid, xw_t, w_next, ss_out)
-    _check(0 < M <= FUSED_DECODE_MAX_ROWS, "decode product: %d rows (1..%d allowed)" % (M, FUSED_DECODE_MAX_ROWS))
+    _check(0 < M <= FUSED_DECODE_MAX_ROWS, "decode product: %d rows (1..%d allowed)", M, FUSED_DECODE_MAX_ROWS)
     ws = decode_workspace(xs.device)
     hip().call("spy_gemm_decode", _ptr(xs), ctypes.c_int(0 if ss is None else 1), _ptr(ss), ctypes.c_int(0 if ss is None else ss.shape[0]),
                ctypes.c_float(eps), _ptr(tiled), ctypes.c_int(epi), _ptr(out_t), ctypes.c_int(0 if out_t is None else _code(out_t, "out")),
@@ -506,9 +514,9 @@ def decode_linear_residual(x, tiled: torch.Tensor, resid: torch.Tensor, next_nor
     N = tiled.shape[0]
     M = _rows_of(x)
     _check(resid.dtype == torch.float32 and resid.dim() == 2 and resid.shape == (M, N),
-           "decode_linear_residual: the stream must be float32 [M, %d]" % N)
+           "decode_linear_residual: the stream must be float32 [M, %d]", N)
     _check(next_norm_weight.dtype == torch.bfloat16 and next_norm_weight.shape == (N,),
-           "decode_linear_residual: the next norm's weight must be bfloat16 [%d]" % N)
+           "decode_linear_residual: the next norm's weight must be bfloat16 [%d]", N)
     ss = torch.empty((N // 16, 16 * row_tiles(M)), dtype=torch.float32, device=resid.device)
     if _operand_order_ok(N):
         xw = OperandRows.empty(M, N, resid.device)
@@ -522,7 +530,7 @@ def embedding_scaled(ids: torch.Tensor, table: torch.Tensor, norm_weight: torch.
     """embedding() for few tokens -> (stream, ScaledInput of the first norm)."""
     _dev(ids, table, norm_weight)
     _check(ids.dtype == torch.int32 and ids.dim() == 1 and 0 < ids.shape[0] <= FUSED_DECODE_MAX_ROWS,
-           "embedding_scaled: ids must be int32 [1..%d]" % FUSED_DECODE_MAX_ROWS)
+           "embedding_scaled: ids must be int32 [1..%d]", FUSED_DECODE_MAX_ROWS)
     _check(table.dim() == 2, "embedding: table must be [V, H]")
     T, (V, H) = ids.shape[0], table.shape
     _check(norm_weight.dtype == torch.bfloat16 and norm_weight.shape == (H,), "embedding_scaled: the norm weight must be bfloat16 [H]")
@@ -862,7 +870,7 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
     for name, t, shape in (("cu_q", meta.cu_q, (S + 1,)), ("pos0", meta.pos0, (S,)), ("kv_len", meta.kv_len, (S,)),
                            ("block_table", meta.block_table, (S, meta.max_blocks)), ("token_entry", meta.token_entry, (T,)),
                            ("positions", meta.positions, (T,))):
-        _check(t.dtype == torch.int32 and tuple(t.shape) == shape, "paged_attention: %s must be int32 %s" % (name, shape))
+        _check(t.dtype == torch.int32 and tuple(t.shape) == shape, "paged_attention: %s must be int32 %s", name, shape)
     _check(meta.max_kv_len <= meta.max_blocks * page_size, "paged_attention: block tables are shorter than the longest request")
     win = 0 if window is None else int(window)
     _check(win >= 0, "paged_attention: window must be positive")
@@ -880,7 +888,7 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
         big_entry, big_row0, n_big = meta.tiles["big"]
         for name, t, n in (("small tile entries", small_entry, n_small), ("small tile rows", small_row0, n_small),
                            ("big tile entries", big_entry, n_big), ("big tile rows", big_row0, n_big)):
-            _check(t.dtype == torch.int32 and tuple(t.shape) == (n,), "paged_attention: %s must be int32 [%d]" % (name, n))
+            _check(t.dtype == torch.int32 and tuple(t.shape) == (n,), "paged_attention: %s must be int32 [%d]", name, n)
         common = (ctypes.c_int(page_size), ctypes.c_int(num_pages), _ptr(meta.cu_q), _ptr(meta.pos0), _ptr(meta.kv_len),
                   _ptr(meta.block_table), ctypes.c_int(meta.max_blocks))
         sizes = (ctypes.c_int(S), ctypes.c_int(T), ctypes.c_int(n_q), ctypes.c_int(n_kv), ctypes.c_int(d), ctypes.c_float(scale),
