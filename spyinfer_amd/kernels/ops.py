@@ -79,6 +79,10 @@ class _Hip:
                 raise KernelError("the kernel library %s lacks %s: it is older than its sources; build it again "
                                   "(spyinfer_amd.kernels.build.build())" % (self.lib._name, name))
             getattr(self.lib, name).restype = ctypes.c_int64 if name.endswith("_workspace") else ctypes.c_int
+        # the entry point that a step calls most: with its argument types declared, plain numbers go in as they are (no
+        # ctypes object per argument: 3 us of the host's 14 per call)
+        P, I = ctypes.c_void_p, ctypes.c_int
+        self.lib.spy_gemm_decode.argtypes = [P, I, P, I, ctypes.c_float, P, I, P, I, P, P, P, P, I, I, I, I, I, P, ctypes.c_int64, P]
 
     def call(self, name, *args):
         rc = getattr(self.lib, name)(*args)
@@ -469,11 +473,10 @@ def _gemm_decode(x, tiled: torch.Tensor, epi: int, n_out: int, out, resid, xw_ou
     _dev(xs, ss, tiled, out_t, resid, xw_t, w_next, ss_out)
     _check(0 < M <= FUSED_DECODE_MAX_ROWS, "decode product: %d rows (1..%d allowed)", M, FUSED_DECODE_MAX_ROWS)
     ws = decode_workspace(xs.device)
-    hip().call("spy_gemm_decode", _ptr(xs), ctypes.c_int(0 if ss is None else 1), _ptr(ss), ctypes.c_int(0 if ss is None else ss.shape[0]),
-               ctypes.c_float(eps), _ptr(tiled), ctypes.c_int(epi), _ptr(out_t), ctypes.c_int(0 if out_t is None else _code(out_t, "out")),
-               _ptr(resid), _ptr(xw_t), _ptr(w_next), _ptr(ss_out), ctypes.c_int(M), ctypes.c_int(n_out), ctypes.c_int(K),
-               ctypes.c_int(1 if x_tiled else 0), ctypes.c_int(1 if out_tiled else 0), _ptr(ws),
-               ctypes.c_int64(0 if ws is None else ws.numel()), _Hip.stream())
+    at = lambda t: None if t is None else t.data_ptr()              # (argument types are declared: see _Hip)
+    hip().call("spy_gemm_decode", at(xs), 0 if ss is None else 1, at(ss), 0 if ss is None else ss.shape[0], eps, at(tiled), epi,
+               at(out_t), 0 if out_t is None else _code(out_t, "out"), at(resid), at(xw_t), at(w_next), at(ss_out), M, n_out, K,
+               1 if x_tiled else 0, 1 if out_tiled else 0, at(ws), 0 if ws is None else ws.numel(), _Hip.stream())
 
 
 def _rows_of(x) -> int:
