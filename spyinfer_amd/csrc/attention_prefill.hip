@@ -37,7 +37,7 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kern
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tile_entry, const int* __restrict__ tile_row0,
-    int n_q, int n_kv, int d, float scale, int window, int log2p, int num_tiles, int splits, float* __restrict__ ws) {
+    int n_q, int n_kv, int d, float scale, int window, int log2p, int num_tiles, int splits, float* __restrict__ ws, int out_tiles) {
     constexpr int KK = DMAX / 32, DT = DMAX / 16;
     // 16 elements of padding per staged row: the products' 16-byte reads then have no bank conflicts (measured with
     // SQ_LDS_BANK_CONFLICT: 40 % of the LDS cycles with 8, none with 16; the kernel's time follows only by 0-3 %)
@@ -348,7 +348,9 @@ __global__ __launch_bounds__(PF_ROWS / RT * 4, MINW) void attention_prefill_kern
                 uint2 w;
                 w.x = pack_bf16x2(acc[t][dt][0] * inv, acc[t][dt][1] * inv);
                 w.y = pack_bf16x2(acc[t][dt][2] * inv, acc[t][dt][3] * inv);
-                *reinterpret_cast<uint2*>(op + dd) = w;
+                // (four columns from a multiple of 4 never cross a group of 8: one store either way)
+                if (out_tiles) *reinterpret_cast<uint2*>(out + attention_out_operand_order(q0 + tq[t], head[t] * d + dd, out_tiles)) = w;
+                else *reinterpret_cast<uint2*>(op + dd) = w;
             }
         }
     }
@@ -381,7 +383,7 @@ static long long cu_count() {
 extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, const void* vc, int P, int num_pages, const int* cu_q,
                                      const int* pos0, const int* kv_len, const int* block_table, int max_blocks,
                                      const int* tile_entry, const int* tile_row0, int num_tiles, int tile_rows, int S, int T, int n_q,
-                                     int n_kv, int d, float scale, int window, int splits, float* ws, hipStream_t st) {
+                                     int n_kv, int d, float scale, int window, int splits, float* ws, int out_tiles, hipStream_t st) {
     SPY_REQUIRE(num_tiles > 0 && S > 0 && T > 0 && n_q > 0 && n_kv > 0 && num_pages > 0 && max_blocks > 0,
                 "spy_attention_prefill: empty operand");
     SPY_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "spy_attention_prefill: head_dim %d is not a multiple of 16 in 16..128", d);
@@ -394,11 +396,15 @@ extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, c
     SPY_REQUIRE(splits == 1 || ws, "spy_attention_prefill: key parts without a workspace");
     SPY_REQUIRE(tile_rows == 128 || (tile_rows == 256 && (d == 64 || d == 128)),
                 "spy_attention_prefill: tiles of %d rows (128, or 256 for head sizes 64 and 128)", tile_rows);
+    // out_tiles > 0: the output [T, n_q d] goes out in MFMA operand order for that many row tiles (attention_merge.h), for a
+    // decode product that reads it next
+    SPY_REQUIRE(out_tiles >= 0 && out_tiles <= 8 && (!out_tiles || (T <= 16 * out_tiles && (n_q * d) % 32 == 0 && d % 8 == 0)),
+                "spy_attention_prefill: operand order is for at most 128 rows (%d here) of a width that is a multiple of 32", T);
     const dim3 grid(splits > 1 ? num_tiles : (num_tiles + 1) / 2, n_kv, splits);
     const dim3 mgrid(num_tiles * (tile_rows / 16), n_kv);
     const bool one_per_cu = (long long)grid.x * grid.y * grid.z <= cu_count();
 #define PF_ARGS (bf16_t*)out, (const bf16_t*)q, (const bf16_t*)kc, (const bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table,   \
-                max_blocks, tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p, num_tiles, splits, ws
+                max_blocks, tile_entry, tile_row0, n_q, n_kv, d, scale, window, log2p, num_tiles, splits, ws, out_tiles
     // (head sizes other than 64 and 128 keep the 4-wave shape: with conditions in the head-dim loops the other needs too many registers)
 #define PF_CASE(DM)                                                                                                              \
     if (tile_rows == 256) attention_prefill_kernel<DM, true, 2, 2, 256><<<grid, 512, 0, st>>>(PF_ARGS);                          \
@@ -408,7 +414,7 @@ extern "C" int spy_attention_prefill(void* out, const void* q, const void* kc, c
     } else attention_prefill_kernel<DM, false, 2, 2, 128><<<grid, 256, 0, st>>>(PF_ARGS);                                        \
     if (splits > 1)                                                                                                              \
         attention_merge_kernel<DM><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits,    \
-                                                          tile_rows / 16);
+                                                          tile_rows / 16, out_tiles);
     if (d <= 64) { PF_CASE(64) } else { PF_CASE(128) }
 #undef PF_CASE
 #undef PF_ARGS

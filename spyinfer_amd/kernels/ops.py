@@ -814,6 +814,12 @@ def mfma_attention_ok(dtype, d: int, page_size: int) -> bool:
     return MFMA_ATTENTION and dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256 and page_size % 8 == 0
 
 
+def attention_hands_over_operand_rows(dtype, n_q: int, d: int, page_size: int) -> bool:
+    """Whether ``paged_attention(..., for_product=True)`` gives a step of at most 128 tokens, single or in portions, as
+    OperandRows: what the folded decode products need of their input beyond 64 rows."""
+    return _operand_order_ok(n_q * d) and mfma_attention_ok(dtype, d, page_size)
+
+
 class RawQKV:
     """The step's raw product [q | k | v] with what turns it into queries, keys and values: the per-head norm weights
     (or None), eps, the rotation tables (or None) and whether this call stores its keys and values.  Handed to
@@ -846,8 +852,8 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
     """Causal grouped-query attention of the step's query tokens over the paged cache
     (which already holds this step's keys and values, or gets them from ``raw`` in this call).  Query at position p
     reads keys max(0, p - window + 1) .. p.  Scores, softmax and the weighted sum are float32.
-    ``for_product``: the result goes into a decode product only and may come as OperandRows (it does when all of the
-    step runs through the 16-row-tile kernel and has few rows)."""
+    ``for_product``: the result goes into a decode product only and may come as OperandRows (it does for steps of at
+    most 128 tokens, ``attention_hands_over_operand_rows``)."""
     T, S = meta.T, meta.S
     if raw is not None:
         _dev(raw.qkv, raw.q_norm_w, raw.k_norm_w, raw.cos, raw.sin)
@@ -882,8 +888,8 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
         return out
     group = n_q // n_kv
     operand = None
-    if for_product and _operand_order_ok(n_q * d) and T <= FUSED_DECODE_MAX_ROWS and d % 8 == 0 and meta.tiles is not None \
-            and meta.tiles_group == group and meta.tiles["big"][2] == 0 and mfma_attention_ok(q.dtype, d, page_size):
+    if for_product and T <= FUSED_DECODE_MAX_ROWS and meta.tiles is not None and meta.tiles_group == group \
+            and attention_hands_over_operand_rows(q.dtype, n_q, d, page_size):
         operand = OperandRows.empty(T, n_q * d, q.device)
         out = operand.data
     if mfma_attention_ok(q.dtype, d, page_size) and meta.tiles is not None and meta.tiles_group == group:
@@ -909,7 +915,8 @@ def paged_attention(q: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: t
                                                                    ctypes.c_int(d), ctypes.c_int(bsplits))
             bws = torch.empty((max(1, bws_floats),), dtype=torch.float32, device=q.device)
             hip().call("spy_attention_prefill", _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), *common, _ptr(big_entry),
-                       _ptr(big_row0), ctypes.c_int(n_big), ctypes.c_int(meta.big_rows), *sizes, ctypes.c_int(bsplits), _ptr(bws), _Hip.stream())
+                       _ptr(big_row0), ctypes.c_int(n_big), ctypes.c_int(meta.big_rows), *sizes, ctypes.c_int(bsplits), _ptr(bws),
+                       ctypes.c_int(operand.tiles if operand is not None else 0), _Hip.stream())
         if n_small:
             # Few 16-row tiles cannot fill the chip by themselves (decoding requests, short portions): their keys are
             # split into parts, each part a block of 4 waves that wants 128 keys at least, and a second kernel merges.

@@ -175,9 +175,8 @@ class PagedAttention(Mixer):
         return self.position is None or self.position.capturable(batch)
 
     def can_fold(self, batch):
-        # (beyond 64 rows the products take their inputs in operand order only, which the attention hands over when every
-        # entry is a single token)
-        if batch.T > 64 and batch.max_q_len != 1:
+        # (beyond 64 rows the products take their inputs in operand order only: the attention must hand its result over so)
+        if batch.T > 64 and not ops.attention_hands_over_operand_rows(batch.act_dtype, self.num_heads, self.head_dim, batch.page_size):
             return False
         return ops.fused_decode_ok(batch.T, batch.act_dtype, self.w_qkv_tiled, self.w_o_tiled, max_rows=self.fold_rows)
 

@@ -413,6 +413,63 @@ def test_folded_decode_steps(tmp_path_factory):
     assert torch.allclose(mixed[1:3], ref4[[1, 4]], **TOL["bfloat16"])
 
 
+def test_portions_of_65_to_128_tokens_take_the_folded_products(tmp_path_factory):
+    """Steps of 65 to 128 tokens that hold portions (a whole prompt of 100 tokens, 70 tokens of a prompt beside 20 decoded
+    tokens, a portion of 128 late in a prompt) run the folded products too: both attention kernels hand their rows over
+    in operand order.  Same logits, up to bfloat16 rounding, as with the library's products and norm kernels, and as
+    the plain pass."""
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.runner import ModelRunner, load_model
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.weights import write_random_model
+    dev = require_gpu()
+    folder = write_random_model(str(tmp_path_factory.mktemp("eng_e")), TINY_E, 65, torch.bfloat16, **INIT)
+    plain = PlainQwen3(folder)
+    model = load_model(folder, "bfloat16", dev)
+    V = TINY_E["vocab_size"]
+    g = torch.Generator().manual_seed(12)
+    whole = torch.randint(0, V, (100,), generator=g).tolist()
+    late = torch.randint(0, V, (50 + 70 + 128,), generator=g).tolist()
+    others = [torch.randint(0, V, (n + 1,), generator=g).tolist() for n in range(3, 23)]      # 20 requests that decode one token
+    runs, calls = [], []
+    real = ops.decode_linear_residual
+    for folded in (True, False):
+        ops.FUSED_DECODE = folded
+        n = [0]
+        ops.decode_linear_residual = lambda *a, **k: (n.__setitem__(0, n[0] + 1), real(*a, **k))[1]
+        try:
+            runner = ModelRunner(model, "bfloat16", dev, 16, 80, 22, enforce_eager=True, max_model_len=320)
+            caches = [runner.manager.admit(i) for i in range(22)]
+            outs = []
+            runner.manager.reserve(caches[0], 100)
+            outs.append(runner.step([StepEntry(caches[0], whole, [0, 63, 64, 99])]).cpu().clone())
+            for c, q in zip(caches[2:], others):
+                runner.manager.reserve(c, len(q) - 1)
+            runner.step([StepEntry(c, q[:-1], []) for c, q in zip(caches[2:], others)])
+            runner.manager.reserve(caches[1], 50)
+            runner.step([StepEntry(caches[1], late[:50], [])])
+            before = n[0]
+            for c in caches[1:]:
+                runner.manager.reserve(c, 70 if c is caches[1] else 1)
+            outs.append(runner.step([StepEntry(caches[1], late[50:120], [0, 69])] + [StepEntry(c, [q[-1]], [0]) for c, q in zip(caches[2:], others)]).cpu().clone())
+            runner.manager.reserve(caches[1], 128)
+            outs.append(runner.step([StepEntry(caches[1], late[120:], [0, 127])]).cpu().clone())
+            calls.append((before, n[0]))
+            runs.append(outs)
+        finally:
+            ops.FUSED_DECODE = True
+            ops.decode_linear_residual = real
+    layers = TINY_E["num_hidden_layers"]
+    assert calls[0][1] - calls[0][0] == 2 * 2 * layers and calls[1] == (0, 0), calls      # two products a layer in each of the last two steps
+    for a, b in zip(*runs):
+        assert a.shape == b.shape and torch.allclose(a, b, **TOL["bfloat16"]), (a - b).abs().max()
+    ref_whole, ref_late = plain.forward(whole), plain.forward(late)
+    assert torch.allclose(runs[0][0], ref_whole[[0, 63, 64, 99]], **TOL["bfloat16"])
+    assert torch.allclose(runs[0][1][:2], ref_late[[50, 119]], **TOL["bfloat16"])
+    assert torch.allclose(runs[0][1][2:], torch.stack([plain.forward(q)[-1] for q in others]), **TOL["bfloat16"])
+    assert torch.allclose(runs[0][2], ref_late[[120, 247]], **TOL["bfloat16"])
+
+
 @pytest.mark.parametrize("requests", [19, 37, 57, 64, 70, 100, 130])
 def test_folded_decode_steps_of_many_requests(tmp_path_factory, requests):
     """Decode steps of 17 to 128 requests take the folded products with two to eight row tiles (130 requests: the library's); their logits equal, up to

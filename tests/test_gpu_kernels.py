@@ -858,18 +858,26 @@ def test_attention_of_requests_of_uneven_lengths_cut_by_the_host(case):
     assert ops.workspace_counters_clean(dev)
 
 
-@pytest.mark.parametrize("case", [1, 3, 8, 9])
-def test_attention_output_in_operand_order(case):
-    """Steps of few rows without 128-row tiles can hand the attention's output over in MFMA operand order: the values
-    are those of the ordinary output, element for element (portions and single tokens, one and several key parts)."""
+@pytest.mark.parametrize("case", range(len(ATT_CASES)))
+@pytest.mark.parametrize("big_rows", [128, 256])
+def test_attention_output_in_operand_order(case, big_rows):
+    """Steps of at most 128 tokens can hand the attention's output over in MFMA operand order: the values are those of
+    the ordinary output, element for element (portions through the 16-row tiles and through the 128- and 256-row tiles,
+    single tokens, their mix, one and several key parts)."""
     from spyinfer_amd.kernels import ops
     dev = require_gpu()
     n_q, n_kv, d, P, entries, window = ATT_CASES[case]
-    q, kc, vc, bt, te, ps, meta = make_attention_case(torch.bfloat16, dev, n_q, n_kv, d, P, entries, seed=case, window=window)
+    if not ops.mfma_attention_ok(torch.bfloat16, d, P):
+        pytest.skip("the MFMA kernels take head sizes in steps of 16 and pages of a multiple of 8")
+    big = d <= 128 and P & (P - 1) == 0 and any(n * (n_q // n_kv) >= 64 for _, n in entries)
+    if big_rows == 256 and not (big and d in (64, 128)):
+        pytest.skip("tiles of 256 rows are for head sizes 64 and 128 and entries of many rows")
+    q, kc, vc, bt, te, ps, meta = make_attention_case(torch.bfloat16, dev, n_q, n_kv, d, P, entries, seed=case, window=window, big_rows=big_rows)
     scale = 1.0 / math.sqrt(d)
     rows = ops.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), P, meta, n_q, n_kv, d, scale, window)
     got = ops.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), P, meta, n_q, n_kv, d, scale, window, for_product=True)
-    if meta.tiles["big"][2] == 0 and meta.T <= ops.FUSED_DECODE_MAX_ROWS and (n_q * d) % 32 == 0:
+    if meta.T <= ops.FUSED_DECODE_MAX_ROWS and (n_q * d) % 32 == 0:
+        assert ops.attention_hands_over_operand_rows(torch.bfloat16, n_q, d, P)
         assert isinstance(got, ops.OperandRows) and got.rows == meta.T and torch.equal(got.to_rows(), rows)
     else:
         assert torch.equal(got, rows)
