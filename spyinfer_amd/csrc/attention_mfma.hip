@@ -16,7 +16,9 @@
 //                   (d row, g) loads the 8 keys c0 + 8g .. +7 of row d with one 16-byte load.
 // Keys lie [key][d] within a page: lane (key, g) loads 16 bytes K[key][32 kk + 8 g ..].
 // With several parts per tile the partial (O, m, l) go to a workspace; the tile's last block merges them (given
-// counters), or a second kernel does.
+// counters), or a second kernel does.  The parts of a tile are of one size, set by the grid, or (steps of single tokens)
+// cut by the host from the lengths of all of the step's requests, a record per block: long requests in many parts,
+// short ones whole, every compute unit about the same number of keys.
 //
 // FUSED (steps in which every entry is a single token, head_dim 64, 128 or 256, whole head rotated): the kernel reads
 // the raw q, k, v of the step's product itself.  A query row's values lie in one lane and the three lanes beside it the
