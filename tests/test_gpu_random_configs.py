@@ -67,3 +67,52 @@ def test_random_configuration(seed, tmp_path):
             if dtype == "bfloat16":
                 tol["atol"] *= max(1.0, rms / 0.7)
             rc.compare(rc.collect(str(out), steps, cfg["vocab_size"]), ref, what="%s/%s/%s" % (what, mode, dtype), **tol)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_decode_steps_of_uneven_lengths(seed, tmp_path):
+    """Decode steps of 2 to 40 requests of 1 to 1900 tokens at head sizes 64 and 128, where the host cuts the keys into
+    pieces: kv heads, groups, pages and lengths drawn at random, eagerly or from a recorded graph; every step's logits
+    against the plain pass.  (60 further seeds, run once: no failure.)"""
+    from spyinfer_amd.engine.batch import StepEntry
+    from spyinfer_amd.engine.runner import ModelRunner, load_model
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.weights import write_random_model
+    dev = require_gpu()
+    rng = random.Random(7000 + seed)
+    d, n_kv, group, page = rng.choice([64, 128]), rng.choice([1, 2, 3, 4, 8]), rng.choice([1, 2, 4, 5, 8]), rng.choice([8, 16, 32, 64])
+    cfg = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_act="silu", num_hidden_layers=rng.randint(1, 2),
+               hidden_size=rng.choice([128, 256]), num_attention_heads=n_kv * group, num_key_value_heads=n_kv, head_dim=d,
+               intermediate_size=rng.choice([128, 384]), vocab_size=rng.randint(90, 400), rope_theta=1e6, rms_norm_eps=1e-6,
+               tie_word_embeddings=False, max_position_embeddings=2048, bos_token_id=0, eos_token_id=1)
+    R = rng.randint(2, 40)
+    lengths = [rng.randint(1, rng.choice([100, 600, 1500])) for _ in range(R)]
+    if seed % 2:
+        lengths[0] = 1900
+    steps, eager = 5, seed % 3 == 0
+    print("seed %d: head_dim %d, %d kv heads of %d, page %d, %d requests up to %d tokens, %s" % (
+        seed, d, n_kv, group, page, R, max(lengths), "eager" if eager else "graphs"), flush=True)
+    folder = write_random_model(str(tmp_path / "m"), cfg, 500 + seed, torch.bfloat16, **INIT)
+    g = torch.Generator().manual_seed(seed)
+    seqs = [torch.randint(0, cfg["vocab_size"], (n + steps,), generator=g).tolist() for n in lengths]
+    plain = PlainQwen3(folder)
+    ref = [plain.forward(q)[n:n + steps] for q, n in zip(seqs, lengths)]
+    rms = float(torch.cat(ref).pow(2).mean().sqrt())
+    atol = TOL["bfloat16"]["atol"] * max(1.0, rms / 0.7)
+    runner = ModelRunner(load_model(folder, "bfloat16", dev), "bfloat16", dev, page, sum(-(-(n + steps) // page) for n in lengths) + 4, R,
+                         enforce_eager=eager, max_model_len=2048)
+    caches = [runner.manager.admit(i) for i in range(R)]
+    for c, q, n in zip(caches, seqs, lengths):
+        runner.manager.reserve(c, n)
+        runner.step([StepEntry(c, q[:n], [])])
+    cut = False
+    for i in range(steps):
+        for c in caches:
+            runner.manager.reserve(c, 1)
+        got = runner.step([StepEntry(c, [q[n + i]], [0]) for c, q, n in zip(caches, seqs, lengths)]).cpu()
+        want = torch.stack([r[i] for r in ref])
+        assert torch.allclose(got, want, atol=atol, rtol=TOL["bfloat16"]["rtol"]), "step %d: off by %s" % (i, (got - want).abs().max(1).values.tolist())
+        rec = ops.decode_pieces([n + i + 1 for n in lengths], n_kv, 0, head_dim=d)
+        cut = cut or int(rec[:, 5].max()) > 1
+    assert ops.workspace_counters_clean(dev)
+    assert cut or max(lengths) < 300, "a long request among these is cut into parts"
