@@ -644,7 +644,7 @@ PIECE_BLOCK_US = 0.45       # a unit's time for a block of 32 keys (16 KB) while
 PIECE_SHARED_US = 0.56      # what all units reading at once add to it (the two add as squares)
 
 
-DECODE_PIECES = True        # False: every entry's keys in one number of parts (the kernel tests flip it; nothing else does)
+DECODE_PIECES = True        # False: every entry's keys in one number of parts (for comparison: tests and the benchmark's --even-key-parts flip it)
 
 
 def decode_pieces_ok(entries: int, tokens: int, act_dtype, n_kv: int, d: int) -> bool:
