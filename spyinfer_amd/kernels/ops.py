@@ -718,9 +718,10 @@ def _piece_choice(nblk, n_kv, d=128):
         return _piece_choices[key]
     rounded = (coarse << 3) + 7
     total = int(rounded.sum()) * n_kv
-    if 2 * PIECE_UNITS * int(rounded.max(initial=1)) <= total:
-        # the longest entry is no more than half a unit's even share: the units' two blocks each are whole entries, and
-        # the blocks that follow even out what is left (measured: no cut is faster then)
+    if 4 * PIECE_UNITS * int(rounded.max(initial=1)) <= total:
+        # the longest entry is no more than a quarter of a unit's even share: whole entries, dealt out as blocks end,
+        # even the units out by themselves (and the estimates of thousands of pieces would cost the host half a
+        # millisecond a step)
         _piece_choices[key] = None
         return None
     floor = max(1, -(-int(rounded.max(initial=1)) // DECODE_MAX_SPLITS))
