@@ -122,8 +122,8 @@ __device__ __forceinline__ void norm_rotate(bf16x8_t (&x)[KK], bool normed, cons
 }
 
 // FULL: head_dim == DMAX.  The loads of keys and values then have no conditions (a page that does not exist is read as
-// page 0 and what was read is masked: scores by position, values by the count of keys that exist), so the compiler knows
-// how many loads are in flight and a wait is for the oldest only.
+// page 0 and what was read is masked: scores by position, values by the count of keys that exist and, under a window, by
+// the page's absence), so the compiler knows how many loads are in flight and a wait is for the oldest only.
 template <int DMAX, bool FUSED, bool FULL>
 __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void attention_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, bf16_t* kc, bf16_t* vc,
@@ -314,6 +314,13 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
             const int dd = dt * 16 + r16;
             if (FULL) vt[dt] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P));
             else vt[dt] = (v_ok && dd < d) ? *reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P) : zero8();
+        }
+        if (FULL && window > 0 && !v_ok) {
+            // The window's first block of 32 keys may begin in a page that the window has passed and the request has
+            // given back: its keys are masked by their positions, but what page 0 holds in their values' place would
+            // still be multiplied (by a weight of zero: harmless for numbers, not for a NaN or an infinity).
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vt[dt] = zero8();
         }
         int kpage_nn, vpage_nn;
         AM_LOOKUP(b + 2 * AW, kpage_nn, vpage_nn)

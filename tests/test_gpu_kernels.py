@@ -636,6 +636,36 @@ def test_paged_attention(dtype, case, mfma):
     close(out, ref, dtype, scale=2.0, what="attention case %d" % case)
 
 
+@pytest.mark.parametrize("case", [(8, 2, 128, 16, [(700, 1), (333, 1), (90, 1)], 100), (4, 4, 64, 16, [(500, 3), (77, 1), (260, 2)], 70),
+                                  (6, 2, 96, 8, [(300, 1), (40, 2)], 33)])
+def test_pages_that_a_window_has_passed_are_not_read(case):
+    """Under a window a request gives back the pages that no later query reads, and its block table says -1 there.  A
+    kernel's first block of keys may begin inside such a page (blocks are aligned, windows are not): those keys are
+    masked, and what lies in page 0 in their place must not reach the result.  Here page 0 holds NaN and belongs to
+    nobody, every page that the window has passed is taken out of the tables, and the result must be that of the keys
+    inside the window: single tokens and short portions, full head sizes and one that is not."""
+    from spyinfer_amd.kernels import ops
+    dev = require_gpu()
+    n_q, n_kv, d, P, entries, window = case
+    dtype = torch.bfloat16
+    q, kc, vc, bt, te, ps, meta = make_attention_case(dtype, dev, n_q, n_kv, d, P, entries, seed=n_q, window=window, spike=True)
+    scale = 1.0 / math.sqrt(d)
+    ref = plain_paged_attention(q, kc, vc, P, bt, te, ps, n_q, n_kv, d, scale, window)
+    nan_page = lambda t: torch.full_like(t[:1], float("nan"))
+    kc2, vc2 = torch.cat([nan_page(kc), kc]), torch.cat([nan_page(vc), vc])              # every page one further on, page 0 poisoned
+    table = torch.tensor(bt, dtype=torch.int32)
+    table = torch.where(table >= 0, table + 1, table)
+    gone = 0
+    for s, (a, n) in enumerate(entries):
+        passed = max(0, a - window + 1) // P                                              # the first query of the step sits at position a
+        table[s, :passed] = -1
+        gone += passed
+    assert gone > 10
+    meta.block_table = table.to(dev)
+    out = ops.paged_attention(q.to(dev), kc2.to(dev), vc2.to(dev), P, meta, n_q, n_kv, d, scale, window)
+    close(out, ref, dtype, scale=2.0, what="window %d over pages given back" % window)
+
+
 def _long_case(dtype, dev, n_q, n_kv, d, P, entries, seed, big_rows=128):
     """As make_attention_case, for thousands of keys: filled and gathered with tensor operations.  Returns also the
     keys and values of each entry in order, for the reference."""

@@ -105,6 +105,64 @@ def test_attention_part_in_cuts(dtype, window):
     manager.check()
 
 
+@pytest.mark.parametrize("window", [None, 900])
+def test_attention_part_decoding_long_requests_with_the_keys_cut_by_the_host(window):
+    """The attention part with heads of 64 in bfloat16: two requests of 1500 and 300 tokens, their prompts in portions,
+    then 40 steps of single tokens.  The host cuts the long request's keys into more parts than the short one's;
+    with a window of 900 the pages that it has passed are given back (the block table says -1 there) and the blocks
+    are counted from the window's start.  Every decoded row against the plain functions over the whole sequences."""
+    from spyinfer_amd.cache import CacheManager
+    from spyinfer_amd.cache.storage import CacheStorage
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.parts import PagedAttention, RotaryEmbedding
+    dev = require_gpu()
+    dtype = torch.bfloat16
+    H, nq, nkv, d, steps = 128, 4, 2, 64, 40
+    lengths = (1500, 300)
+    rope = RotaryEmbedding(d, 30000.0)
+    rope.prepare(dev, 2048)
+    part = PagedAttention(H, nq, nkv, d, rope, qk_norm_eps=1e-5, window=window)
+    w = bind(part, "a", dtype, dev, 30, 0.1)
+    xs = [rnd((n + steps, H), dtype, 40 + i) for i, n in enumerate(lengths)]
+    refs = []
+    for x in xs:
+        T, xf = x.shape[0], x.float()
+        q = P.rms_norm(P.linear(xf, w["a.q_proj.weight"]).view(T, nq, d), w["a.q_norm.weight"], 1e-5)
+        k = P.rms_norm(P.linear(xf, w["a.k_proj.weight"]).view(T, nkv, d), w["a.k_norm.weight"], 1e-5)
+        v = P.linear(xf, w["a.v_proj.weight"]).view(T, nkv, d)
+        cos, sin = P.rope_tables(T, d, 30000.0)
+        pos = torch.arange(T)
+        refs.append(P.linear(P.attention(P.rope_apply(q, pos, cos, sin), P.rope_apply(k, pos, cos, sin), v, window).reshape(T, nq * d),
+                             w["a.o_proj.weight"]))
+    manager = CacheManager([part.cache_spec()], page_size=16, num_pages=130, max_num_seqs=2, max_step_tokens=512)
+    storage = CacheStorage(manager, dtype, dev)
+    caches = [manager.admit(i) for i in range(2)]
+
+    def run(spans, rows):
+        batch, entries = make_batch(manager, dtype, dev, spans)
+        part.plan(batch)
+        batch.upload()
+        out = part.forward(torch.cat(rows).to(dev), batch, storage.layer(0))
+        for e in entries:
+            manager.commit(e.cache, len(e.tokens))
+        return out, batch
+
+    for c, x, n in zip(caches, xs, lengths):
+        for lo in range(0, n, 512):
+            run([(c, min(512, n - lo))], [x[lo:min(lo + 512, n)]])
+    cut = set()
+    for i in range(steps):
+        out, batch = run([(c, 1) for c in caches], [x[n + i:n + i + 1] for x, n in zip(xs, lengths)])
+        rec = batch.host_array("decode_pieces_%d_%d_%d" % (nkv, window or 0, d)).reshape(-1, ops.PIECE_RECORD)
+        cut.add((int(rec[rec[:, 0] == 0][0, 5]), int(rec[rec[:, 0] == 1][0, 5])))
+        close(out, torch.stack([r[n + i] for r, n in zip(refs, lengths)]), dtype, scale=2.0, what="step %d" % i)
+    assert all(long > short >= 1 for long, short in cut), cut
+    if window:
+        assert min(caches[0].tables[0][:30]) == -1, "the pages that the window has passed are given back"
+    manager.check()
+    assert ops.workspace_counters_clean(dev)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_mlp_part(dtype):
     from spyinfer_amd.parts import GatedMLP
