@@ -637,13 +637,15 @@ def test_paged_attention(dtype, case, mfma):
 
 
 @pytest.mark.parametrize("case", [(8, 2, 128, 16, [(700, 1), (333, 1), (90, 1)], 100), (4, 4, 64, 16, [(500, 3), (77, 1), (260, 2)], 70),
-                                  (6, 2, 96, 8, [(300, 1), (40, 2)], 33)])
+                                  (6, 2, 96, 8, [(300, 1), (40, 2)], 33),
+                                  (8, 2, 128, 16, [(600, 40), (900, 1)], 200), (4, 1, 64, 32, [(1000, 100)], 300)])
 def test_pages_that_a_window_has_passed_are_not_read(case):
     """Under a window a request gives back the pages that no later query reads, and its block table says -1 there.  A
     kernel's first block of keys may begin inside such a page (blocks are aligned, windows are not): those keys are
     masked, and what lies in page 0 in their place must not reach the result.  Here page 0 holds NaN and belongs to
     nobody, every page that the window has passed is taken out of the tables, and the result must be that of the keys
-    inside the window: single tokens and short portions, full head sizes and one that is not."""
+    inside the window: single tokens, short portions and portions that the prefill kernel takes, full head sizes and one
+    that is not."""
     from spyinfer_amd.kernels import ops
     dev = require_gpu()
     n_q, n_kv, d, P, entries, window = case
