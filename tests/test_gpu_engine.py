@@ -623,7 +623,7 @@ def test_command_line(folder_a, tmp_path):
 # A toy architecture defined here: blocks whose mixer keeps a running mean of its inputs per
 # request (state of fixed size in a slot) beside ordinary attention blocks.
 
-def _toy_parts():
+def _toy_parts(head_dim=16):
     from spyinfer_amd.cache import FixedState
     from spyinfer_amd.config import ModelConfig
     from spyinfer_amd.models import DecoderModel, LayerCall
@@ -672,10 +672,10 @@ def _toy_parts():
 
     def build(cfg):
         emb = TokenEmbedding(cfg.vocab_size, cfg.hidden_size)
-        rope = RotaryEmbedding(16, 10000.0)
+        rope = RotaryEmbedding(head_dim, 10000.0)
         layers = []
         for i in range(cfg.num_hidden_layers):
-            mixer = RunningMean(cfg.hidden_size) if i % 2 == 0 else PagedAttention(cfg.hidden_size, 4, 2, 16, rope, window=24)
+            mixer = RunningMean(cfg.hidden_size) if i % 2 == 0 else PagedAttention(cfg.hidden_size, 4, 2, head_dim, rope, window=24)
             layers.append(PreNormBlock(RMSNorm(cfg.hidden_size, 1e-5), mixer, RMSNorm(cfg.hidden_size, 1e-5),
                                        GatedMLP(cfg.hidden_size, cfg.intermediate_size)))
         # the run order names layer 1 twice (its weights run again with a cache of their own)
@@ -686,23 +686,23 @@ def _toy_parts():
     return ToyConfig, build
 
 
-def _plain_running_mean_lm(folder, tokens):
+def _plain_running_mean_lm(folder, tokens, head_dim=16):
     """The toy model of ``_toy_parts`` on a whole sequence, no cache, from the plain functions: layers 0 and 2 mix by a
     running mean, layer 1 by attention over a window of 24, and the run order is layers 0, 1, 2, 1."""
     from safetensors.torch import load_file
     from tests.plain import qwen3_plain as P
     w = {k: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
     T = len(tokens)
-    cos, sin = P.rope_tables(T, 16, 10000.0)
+    cos, sin = P.rope_tables(T, head_dim, 10000.0)
     pos = torch.arange(T)
     h = P.embedding(torch.tensor(tokens), w["model.embed_tokens.weight"])
     for layer in (0, 1, 2, 1):
         p = "model.layers.%d." % layer
         n1 = P.rms_norm(h, w[p + "input_layernorm.weight"], 1e-5)
         if layer == 1:
-            q = P.rope_apply(P.linear(n1, w[p + "self_attn.q_proj.weight"]).view(T, 4, 16), pos, cos, sin)
-            k = P.rope_apply(P.linear(n1, w[p + "self_attn.k_proj.weight"]).view(T, 2, 16), pos, cos, sin)
-            v = P.linear(n1, w[p + "self_attn.v_proj.weight"]).view(T, 2, 16)
+            q = P.rope_apply(P.linear(n1, w[p + "self_attn.q_proj.weight"]).view(T, 4, head_dim), pos, cos, sin)
+            k = P.rope_apply(P.linear(n1, w[p + "self_attn.k_proj.weight"]).view(T, 2, head_dim), pos, cos, sin)
+            v = P.linear(n1, w[p + "self_attn.v_proj.weight"]).view(T, 2, head_dim)
             a = P.linear(P.attention(q, k, v, 24).reshape(T, -1), w[p + "self_attn.o_proj.weight"])
         else:
             a = torch.cumsum(n1, 0) / (pos + 1).float()[:, None] * w[p + "self_attn.gain"]
@@ -714,11 +714,14 @@ def _plain_running_mean_lm(folder, tokens):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_toy_architecture_with_state(dtype, tmp_path):
+@pytest.mark.parametrize("head_dim", [16, 64])
+def test_toy_architecture_with_state(dtype, head_dim, tmp_path):
+    """(Heads of 64 take the attention kernels' paths for full head sizes, whose loads have no conditions: the window of
+    24 then runs over pages that the requests have given back.)"""
     from spyinfer_amd.config import register_architecture, unregister_architecture
     from spyinfer_amd.weights import write_random_model
     require_gpu()
-    ToyConfig, build = _toy_parts()
+    ToyConfig, build = _toy_parts(head_dim)
     register_architecture("ToyRunningMeanLM", ToyConfig, build)
     try:
         cfg = dict(architectures=["ToyRunningMeanLM"], hidden_size=64, num_hidden_layers=3, vocab_size=97, intermediate_size=80)
@@ -731,7 +734,7 @@ def test_toy_architecture_with_state(dtype, tmp_path):
             rc.run_replay_inprocess(folder, dtype, out, steps, rc.max_live_tokens(steps))
             outs[mode] = rc.collect(out, steps, 97)
         tol = TOL[dtype]
-        ref = {rid: _plain_running_mean_lm(folder, t) for rid, t in reqs.items()}
+        ref = {rid: _plain_running_mean_lm(folder, t, head_dim) for rid, t in reqs.items()}
         for mode in ("whole", "portions", "mixed"):
             rc.compare(outs[mode], ref, what="toy with state/%s/%s" % (mode, dtype), **tol)
         # the state matters: a request's logits differ from those of its second half alone
@@ -771,8 +774,8 @@ def _running_mean_on_device(base):
     return RunningMeanOnDevice
 
 
-@pytest.mark.parametrize("kind", ["host", "device"])
-def test_toy_with_state_through_the_entry_point_with_graphs(kind, tmp_path):
+@pytest.mark.parametrize("kind,head_dim", [("host", 16), ("device", 16), ("device", 64)])
+def test_toy_with_state_through_the_entry_point_with_graphs(kind, head_dim, tmp_path):
     """The toy architecture with a running state behind ``LLMEngine`` with graphs allowed (the default): seven requests
     of different lengths, three at a time, so that slots and pages are handed out again.  The mixer that walks
     ``batch.entries`` on the host does not call itself capturable, so no step of its model is recorded; the same
@@ -784,7 +787,7 @@ def test_toy_with_state_through_the_entry_point_with_graphs(kind, tmp_path):
     from spyinfer_amd.weights import write_random_model
     import spyinfer_amd.parts.base as parts_base
     require_gpu()
-    ToyConfig, build = _toy_parts()
+    ToyConfig, build = _toy_parts(head_dim)
     if kind == "device":
         host_build = build
 
@@ -817,7 +820,7 @@ def test_toy_with_state_through_the_entry_point_with_graphs(kind, tmp_path):
         for p, n, g in zip(ps, news, got):
             toks = list(p)
             for t in g:
-                logits = _plain_running_mean_lm(folder, toks)[-1]
+                logits = _plain_running_mean_lm(folder, toks, head_dim)[-1]
                 best = int(torch.argmax(logits))
                 assert t == best or float(logits[best] - logits[t]) < 1e-3, "request of %d tokens leaves the plain pass" % len(p)
                 toks.append(t)
