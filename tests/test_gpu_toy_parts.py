@@ -21,6 +21,7 @@ from tests.plain import qwen3_plain as P
 pytestmark = pytest.mark.gpu
 TOL = {"float32": dict(atol=1e-4, rtol=1e-4), "bfloat16": dict(atol=8e-2, rtol=2e-2)}
 EPS, WINDOW, TOP = 1e-5, 24, 2
+HEAD = {"dim": 16}   # head size of the routed toy's attention layers (the test sets it)
 
 
 def _toy():
@@ -111,7 +112,7 @@ def _toy():
         H = cfg.hidden_size
         emb = TokenEmbedding(cfg.vocab_size, H)
         pos = LearnedPositions(cfg.max_positions, H)
-        attn = lambda window: PagedAttention(H, 6, 2, 16, None, qk_norm_eps=None, window=window)
+        attn = lambda window: PagedAttention(H, 6, 2, HEAD["dim"], None, qk_norm_eps=None, window=window)
         norm = lambda: CentredNorm(H, EPS)
         layers = [PreNormBlock(norm(), attn(None), norm(), RoutedMLP(H, cfg.intermediate_size, cfg.num_experts)),
                   PreNormBlock(norm(), attn(WINDOW), norm(), GatedMLP(H, cfg.intermediate_size)),
@@ -149,8 +150,8 @@ def plain_forward(folder, tokens):
 
     def qkv(x, p):
         a = p + ".self_attn."
-        return (P.linear(x, w[a + "q_proj.weight"]).view(T, 6, 16), P.linear(x, w[a + "k_proj.weight"]).view(T, 2, 16),
-                P.linear(x, w[a + "v_proj.weight"]).view(T, 2, 16))
+        return (P.linear(x, w[a + "q_proj.weight"]).view(T, 6, HEAD["dim"]), P.linear(x, w[a + "k_proj.weight"]).view(T, 2, HEAD["dim"]),
+                P.linear(x, w[a + "v_proj.weight"]).view(T, 2, HEAD["dim"]))
 
     h = P.embedding(torch.tensor(tokens), w["model.embed_tokens.weight"]) + w["model.position.table"][:T]
     kept = None
@@ -167,10 +168,14 @@ def plain_forward(folder, tokens):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_toy_parts_and_shared_cache(dtype, tmp_path):
+@pytest.mark.parametrize("head_dim", [16, 128])
+def test_toy_parts_and_shared_cache(dtype, head_dim, tmp_path, monkeypatch):
+    """(Heads of 128: single tokens then take the attention that reads the raw product, here without head norms and
+    without rotation, once over a cache that another call has stored, once under a window.)"""
     from spyinfer_amd.config import register_architecture, unregister_architecture
     from spyinfer_amd.weights import write_random_model
     require_gpu()
+    monkeypatch.setitem(HEAD, "dim", head_dim)
     ToyConfig, build = _toy()
     register_architecture("ToyRoutedLM", ToyConfig, build)
     try:
