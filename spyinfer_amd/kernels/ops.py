@@ -682,16 +682,17 @@ def _piece_sizes(nblk, width, even):
 
 
 def _estimated_time(sizes_per_entry, n_kv, d=128) -> float:
-    """Microseconds of the attention kernel for a cut.  The blocks go out largest first, unit c taking blocks c and
-    c + 256 and later blocks going where least is left; the units share the memory evenly (a unit with one block gets as
-    much as one with two), so a step ends with its fullest unit, which reads alone at the end at what a unit can take."""
+    """Microseconds of the attention kernel for a cut.  Unit c takes blocks c and c + 256 of the records' order (the
+    largest 256 pieces, then the next 256 from the smallest up, so that a long first piece meets a short second one), and
+    later blocks go where least is left; the units share the memory evenly (a unit with one block gets as much as one
+    with two), so a step ends with its fullest unit, which reads alone at the end at what a unit can take."""
     s = np.repeat(sizes_per_entry[sizes_per_entry > 0], n_kv).astype(np.float64)
     s = -np.sort(-s)
     U = PIECE_UNITS
     load = np.zeros(U)
-    for r0 in (0, U):
-        chunk = s[r0:r0 + U]
-        load[:chunk.shape[0]] += chunk
+    load[:min(U, s.shape[0])] += s[:U]
+    second = s[U:2 * U][::-1]                                # (the second round goes out smallest first: decode_pieces)
+    load[:second.shape[0]] += second
     for r0 in range(2 * U, s.shape[0], U):
         chunk = s[r0:r0 + U]
         load = np.sort(load)
@@ -754,8 +755,8 @@ def decode_pieces(kv_len, n_kv: int, window: int = 0, capacity: Optional[int] = 
     compute units have even shares whatever the requests' lengths are (with one number of parts for all entries, a step
     takes as long as its longest request's part).  ``kv_len`` [S]: keys of every entry after this step.  Returns int32
     [capacity, 8] records { entry, kv head, first and end block of 32 keys (counted from the first block the entry's
-    window sees), number of the part, parts of the (entry, kv head), workspace slot of its first part, kv_len }, largest
-    pieces first, entry -1 in the unused ones.
+    window sees), number of the part, parts of the (entry, kv head), workspace slot of its first part, kv_len }, the
+    largest pieces first (see below for the order), entry -1 in the unused ones.
 
     Entries are cut into parts of at most W blocks, W being the whole step's blocks over the 256 compute units or over
     twice as many, the parts of an entry even or W and a rest, or they are not cut at all: whichever of the five gives
@@ -774,6 +775,13 @@ def decode_pieces(kv_len, n_kv: int, window: int = 0, capacity: Optional[int] = 
         raise KernelError("decode_pieces: %d pieces for %d records" % (count * n_kv, capacity))
     order = np.argsort(-sizes[ent, part], kind="stable")
     ent, part = ent[order], part[order]
+    # The records' order is the blocks' order, and the first 2 x 256 blocks go to the 256 units in turn: the largest 256
+    # pieces first, then the next 256 / n_kv from the smallest up (measured against all in falling order, requests of 128
+    # to 2560 keys: 55.2 / 56.8 us at 40 requests, 84.0 / 86.3 at 64, 24.4 / 25.4 at 16; even lengths: no difference).
+    per = max(1, PIECE_UNITS // n_kv)
+    if count > per:
+        second = slice(per, min(count, 2 * per))
+        ent[second], part[second] = ent[second][::-1].copy(), part[second][::-1].copy()
     # workspace slots: the parts of an (entry, kv head) lie together, entries and heads in order
     first_slot = (np.cumsum(parts) - parts) * n_kv
     rec = np.full((capacity, PIECE_RECORD), -1, dtype=np.int32)

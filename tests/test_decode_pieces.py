@@ -12,7 +12,13 @@ def _check(kv_len, n_kv, window):
     live = rec[rec[:, 0] >= 0]
     assert (rec[len(live):] == -1).all(), "unused records come last and say so"
     sizes = live[:, 3] - live[:, 2]
-    assert (sizes > 0).all() and (np.diff(sizes) <= 0).all(), "no empty piece; largest first"
+    assert (sizes > 0).all(), "no empty piece"
+    # the order of the blocks: the largest 256 pieces, then the next 256 from the smallest up (a unit's second block
+    # evens out its first), then what is left, falling
+    per = max(1, ops.PIECE_UNITS // n_kv) * n_kv
+    assert (np.diff(sizes[:per]) <= 0).all() and (np.diff(sizes[per:2 * per]) >= 0).all() and (np.diff(sizes[2 * per:]) <= 0).all()
+    if len(sizes) > per:
+        assert sizes[:per].min() >= sizes[per:].max() and (len(sizes) <= 2 * per or sizes[per:2 * per].min() >= sizes[2 * per:].max())
     slots = set()
     for s, kvl in enumerate(kv_len):
         p0 = kvl - 1
