@@ -668,7 +668,7 @@ def _piece_sizes(nblk, width, even):
     instead of 12, 12, 13)."""
     n = nblk.astype(np.int64)
     idx = np.arange(DECODE_MAX_SPLITS, dtype=np.int64)[None, :]
-    w = np.full_like(n, width)
+    w = np.broadcast_to(np.asarray(width, dtype=np.int64), n.shape).copy()      # (one width, or one per entry)
     if even:
         w = np.maximum(1, -(-n // np.maximum(1, -(-n // width))))
     full = n // w
@@ -704,13 +704,41 @@ def _estimated_time(sizes_per_entry, n_kv, d=128) -> float:
     return t + PIECE_START_US + PIECE_ROUND_US * max(0, -(-int(s.shape[0]) // (2 * U)) - 1)
 
 
+def _fill_widths(nblk, n_kv):
+    """Widths per entry for the cut that fills the units in two rounds: the longest entries, as many as give the units
+    their first blocks (cut only where longer than a unit's even share), and the others cut so finely that they make
+    about one second block per unit: 40 requests of one length are 32 whole and 8 in four parts each, and every unit
+    has a whole entry and a quarter.  Never more second blocks than units, in coarser parts if need be (44 requests: 32
+    whole and 12 in two parts each, not in three: a third round costs more than the uneven second).  None if the first
+    round takes all entries."""
+    n = nblk.astype(np.int64)
+    total = int(n.sum()) * n_kv
+    share = max(1, -(-total // PIECE_UNITS))
+    floor = -(-n // DECODE_MAX_SPLITS)
+    first_parts = -(-n // np.maximum(share, floor))
+    order = np.argsort(-n, kind="stable")
+    taken = np.cumsum(first_parts[order]) * n_kv
+    first = np.zeros(n.shape[0], dtype=bool)
+    first[order[:int(np.searchsorted(taken, PIECE_UNITS, side="left")) + 1]] = True
+    if first.all():
+        return None
+    rest = int(n[~first].sum()) * n_kv
+    fine = max(PIECE_MIN_BLOCKS, -(-rest // PIECE_UNITS))
+    longest = int(n[~first].max())
+    for parts in range(DECODE_MAX_SPLITS, 0, -1):
+        fine = max(fine, -(-longest // parts))
+        if int((-(-n[~first] // fine)).sum()) * n_kv <= PIECE_UNITS:
+            break
+    return np.where(first, np.maximum(share, floor), np.maximum(fine, floor))
+
+
 _piece_choices = {}
 
 
 def _piece_choice(nblk, n_kv, d=128):
-    """How a step whose entries have ``nblk`` blocks of keys is cut: None (not at all) or (W, even): parts of at most W
+    """How a step whose entries have ``nblk`` blocks of keys is cut: None (not at all), (W, even): parts of at most W
     blocks, W being the whole step's blocks over the compute units or over twice as many, an entry's parts of one size
-    or W and a rest: whichever of the five has the shortest estimated time.  Decided from the lengths rounded up to 8
+    or W and a rest, or ("fill", True) (``_fill_widths``): whichever of the six has the shortest estimated time.  Decided from the lengths rounded up to 8
     blocks, so that a step is always cut the same way and the choice is looked up in most steps (a request's rounded
     length changes once in 256 steps); the last choices are kept."""
     coarse = nblk >> 3
@@ -736,6 +764,13 @@ def _piece_choice(nblk, n_kv, d=128):
                 t = _estimated_time(sizes, n_kv, d) + PIECE_MERGE_US
                 if t < best[0]:
                     best = (t, (width, even))
+    widths = _fill_widths(rounded, n_kv)
+    if widths is not None:
+        sizes, parts = _piece_sizes(rounded, widths, True)
+        if int(parts.max(initial=1)) > 1:
+            t = _estimated_time(sizes, n_kv, d) + PIECE_MERGE_US
+            if t < best[0]:
+                best = (t, ("fill", True))
     if len(_piece_choices) >= 64:
         _piece_choices.pop(next(iter(_piece_choices)))
     _piece_choices[key] = best[1]
@@ -745,6 +780,9 @@ def _piece_choice(nblk, n_kv, d=128):
 def _piece_plan(nblk, n_kv, d=128):
     """(sizes [S, 16], parts [S]) for entries of ``nblk`` blocks (``_piece_choice``, ``_piece_sizes``)."""
     choice = _piece_choice(nblk, n_kv, d)
+    if choice is not None and choice[0] == "fill":
+        widths = _fill_widths(nblk, n_kv)
+        choice = None if widths is None else (widths, True)
     if choice is None:
         return nblk[:, None] * (np.arange(DECODE_MAX_SPLITS)[None, :] == 0), np.ones(nblk.shape[0], dtype=np.int64)
     return _piece_sizes(nblk, choice[0], choice[1])
