@@ -60,6 +60,19 @@ def test_few_requests_are_cut_to_fill_the_chip():
     assert len(live) == 256 and (live[:, 5] == 4).all()
 
 
+def test_a_few_requests_more_than_fill_the_chip_give_every_unit_a_whole_entry_and_a_part():
+    """40 requests of one length and 8 kv heads are 320 (entry, kv head) pairs for 256 units: 32 requests stay whole (a
+    unit's first block), 8 are cut in four (a quarter as every unit's second block), 512 blocks in all."""
+    live = _check(np.full(40, 1153), 8, 0)
+    parts = {s: int(live[live[:, 0] == s][0, 5]) for s in range(40)}
+    assert sorted(parts.values()) == [1] * 32 + [4] * 8 and len(live) == 512
+    sizes = live[:, 3] - live[:, 2]
+    assert (sizes[:256] == 37).all() and sizes[256:].max() <= 10
+    # 44 requests: a third part each would make more second blocks than units
+    live = _check(np.full(44, 1153), 8, 0)
+    assert sorted(int(live[live[:, 0] == s][0, 5]) for s in range(44)) == [1] * 32 + [2] * 12 and len(live) == 448
+
+
 def test_a_long_request_among_short_ones_is_cut_and_the_short_ones_are_not():
     kv_len = np.array([6000] + [200] * 40)
     live = _check(kv_len, 8, 0)
