@@ -663,9 +663,9 @@ def decode_pieces_capacity(entries: int, n_kv: int) -> int:
 def _piece_sizes(nblk, width, even):
     """How entries of ``nblk`` blocks of 32 keys are cut into parts of at most ``width`` blocks: [entries, 16] sizes (0:
     no such part) and the numbers of parts.  Parts of one size and the rest (the last part, which also prepares and
-    stores the new key, is the shortest); a rest shorter than half of what a part may be joins the part before it.  ``even``: the
-    size is the least that gives the entry no more parts than ``width`` does (37 blocks at width 12: 10, 10, 10, 7
-    instead of 12, 12, 13)."""
+    stores the new key, is the shortest); a rest shorter than half of what a part may be joins the part before it.
+    ``even``: the size is the least that gives the entry no more parts than ``width`` does (37 blocks at width 12: 10,
+    10, 10, 7 instead of 12, 12, 13).  ``width``: one for all entries, or one per entry."""
     n = nblk.astype(np.int64)
     idx = np.arange(DECODE_MAX_SPLITS, dtype=np.int64)[None, :]
     w = np.broadcast_to(np.asarray(width, dtype=np.int64), n.shape).copy()      # (one width, or one per entry)
@@ -738,9 +738,9 @@ _piece_choices = {}
 def _piece_choice(nblk, n_kv, d=128):
     """How a step whose entries have ``nblk`` blocks of keys is cut: None (not at all), (W, even): parts of at most W
     blocks, W being the whole step's blocks over the compute units or over twice as many, an entry's parts of one size
-    or W and a rest, or ("fill", True) (``_fill_widths``): whichever of the six has the shortest estimated time.  Decided from the lengths rounded up to 8
-    blocks, so that a step is always cut the same way and the choice is looked up in most steps (a request's rounded
-    length changes once in 256 steps); the last choices are kept."""
+    or W and a rest, or ("fill", True) (``_fill_widths``): whichever of the six has the shortest estimated time.
+    Decided from the lengths rounded up to 8 blocks, so that a step is always cut the same way and the choice is looked
+    up in most steps (a request's rounded length changes once in 256 steps); the last choices are kept."""
     coarse = nblk >> 3
     key = (coarse.tobytes(), n_kv, d, PIECE_UNITS, PIECE_MIN_BLOCKS, PIECE_START_US, PIECE_MERGE_US, PIECE_ROUND_US)
     if key in _piece_choices:
