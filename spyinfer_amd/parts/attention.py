@@ -18,7 +18,7 @@ import numpy as np
 import torch
 
 from ..cache.spec import PagedKV
-from ..kernels import ops
+from ..kernels import key_pieces, ops
 from ..weights.loader import WeightSpec
 from .base import Mixer, PositionEncoding
 
@@ -62,12 +62,12 @@ def plan_attention_tiles(batch, group_size: int, big_rows: int = 0, key_parts: b
 
 
 def plan_decode_pieces(batch, n_kv: int, window: int, head_dim: int) -> None:
-    """Adds to the arrays of a step of single tokens its keys cut into pieces of even size (``ops.decode_pieces``), for
+    """Adds to the arrays of a step of single tokens its keys cut into pieces of even size (``key_pieces.decode_pieces``), for
     layers of ``n_kv`` kv heads of ``head_dim`` and this window.  The array's length follows the numbers of entries and
     heads alone."""
     note = ("decode_pieces", n_kv, window, head_dim)
     if note not in batch.shared:
-        batch.add_array("decode_pieces_%d_%d_%d" % note[1:], ops.decode_pieces(batch.host_array("kv_len"), n_kv, window, head_dim=head_dim))
+        batch.add_array("decode_pieces_%d_%d_%d" % note[1:], key_pieces.decode_pieces(batch.host_array("kv_len"), n_kv, window, head_dim=head_dim))
         batch.shared[note] = True
 
 
@@ -82,7 +82,7 @@ def attention_meta(batch, group: int, group_size: int, big_rows: int = 0) -> ops
         if counts is not None:
             tiles = {kind: (batch.array("tile_entry_%s_%d_%d" % (kind, group_size, big_rows)),
                             batch.array("tile_row0_%s_%d_%d" % (kind, group_size, big_rows)), n) for kind, n in counts.items()}
-        pieces = {key[1:]: batch.array("decode_pieces_%d_%d_%d" % key[1:]).view(-1, ops.PIECE_RECORD)
+        pieces = {key[1:]: batch.array("decode_pieces_%d_%d_%d" % key[1:]).view(-1, key_pieces.PIECE_RECORD)
                   for key in batch.shared if isinstance(key, tuple) and key[0] == "decode_pieces"}
         meta = ops.AttentionMeta(batch.array("cu_q"), batch.array("pos0"), batch.array("kv_len"), batch.block_table(group),
                                  batch.array("token_entry"), batch.array("positions"), batch.S, batch.T, batch.max_blocks[group],
@@ -149,7 +149,7 @@ class PagedAttention(Mixer):
         out = {"tile_entry_small_%d" % G: entries, "tile_row0_small_%d" % G: entries}
         if ops.decode_pieces_ok(entries, entries, torch.bfloat16, self.num_kv_heads, self.head_dim):
             out["decode_pieces_%d_%d_%d" % (self.num_kv_heads, int(self.window or 0), self.head_dim)] = \
-                ops.decode_pieces_capacity(entries, self.num_kv_heads) * ops.PIECE_RECORD
+                key_pieces.decode_pieces_capacity(entries, self.num_kv_heads) * key_pieces.PIECE_RECORD
         return out
 
     def _rotated_whole(self) -> bool:

@@ -1,21 +1,21 @@
-"""The host's cut of a decode step's keys into pieces (``ops.decode_pieces``): every block of 32 keys of every (entry,
+"""The host's cut of a decode step's keys into pieces (``key_pieces.decode_pieces``): every block of 32 keys of every (entry,
 kv head) lies in exactly one piece, whatever the lengths, the window and the numbers of entries and heads are."""
 import numpy as np
 import pytest
 
-from spyinfer_amd.kernels import ops
+from spyinfer_amd.kernels import key_pieces
 
 
 def _check(kv_len, n_kv, window):
-    rec = ops.decode_pieces(kv_len, n_kv, window)
-    assert rec.dtype == np.int32 and rec.shape == (ops.decode_pieces_capacity(len(kv_len), n_kv), ops.PIECE_RECORD)
+    rec = key_pieces.decode_pieces(kv_len, n_kv, window)
+    assert rec.dtype == np.int32 and rec.shape == (key_pieces.decode_pieces_capacity(len(kv_len), n_kv), key_pieces.PIECE_RECORD)
     live = rec[rec[:, 0] >= 0]
     assert (rec[len(live):] == -1).all(), "unused records come last and say so"
     sizes = live[:, 3] - live[:, 2]
     assert (sizes > 0).all(), "no empty piece"
     # the order of the blocks: the largest 256 pieces, then the next 256 from the smallest up (a unit's second block
     # evens out its first), then what is left, falling
-    per = max(1, ops.PIECE_UNITS // n_kv) * n_kv
+    per = max(1, key_pieces.PIECE_UNITS // n_kv) * n_kv
     assert (np.diff(sizes[:per]) <= 0).all() and (np.diff(sizes[per:2 * per]) >= 0).all() and (np.diff(sizes[2 * per:]) <= 0).all()
     if len(sizes) > per:
         assert sizes[:per].min() >= sizes[per:].max() and (len(sizes) <= 2 * per or sizes[per:2 * per].min() >= sizes[2 * per:].max())
@@ -28,7 +28,7 @@ def _check(kv_len, n_kv, window):
             mine = live[(live[:, 0] == s) & (live[:, 1] == hk)]
             mine = mine[np.argsort(mine[:, 4])]
             parts = len(mine)
-            assert 1 <= parts <= ops.DECODE_MAX_SPLITS
+            assert 1 <= parts <= key_pieces.MAX_PARTS
             assert (mine[:, 4] == np.arange(parts)).all() and (mine[:, 5] == parts).all() and (mine[:, 7] == kvl).all()
             assert mine[0, 2] == 0 and mine[-1, 3] == nblk and (mine[1:, 2] == mine[:-1, 3]).all(), "the parts tile the entry's blocks"
             assert (mine[:, 6] == mine[0, 6]).all(), "one first slot for all parts of an (entry, kv head)"
@@ -78,13 +78,13 @@ def test_a_long_request_among_short_ones_is_cut_and_the_short_ones_are_not():
     live = _check(kv_len, 8, 0)
     assert live[live[:, 0] == 0][0, 5] > 4 and (live[live[:, 0] > 0][:, 5] == 1).all()
     # no piece is far above an even share of the step's blocks
-    share = (live[:, 3] - live[:, 2]).sum() / ops.PIECE_UNITS
-    assert (live[:, 3] - live[:, 2]).max() <= 1.5 * share + ops.PIECE_MIN_BLOCKS
+    share = (live[:, 3] - live[:, 2]).sum() / key_pieces.PIECE_UNITS
+    assert (live[:, 3] - live[:, 2]).max() <= 1.5 * share + key_pieces.PIECE_MIN_BLOCKS
 
 
 def test_the_longest_request_never_has_more_parts_than_the_kernel_merges():
     live = _check(np.array([100000, 5]), 1, 0)
-    assert live[:, 5].max() <= ops.DECODE_MAX_SPLITS
+    assert live[:, 5].max() <= key_pieces.MAX_PARTS
 
 
 def test_a_window_counts_the_blocks_it_sees_only():

@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 import torch
 
+from spyinfer_amd.kernels import key_pieces
 from tests import replay_cases as rc
 from tests.configs import INIT, TINY_A, TINY_B, TINY_C, TINY_D, TINY_E
 from tests.gpu_util import require_gpu
@@ -916,7 +917,7 @@ def test_requests_of_uneven_lengths_decode_under_graphs(tmp_path):
         got = runner.step([StepEntry(c, [q[n + i]], [0]) for c, q, n in zip(caches, seqs, lengths)]).cpu()
         want = torch.stack([r[n + i] for r, n in zip(ref, lengths)])
         assert torch.allclose(got, want, **TOL["bfloat16"]), "step %d: off by %s" % (i, (got - want).abs().max(1).values.tolist())
-        rec = ops.decode_pieces([n + i + 1 for n in lengths], raw["num_key_value_heads"], 0, head_dim=raw["head_dim"])
+        rec = key_pieces.decode_pieces([n + i + 1 for n in lengths], raw["num_key_value_heads"], 0, head_dim=raw["head_dim"])
         cuts.add(tuple(rec[rec[:, 4] == 0][:, 5].tolist()))
     assert runner.graph_replays >= steps - 2 and len(runner._graphs) == 1
     assert len(cuts) > 1 and max(max(c) for c in cuts) > 1 and min(min(c) for c in cuts) == 1
@@ -977,7 +978,7 @@ def test_a_request_of_4200_tokens_decodes_under_graphs(dtype, long_model):
         parts.add(ops.key_parts_for(long_n + i + 1))
         if dtype == "bfloat16":
             # how the host cuts this step's keys: the long request in a dozen parts and more, the short one whole
-            rec = ops.decode_pieces([long_n + i + 1, short_n + i + 1], TINY_E["num_key_value_heads"], 0, head_dim=TINY_E["head_dim"])
+            rec = key_pieces.decode_pieces([long_n + i + 1, short_n + i + 1], TINY_E["num_key_value_heads"], 0, head_dim=TINY_E["head_dim"])
             assert rec[rec[:, 0] == 0][0, 5] >= 12 and rec[rec[:, 0] == 1][0, 5] == 1
         want = torch.stack([ref[0][long_n + i], ref[1][short_n + i]])
         assert torch.allclose(got, want, **tol), "decode step %d (%s): off by %g / %g" % (

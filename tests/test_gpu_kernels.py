@@ -6,6 +6,7 @@ import math
 import pytest
 import torch
 
+from spyinfer_amd.kernels import key_pieces
 from tests.gpu_util import close, require_gpu
 
 pytestmark = pytest.mark.gpu
@@ -763,7 +764,7 @@ FUSED_CASES = [
 def _with_pieces(meta, kv_len, n_kv, window, d, dev):
     """The step's keys cut on the host, as the attention part plans them."""
     from spyinfer_amd.kernels import ops
-    rec = ops.decode_pieces(kv_len, n_kv, int(window or 0), head_dim=d)
+    rec = key_pieces.decode_pieces(kv_len, n_kv, int(window or 0), head_dim=d)
     meta.pieces = {(n_kv, int(window or 0), d): torch.from_numpy(rec).to(dev)}
     return rec
 
@@ -789,10 +790,10 @@ def test_attention_taking_the_raw_product(case, wdtype, keys_per_part, cut, monk
     if cut == "by_the_host":
         if d > 128:
             pytest.skip("head sizes beyond 128 are not cut by the host")
-        monkeypatch.setattr(ops, "PIECE_MIN_BLOCKS", keys_per_part // 32)
+        monkeypatch.setattr(key_pieces, "PIECE_MIN_BLOCKS", keys_per_part // 32)
         if keys_per_part < 256:                  # as many parts as there can be
             for name, value in (("PIECE_UNITS", 64 * len(cached)), ("PIECE_START_US", 0.0), ("PIECE_MERGE_US", 0.0), ("PIECE_ROUND_US", 0.0)):
-                monkeypatch.setattr(ops, name, value)
+                monkeypatch.setattr(key_pieces, name, value)
         rec = _with_pieces(meta, [a + 1 for a in cached], n_kv, window, d, dev)
         assert keys_per_part == 256 or max(cached) < 128 or rec[:, 5].max() > 1
     T = len(entries)

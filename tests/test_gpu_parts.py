@@ -4,6 +4,7 @@ import math
 import pytest
 import torch
 
+from spyinfer_amd.kernels import key_pieces
 from tests.gpu_util import close, require_gpu
 from tests.plain import qwen3_plain as P
 
@@ -153,7 +154,7 @@ def test_attention_part_decoding_long_requests_with_the_keys_cut_by_the_host(win
     cut = set()
     for i in range(steps):
         out, batch = run([(c, 1) for c in caches], [x[n + i:n + i + 1] for x, n in zip(xs, lengths)])
-        rec = batch.host_array("decode_pieces_%d_%d_%d" % (nkv, window or 0, d)).reshape(-1, ops.PIECE_RECORD)
+        rec = batch.host_array("decode_pieces_%d_%d_%d" % (nkv, window or 0, d)).reshape(-1, key_pieces.PIECE_RECORD)
         cut.add((int(rec[rec[:, 0] == 0][0, 5]), int(rec[rec[:, 0] == 1][0, 5])))
         close(out, torch.stack([r[n + i] for r, n in zip(refs, lengths)]), dtype, scale=2.0, what="step %d" % i)
     assert all(long > short >= 1 for long, short in cut), cut

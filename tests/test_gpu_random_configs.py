@@ -15,6 +15,7 @@ import random
 import pytest
 import torch
 
+from spyinfer_amd.kernels import key_pieces
 from tests import replay_cases as rc
 from tests.configs import INIT
 from tests.gpu_util import require_gpu
@@ -112,7 +113,7 @@ def test_random_decode_steps_of_uneven_lengths(seed, tmp_path):
         got = runner.step([StepEntry(c, [q[n + i]], [0]) for c, q, n in zip(caches, seqs, lengths)]).cpu()
         want = torch.stack([r[i] for r in ref])
         assert torch.allclose(got, want, atol=atol, rtol=TOL["bfloat16"]["rtol"]), "step %d: off by %s" % (i, (got - want).abs().max(1).values.tolist())
-        rec = ops.decode_pieces([n + i + 1 for n in lengths], n_kv, 0, head_dim=d)
+        rec = key_pieces.decode_pieces([n + i + 1 for n in lengths], n_kv, 0, head_dim=d)
         cut = cut or int(rec[:, 5].max()) > 1
     assert ops.workspace_counters_clean(dev)
     assert cut or max(lengths) < 300, "a long request among these is cut into parts"
