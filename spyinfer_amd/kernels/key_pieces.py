@@ -12,7 +12,8 @@ from typing import Optional
 
 import numpy as np
 
-MAX_PARTS = 16              # most parts of an (entry, kv head) (the merging block's time grows with them)
+MAX_PARTS = 32              # most parts of an (entry, kv head): what the kernel's merging block takes (8 kv heads of one long
+                            # request give every compute unit a block only in 32 parts: 38 000 keys 39.5 us against 53.7 in 16)
 PIECE_UNITS = 256           # compute units that the pieces are dealt to; each runs two blocks at a time
 PIECE_MIN_BLOCKS = 8        # a part wants this many blocks of 32 keys at least (measured at 1100 keys, 1 to 4 requests: 4-8 parts best)
 PIECE_RECORD = 8            # ints per record
@@ -21,6 +22,7 @@ PIECE_RECORD = 8            # ints per record
 # fastest of those measured, to within the timings' noise, in every case):
 PIECE_START_US = 7.0        # from the kernel's start to a block's first keys, and its end
 PIECE_MERGE_US = 3.0        # the way of the parts through memory, once per step that cuts any entry
+PIECE_MERGE_MORE_US = 2.5   # each eight parts beyond sixteen of the entry with the most (the merging block asks for eight at a time)
 PIECE_ROUND_US = 4.0        # each further round of blocks on the units beyond the two that are there from the start
 PIECE_BLOCK_US = 0.45       # a unit's time for a block of 32 keys (16 KB) while it reads alone
 PIECE_SHARED_US = 0.56      # what all units reading at once add to it (the two add as squares)
@@ -33,9 +35,9 @@ def decode_pieces_capacity(entries: int, n_kv: int) -> int:
 
 
 def _piece_sizes(nblk, width, even):
-    """How entries of ``nblk`` blocks of 32 keys are cut into parts of at most ``width`` blocks: [entries, 16] sizes (0:
-    no such part) and the numbers of parts.  Parts of one size and the rest (the last part, which also prepares and
-    stores the new key, is the shortest); a rest shorter than half of what a part may be joins the part before it.
+    """How entries of ``nblk`` blocks of 32 keys are cut into parts of at most ``width`` blocks: [entries, MAX_PARTS]
+    sizes (0: no such part) and the numbers of parts.  Parts of one size and the rest (the last part, which also prepares
+    and stores the new key, is the shortest); a rest shorter than half of what a part may be joins the part before it.
     ``even``: the size is the least that gives the entry no more parts than ``width`` does (37 blocks at width 12: 10,
     10, 10, 7 instead of 12, 12, 13).  ``width``: one for all entries, or one per entry."""
     n = nblk.astype(np.int64)
@@ -76,6 +78,11 @@ def _estimated_time(sizes_per_entry, n_kv, d=128) -> float:
     return t + PIECE_START_US + PIECE_ROUND_US * max(0, -(-int(s.shape[0]) // (2 * U)) - 1)
 
 
+def _merge_time(parts) -> float:
+    """Microseconds that a step's merges add: the last block of the entry with the most parts asks for eight at a time."""
+    return PIECE_MERGE_US + PIECE_MERGE_MORE_US * max(0, -(-int(parts.max(initial=1)) // 8) - 2)
+
+
 def _fill_widths(nblk, n_kv):
     """Widths per entry for the cut that fills the units in two rounds: the longest entries, as many as give the units
     their first blocks (cut only where longer than a unit's even share), and the others cut so finely that they make
@@ -109,12 +116,13 @@ _piece_choices = {}
 
 def _piece_choice(nblk, n_kv, d=128):
     """How a step whose entries have ``nblk`` blocks of keys is cut: None (not at all), (W, even): parts of at most W
-    blocks, W being the whole step's blocks over the compute units or over twice as many, an entry's parts of one size
-    or W and a rest, or ("fill", True) (``_fill_widths``): whichever of the six has the shortest estimated time.
+    blocks, W being the whole step's blocks over the compute units or over twice as many (and no less than gives the
+    longest entry 16 parts, or 32), an entry's parts of one size or W and a rest, or ("fill", True) (``_fill_widths``):
+    whichever has the shortest estimated time.
     Decided from the lengths rounded up to 8 blocks, so that a step is always cut the same way and the choice is looked
     up in most steps (a request's rounded length changes once in 256 steps); the last choices are kept."""
     coarse = nblk >> 3
-    key = (coarse.tobytes(), n_kv, d, PIECE_UNITS, PIECE_MIN_BLOCKS, PIECE_START_US, PIECE_MERGE_US, PIECE_ROUND_US)
+    key = (coarse.tobytes(), n_kv, d, MAX_PARTS, PIECE_UNITS, PIECE_MIN_BLOCKS, PIECE_START_US, PIECE_MERGE_US, PIECE_ROUND_US)
     if key in _piece_choices:
         return _piece_choices[key]
     rounded = (coarse << 3) + 7
@@ -125,22 +133,23 @@ def _piece_choice(nblk, n_kv, d=128):
         # millisecond a step)
         _piece_choices[key] = None
         return None
-    floor = max(1, -(-int(rounded.max(initial=1)) // MAX_PARTS))
+    longest = int(rounded.max(initial=1))
     whole = rounded[:, None] * (np.arange(MAX_PARTS)[None, :] == 0)
     best = (_estimated_time(whole, n_kv, d), None)
-    for k in (1, 2):
-        width = max(PIECE_MIN_BLOCKS, floor, -(-total // (PIECE_UNITS * k)))
+    # (the longest entry in at most 16 parts as well as in at most MAX_PARTS: more than 16 cost the merge further round trips)
+    widths = {max(PIECE_MIN_BLOCKS, -(-longest // most), -(-total // (PIECE_UNITS * k))) for k in (1, 2) for most in (16, MAX_PARTS)}
+    for width in sorted(widths):
         for even in (True, False):
             sizes, parts = _piece_sizes(rounded, width, even)
             if int(parts.max(initial=1)) > 1:
-                t = _estimated_time(sizes, n_kv, d) + PIECE_MERGE_US
+                t = _estimated_time(sizes, n_kv, d) + _merge_time(parts)
                 if t < best[0]:
                     best = (t, (width, even))
-    widths = _fill_widths(rounded, n_kv)
-    if widths is not None:
-        sizes, parts = _piece_sizes(rounded, widths, True)
+    per_entry = _fill_widths(rounded, n_kv)
+    if per_entry is not None:
+        sizes, parts = _piece_sizes(rounded, per_entry, True)
         if int(parts.max(initial=1)) > 1:
-            t = _estimated_time(sizes, n_kv, d) + PIECE_MERGE_US
+            t = _estimated_time(sizes, n_kv, d) + _merge_time(parts)
             if t < best[0]:
                 best = (t, ("fill", True))
     if len(_piece_choices) >= 64:
@@ -170,7 +179,7 @@ def decode_pieces(kv_len, n_kv: int, window: int = 0, capacity: Optional[int] = 
 
     Entries are cut into parts of at most W blocks, W being the whole step's blocks over the 256 compute units or over
     twice as many, the parts of an entry even or W and a rest, or the longest entries whole and the others fine
-    (``_fill_widths``), or they are not cut at all: whichever of the six gives the shortest estimated time."""
+    (``_fill_widths``), or they are not cut at all: whichever gives the shortest estimated time (``_piece_choice``)."""
     kv_len = np.asarray(kv_len, dtype=np.int64)
     S = int(kv_len.shape[0])
     capacity = decode_pieces_capacity(S, n_kv) if capacity is None else capacity

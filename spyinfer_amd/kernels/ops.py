@@ -619,7 +619,7 @@ class AttentionMeta:
 
 
 MFMA_ATTENTION = True      # False forces the plain kernel for bfloat16 too (the kernel tests flip it; nothing else does)
-DECODE_MAX_SPLITS = key_pieces.MAX_PARTS      # most key parts of a tile (the merge kernel's time grows with them)
+DECODE_MAX_SPLITS = 16      # most key parts of a tile where the grid cuts them (the merge's time grows with them)
 DECODE_KEYS_PER_SPLIT = 256  # a part wants this many keys at least (measured at 1100 keys, 1 to 4 requests: 4-8 parts best)
 
 

@@ -947,11 +947,12 @@ def long_model(tmp_path_factory):
     return folder, seqs, ref
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_request_of_4200_tokens_decodes_under_graphs(dtype, long_model):
+@pytest.mark.parametrize("dtype,cut", [("float32", "as measured"), ("bfloat16", "as measured"), ("bfloat16", "finest")])
+def test_a_request_of_4200_tokens_decodes_under_graphs(dtype, cut, long_model, monkeypatch):
     """One long request beside a short one, decode steps recorded and replayed: block tables of the fixed width that
     4608 positions need (288 pages), the long request's keys in 16 parts (float32: the plain kernel reads them in one) or
-    in the dozen and more pieces that the host cuts them into beside the short request, which stays whole.  A part of the keys that is lost, read through
+    in the dozen and more pieces that the host cuts them into beside the short request, which stays whole ("finest": in
+    more than sixteen, which the merging block takes in three and four rounds).  A part of the keys that is lost, read through
     a wrong page or merged wrongly moves the logits far beyond the tolerance (the fixture asserts it on the plain pass).
     Logits of every decode step against the plain pass of the whole sequences."""
     from spyinfer_amd.engine.batch import StepEntry
@@ -960,6 +961,9 @@ def test_a_request_of_4200_tokens_decodes_under_graphs(dtype, long_model):
     dev = require_gpu()
     folder, seqs, ref = long_model
     long_n, short_n, steps = LONG_N, SHORT_N, LONG_STEPS
+    if cut == "finest":
+        monkeypatch.setattr(key_pieces, "PIECE_MIN_BLOCKS", 4)
+        monkeypatch.setattr(key_pieces, "PIECE_MERGE_MORE_US", 0.0)
     runner = ModelRunner(load_model(folder, dtype, dev), dtype, dev, 16, 300, 2, enforce_eager=False, max_model_len=4608)
     assert runner.fixed_max_blocks == 288
     caches = [runner.manager.admit(i) for i in range(2)]
@@ -979,7 +983,7 @@ def test_a_request_of_4200_tokens_decodes_under_graphs(dtype, long_model):
         if dtype == "bfloat16":
             # how the host cuts this step's keys: the long request in a dozen parts and more, the short one whole
             rec = key_pieces.decode_pieces([long_n + i + 1, short_n + i + 1], TINY_E["num_key_value_heads"], 0, head_dim=TINY_E["head_dim"])
-            assert rec[rec[:, 0] == 0][0, 5] >= 12 and rec[rec[:, 0] == 1][0, 5] == 1
+            assert rec[rec[:, 0] == 0][0, 5] >= (20 if cut == "finest" else 12) and rec[rec[:, 0] == 1][0, 5] == 1
         want = torch.stack([ref[0][long_n + i], ref[1][short_n + i]])
         assert torch.allclose(got, want, **tol), "decode step %d (%s): off by %g / %g" % (
             i, "replayed" if i >= 2 else "eager or captured", (got[0] - want[0]).abs().max(), (got[1] - want[1]).abs().max())

@@ -792,10 +792,13 @@ def test_attention_taking_the_raw_product(case, wdtype, keys_per_part, cut, monk
             pytest.skip("head sizes beyond 128 are not cut by the host")
         monkeypatch.setattr(key_pieces, "PIECE_MIN_BLOCKS", keys_per_part // 32)
         if keys_per_part < 256:                  # as many parts as there can be
-            for name, value in (("PIECE_UNITS", 64 * len(cached)), ("PIECE_START_US", 0.0), ("PIECE_MERGE_US", 0.0), ("PIECE_ROUND_US", 0.0)):
+            for name, value in (("PIECE_UNITS", 64 * len(cached)), ("PIECE_START_US", 0.0), ("PIECE_MERGE_US", 0.0), ("PIECE_MERGE_MORE_US", 0.0),
+                                ("PIECE_ROUND_US", 0.0)):
                 monkeypatch.setattr(key_pieces, name, value)
         rec = _with_pieces(meta, [a + 1 for a in cached], n_kv, window, d, dev)
         assert keys_per_part == 256 or max(cached) < 128 or rec[:, 5].max() > 1
+        # (more than sixteen parts: the merging block's third and fourth round of eight)
+        assert keys_per_part == 256 or max(cached) < 600 or window or rec[:, 5].max() > 16
     T = len(entries)
     qkv = rnd((T, (n_q + 2 * n_kv) * d), dtype, "cpu", 60 + case)
     qw = (1 + 0.2 * rnd((d,), torch.float32, "cpu", 61)).to(wdtype) if norm else None
@@ -841,7 +844,7 @@ def test_attention_taking_the_raw_product(case, wdtype, keys_per_part, cut, monk
 
 
 @pytest.mark.parametrize("case", [(16, 4, 128, 16, 40, 2600, None), (8, 8, 64, 32, 70, 900, None), (32, 8, 128, 16, 9, 6000, 1500),
-                                  (16, 2, 128, 16, 130, 400, None)])
+                                  (16, 2, 128, 16, 130, 400, None), (16, 8, 128, 16, 3, 16000, None), (8, 8, 64, 16, 2, 16000, None)])
 def test_attention_of_requests_of_uneven_lengths_cut_by_the_host(case):
     """Dozens of single tokens whose requests have a few to thousands of keys: the host cuts the long ones into pieces,
     leaves the short ones whole, and the kernel's blocks take one piece each.  Every entry's far keys carry weight.
@@ -858,6 +861,7 @@ def test_attention_of_requests_of_uneven_lengths_cut_by_the_host(case):
     _q, kc, vc, kept, cu, meta = _long_case(dtype, dev, n_q, n_kv, d, P, entries, seed=S)
     rec = _with_pieces(meta, [a + 1 for a in cached], n_kv, window, d, dev)
     assert rec[:, 5].max() > 1 and (rec[rec[:, 0] >= 0][:, 5] == 1).any(), "some entries cut, some whole"
+    assert S > 3 or rec[:, 5].max() > 24, "a long request beside one or two others: more parts than sixteen"
     qkv = rnd((S, (n_q + 2 * n_kv) * d), dtype, "cpu", 7)
     qw, kw = ((1 + 0.2 * rnd((d,), torch.float32, "cpu", 8 + i)).to(dtype) for i in range(2))
     rope = RotaryEmbedding(d, theta, d)
