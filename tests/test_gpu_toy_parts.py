@@ -1,7 +1,8 @@
 """Parts that are not in the framework, defined here and put into a model without a change to the
 framework's files: a position encoding that is added to the embeddings, a feed-forward that routes
 every token to two of three experts, a norm that centres before it scales, and a run order in which
-one call reads the keys and values that another call stored.  The toy model is compared with a plain
+one call reads the keys and values that another call stored; a third kind of cache; other arrangements of the parts
+in a block.  Each toy model is compared with a plain
 forward pass of whole sequences written below, and with itself under other cuts of the same requests.
 It is a toy: no model of anyone's."""
 import dataclasses
@@ -339,3 +340,161 @@ def test_a_third_kind_of_cache_defined_in_a_test(dtype, tmp_path):
             rc.compare(rc.collect(out, steps, 101), ref, what="latent/%s/%s" % (mode, dtype), **TOL[dtype])
     finally:
         unregister_architecture("ToyLatentLM")
+
+
+# ---------------------------------------------------------------------------------------------
+# Other arrangements of norm, mixer and feed-forward in a block, defined here: one norm whose output both the mixer and
+# the feed-forward read, their results added to the stream together; and norms before AND behind each of the two.  The
+# toy model puts them between blocks of the framework's own arrangement, at widths whose decode steps fold the norms
+# into the products: so a block that prepares the next norm's input stands before one that does not know of that, and
+# behind one.
+
+ARR = dict(hidden=128, heads=4, kv=2, head_dim=64, inter=256, vocab=131, eps=1e-5, theta=1e4, positions=256)
+
+
+def _toy_arranged():
+    from spyinfer_amd.config import ModelConfig
+    from spyinfer_amd.kernels import ops
+    from spyinfer_amd.models import DecoderModel
+    from spyinfer_amd.parts import GatedMLP, LMHead, PagedAttention, PreNormBlock, RMSNorm, RotaryEmbedding, TokenEmbedding
+    from spyinfer_amd.parts.base import Block
+
+    class Arranged(Block):
+        """Parts by name under the layer's prefix; what a block must have beside ``forward``."""
+
+        def _named(self, prefix):
+            return [(part, prefix + "." + name) for name, part in self.parts.items()]
+
+        def weight_specs(self, prefix):
+            return [s for part, p in self._named(prefix) for s in part.weight_specs(p)]
+
+        def bind(self, prefix, weights):
+            for part, p in self._named(prefix):
+                part.bind(p, weights)
+
+        def capturable(self, batch):
+            return all(part.capturable(batch) for part in self.parts.values())
+
+    class ParallelBlock(Arranged):
+        """n = norm(h);  h += mixer(n) + ffn(n)."""
+
+        def __init__(self, norm, mixer, ffn):
+            self.parts = dict(input_layernorm=norm, self_attn=mixer, mlp=ffn)
+            self.norm, self.mixer, self.ffn = norm, mixer, ffn
+
+        def forward(self, resid, pending, batch, cache, store=True, next_norm=None):
+            # a prepared input of another block's norm means that the stream is complete: nothing is left to add
+            delta = None if isinstance(pending, ops.ScaledInput) else pending
+            n = self.norm.add_norm(resid, delta, batch.act_dtype)
+            a = self.mixer.forward(n, batch, cache, store)
+            f = self.ffn.forward(n, batch)
+            return resid, (a.float() + f.float()).to(batch.act_dtype)
+
+    class SandwichBlock(Arranged):
+        """h += post1(mixer(pre1(h)));  h += post2(ffn(pre2(h))): the norms behind act on the branch, not on the stream."""
+
+        def __init__(self, pre1, mixer, post1, pre2, ffn, post2):
+            self.parts = dict(input_layernorm=pre1, self_attn=mixer, post_mixer_layernorm=post1, pre_mlp_layernorm=pre2, mlp=ffn,
+                              post_mlp_layernorm=post2)
+            self.pre1, self.mixer, self.post1, self.pre2, self.ffn, self.post2 = pre1, mixer, post1, pre2, ffn, post2
+
+        def forward(self, resid, pending, batch, cache, store=True, next_norm=None):
+            act = batch.act_dtype
+            delta = None if isinstance(pending, ops.ScaledInput) else pending
+            a = self.mixer.forward(self.pre1.add_norm(resid, delta, act), batch, cache, store)
+            a = self.post1.add_norm(a.float(), None, act)
+            f = self.ffn.forward(self.pre2.add_norm(resid, a, act), batch)
+            return resid, self.post2.add_norm(f.float(), None, act)
+
+    @dataclasses.dataclass
+    class ArrangedConfig(ModelConfig):
+        vocab_size: int = 0
+
+    def build(cfg):
+        H, eps = ARR["hidden"], ARR["eps"]
+        rotary = RotaryEmbedding(ARR["head_dim"], ARR["theta"])
+        attn = lambda: PagedAttention(H, ARR["heads"], ARR["kv"], ARR["head_dim"], rotary, qk_norm_eps=eps)
+        norm, mlp = (lambda: RMSNorm(H, eps)), (lambda: GatedMLP(H, ARR["inter"]))
+        layers = [PreNormBlock(norm(), attn(), norm(), mlp()),
+                  ParallelBlock(norm(), attn(), mlp()),
+                  PreNormBlock(norm(), attn(), norm(), mlp()),
+                  SandwichBlock(norm(), attn(), norm(), norm(), mlp(), norm()),
+                  PreNormBlock(norm(), attn(), norm(), mlp())]
+        return DecoderModel(cfg, TokenEmbedding(cfg.vocab_size, H), rotary, layers, norm(), LMHead(cfg.vocab_size, H),
+                            max_positions=ARR["positions"])
+
+    return ArrangedConfig, build
+
+
+def plain_arranged(folder, tokens):
+    """Whole sequence, no cache, float32, from the plain functions and the formulas in the blocks' docstrings."""
+    w = {k: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    T, d, eps = len(tokens), ARR["head_dim"], ARR["eps"]
+    cos, sin = P.rope_tables(T, d, ARR["theta"])
+    positions = torch.arange(T)
+
+    def norm(x, name):
+        return P.rms_norm(x, w[name + ".weight"], eps)
+
+    def attn(n, p):
+        a = p + ".self_attn."
+        q = P.linear(n, w[a + "q_proj.weight"]).view(T, ARR["heads"], d)
+        k = P.linear(n, w[a + "k_proj.weight"]).view(T, ARR["kv"], d)
+        v = P.linear(n, w[a + "v_proj.weight"]).view(T, ARR["kv"], d)
+        q = P.rope_apply(P.rms_norm(q, w[a + "q_norm.weight"], eps), positions, cos, sin)
+        k = P.rope_apply(P.rms_norm(k, w[a + "k_norm.weight"], eps), positions, cos, sin)
+        return P.linear(P.attention(q, k, v).reshape(T, -1), w[a + "o_proj.weight"])
+
+    def mlp(n, p):
+        return P.linear(P.swiglu(P.linear(n, w[p + ".mlp.gate_proj.weight"]), P.linear(n, w[p + ".mlp.up_proj.weight"])),
+                        w[p + ".mlp.down_proj.weight"])
+
+    h = P.embedding(torch.tensor(tokens), w["model.embed_tokens.weight"])
+    for i, kind in enumerate(("pre", "parallel", "pre", "sandwich", "pre")):
+        p = "model.layers.%d" % i
+        if kind == "pre":
+            h = h + attn(norm(h, p + ".input_layernorm"), p)
+            h = h + mlp(norm(h, p + ".post_attention_layernorm"), p)
+        elif kind == "parallel":
+            n = norm(h, p + ".input_layernorm")
+            h = h + attn(n, p) + mlp(n, p)
+        else:
+            h = h + norm(attn(norm(h, p + ".input_layernorm"), p), p + ".post_mixer_layernorm")
+            h = h + norm(mlp(norm(h, p + ".pre_mlp_layernorm"), p), p + ".post_mlp_layernorm")
+    return P.linear(norm(h, "model.norm"), w["lm_head.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_other_arrangements_of_a_block(dtype, tmp_path):
+    """Blocks arranged otherwise, defined above, between the framework's own: every way of cutting the requests against
+    the plain pass; then through the entry point with recorded decode steps (the blocks say what their parts say about
+    recording), greedy tokens against the plain pass in float32."""
+    from spyinfer_amd.config import register_architecture, unregister_architecture
+    from spyinfer_amd.engine.llm_engine import LLMEngine
+    from spyinfer_amd.sampling import SamplingParams
+    from spyinfer_amd.weights import write_random_model
+    require_gpu()
+    ArrangedConfig, build = _toy_arranged()
+    register_architecture("ToyArrangedLM", ArrangedConfig, build)
+    try:
+        cfg = dict(architectures=["ToyArrangedLM"], vocab_size=ARR["vocab"])
+        folder = write_random_model(str(tmp_path / "toy"), cfg, 91, torch.bfloat16, **INIT)
+        reqs = rc.random_requests(ARR["vocab"], [70, 9, 41, 120, 33], seed=12)
+        ref = {rid: plain_arranged(folder, t) for rid, t in reqs.items()}
+        for mode in ("whole", "bulk_tail", "portions", "mixed"):
+            steps = getattr(rc, mode)(reqs)
+            out = str(tmp_path / mode)
+            rc.run_replay_inprocess(folder, dtype, out, steps, rc.max_live_tokens(steps))
+            rc.compare(rc.collect(out, steps, ARR["vocab"]), ref, what="arranged/" + mode, **TOL[dtype])
+        eng = LLMEngine(folder, dtype=dtype, max_model_len=200, num_kvcache_blocks=40, max_num_seqs=4)
+        prompts = [t[:n] for t, n in zip(reqs.values(), (30, 9, 41, 5))]
+        got = eng.generate(prompts, SamplingParams(max_new_tokens=12, ignore_eos=True))
+        assert eng.runner.graph_replays > 0, "decode steps of these blocks are recorded"
+        if dtype == "float32":
+            for p, g in zip(prompts, got):
+                toks = list(p)
+                for t in g:
+                    assert t == int(torch.argmax(plain_arranged(folder, toks)[-1]))
+                    toks.append(t)
+    finally:
+        unregister_architecture("ToyArrangedLM")
