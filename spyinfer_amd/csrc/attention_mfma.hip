@@ -675,7 +675,7 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
     const dim3 mgrid(num_tiles, n_kv);
     // The parts merged by each (tile, kv head)'s last block instead of a second kernel: with counters (zeroed once by the
     // caller, one per tile and head, left at zero by every call; calls that overlap on one device race on them), up to
-    // 16 parts and head sizes up to 128.
+    // 16 parts (the grid's; the host's records may name up to 32 of an entry) and head sizes up to 128.
     unsigned* const cnt = (pieces || (counters && splits > 1 && splits <= 16 && d <= 128 && (long long)num_tiles * n_kv <= n_counters)) ? counters : nullptr;
 #define ATT_LAUNCH(DM, FZ, FL)                                                                                                \
     attention_mfma_kernel<DM, FZ, FL><<<grid, AW * 64, (DM <= 128 ? AW : AW - 1) * ((DM / 16) * 4 + 2) * 64 * sizeof(float), st>>>(  \
