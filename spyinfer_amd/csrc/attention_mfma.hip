@@ -121,10 +121,13 @@ __device__ __forceinline__ void norm_rotate(bf16x8_t (&x)[KK], bool normed, cons
     }
 }
 
-// FULL: head_dim == DMAX.  The loads of keys and values then have no conditions (a page that does not exist is read as
+// FULL (not 0): head_dim == DMAX.  The loads of keys and values then have no conditions (a page that does not exist is read as
 // page 0 and what was read is masked: scores by position, values by the count of keys that exist and, under a window, by
 // the page's absence), so the compiler knows how many loads are in flight and a wait is for the oldest only.
-template <int DMAX, bool FUSED, bool FULL>
+// FULL_STREAMED / FULL_KEPT: whether the values are read with the hint that they will not be read again (pages of up to 32
+// keys) or without it (larger pages).
+constexpr int FULL_STREAMED = 1, FULL_KEPT = 2;
+template <int DMAX, bool FUSED, int FULL>
 __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void attention_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, bf16_t* kc, bf16_t* vc,
     int P, int num_pages, const int* __restrict__ cu_q, const int* __restrict__ pos0, const int* __restrict__ kv_len,
@@ -309,11 +312,23 @@ __global__ __launch_bounds__(AW * 64, (FUSED && DMAX <= 128) ? 2 : 1) void atten
         const bool v_ok = vpage >= 0 && vpage < num_pages;
         const bf16_t* vp = vc + (((size_t)(v_ok ? vpage : 0) * n_kv + hk) * d) * P + in_page(key_v);
         bf16x8_t vt[DT];
+        if constexpr (FULL == FULL_STREAMED) {
+            // (a block's 32 keys of a dim are whole lines of pages of up to 32 keys: read once, not to be kept)
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const int dd = dt * 16 + r16;
-            if (FULL) vt[dt] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P));
-            else vt[dt] = (v_ok && dd < d) ? *reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P) : zero8();
+            for (int dt = 0; dt < DT; ++dt) vt[dt] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(vp + (size_t)(dt * 16 + r16) * P));
+        } else if constexpr (FULL == FULL_KEPT) {
+            // (of larger pages they are half a line or less, and the next block, which another wave of this block takes
+            // at about the same time, reads the rest of it: kept, or memory would bring every line twice.  64 requests
+            // of 8337 keys in pages of 64: 397 against 460 us; pages of 16: 357.  A template's value and not a branch:
+            // the compiler makes one load of the two arms of a branch, without the hint)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vt[dt] = *reinterpret_cast<const bf16x8_t*>(vp + (size_t)(dt * 16 + r16) * P);
+        } else {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int dd = dt * 16 + r16;
+                vt[dt] = (v_ok && dd < d) ? *reinterpret_cast<const bf16x8_t*>(vp + (size_t)dd * P) : zero8();
+            }
         }
         if (FULL && window > 0 && !v_ok) {
             // The window's first block of 32 keys may begin in a page that the window has passed and the request has
@@ -682,7 +697,9 @@ extern "C" int spy_attention_mfma(void* out, const void* q, void* kc, void* vc, 
         (bf16_t*)out, (const bf16_t*)q, (bf16_t*)kc, (bf16_t*)vc, P, num_pages, cu_q, pos0, kv_len, block_table, max_blocks,  \
         tile_entry, tile_row0, n_q, n_kv, d, scale, window, splits, ws, fz, out_tiles, cnt, log2p, pieces)
 #define ATT_CASE(DM)                                                                                                          \
-    if (qkv) ATT_LAUNCH(DM, true, true); else if (d == DM) ATT_LAUNCH(DM, false, true); else ATT_LAUNCH(DM, false, false);       \
+    if (qkv && P <= 32) ATT_LAUNCH(DM, true, FULL_STREAMED); else if (qkv) ATT_LAUNCH(DM, true, FULL_KEPT);                      \
+    else if (d == DM && P <= 32) ATT_LAUNCH(DM, false, FULL_STREAMED); else if (d == DM) ATT_LAUNCH(DM, false, FULL_KEPT);       \
+    else ATT_LAUNCH(DM, false, 0);                                                                                            \
     if (cnt) {}                                                                                                               \
     else if (splits > 1 && qkv)                                                                                               \
         attention_merge_kernel<DM, true><<<mgrid, 256, 0, st>>>((bf16_t*)out, ws, cu_q, tile_entry, tile_row0, n_q, n_kv, d, splits, 1, out_tiles); \
