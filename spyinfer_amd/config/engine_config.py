@@ -28,7 +28,8 @@ class EngineConfig:
     enforce_eager: bool = False
     #: tokens in a cache page (config.hpp:26; the reference's default is 4).  Values lie transposed inside a page, and the
     #: decode attention reads 32 keys at a time: whole memory lines with pages of 8 to 32 tokens, half lines with larger
-    #: ones (64 requests of 8337 keys: 397 us a layer with pages of 64 or 128 against 355 with pages of 16)
+    #: ones (64 requests of 8337 keys: 397 us a layer with pages of 64 or 128 against 355 with pages of 16).  A size that
+    #: is no multiple of 8 (the reference's 4) is taken too, by the plain attention kernel, which is built for checking
     kvcache_block_size: int = 16
     #: pages in the pool of every cache group; None = from free memory (config.hpp:27)
     num_kvcache_blocks: Optional[int] = None
